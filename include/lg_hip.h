@@ -1,0 +1,142 @@
+/* lg_hip.h — C ABI of liblg_hip.so, the gfx950 backend of little-gemma's MTP verify step.
+ *
+ * Plain C: opaque handles, pointers, sizes, int status codes (0 = ok, negative = error; the
+ * message is kept per thread and read with lg_hip_last_error()).  No HIP, torch or GGUF types
+ * cross this boundary, so the reference's C host code (or anything with an FFI) can bind it.
+ * model-hip.c (little-gemma_amd/host/) implements the reference's include/model.h on top of
+ * these calls; each entry point below cites the reference interface it stands behind.
+ *
+ * Threading: one caller thread per model, like the reference backends
+ * (src/cuda/model-cuda.cuh:724-726); calls on one model are not re-entrant.
+ * Device errors are returned, never exit(): the caller decides (model-hip.c prints and exits
+ * like CUDA_CHECK, src/cuda/model-cuda.cuh:34-36).
+ */
+#ifndef LG_HIP_H
+#define LG_HIP_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LG_HIP_MAX_ROWS 8          /* widest verify block (LG_MTP_N) the kernels are built for */
+
+typedef struct lg_hip_model lg_hip_model;
+typedef struct lg_hip_kv    lg_hip_kv;
+
+/* Hyper-parameters and per-layer geometry: the fields of struct config / struct model the
+ * forward reads (include/model.h:10-48).  Arrays have n_layer entries and are copied. */
+struct lg_hip_config {
+    int32_t n_layer, n_embd, n_head, n_vocab;
+    int32_t sliding_window, n_embd_per_layer, n_kv_start;
+    float   rms_eps, rope_freq_base, rope_freq_base_swa, logit_softcap;
+    const int32_t *is_local, *ffn_len, *head_dim, *n_head_kv;
+};
+
+const char *lg_hip_last_error(void);
+/* Number of usable devices (0 when there is none); never fails. */
+int lg_hip_device_count(void);
+
+/* ---- model: weights resident on the device ------------------------------------------------
+ * Replaces ensure_weights/ensure_scratch (src/cuda/model-cuda.cuh:738-799,937-970) with an
+ * explicit sequence: create, hand over every tensor once, commit. */
+int  lg_hip_model_create(const struct lg_hip_config *cfg, int device, lg_hip_model **out);
+/* One GGUF tensor by its GGUF name (e.g. "blk.3.attn_q.weight"): ggml type id, dims[0] = row
+ * length, dims[1] = rows, data = host bytes in GGUF layout.  Matrices must be q4_0 with a row
+ * length that is a multiple of 256 and a row count that is a multiple of 8 (the reference's
+ * repack has the same k%256 rule, src/cuda/model-cuda-i8.cu:613-620); vectors must be f32.
+ * Unknown names are ignored (returns 1) so a caller can simply walk the file. */
+int  lg_hip_model_tensor(lg_hip_model *m, const char *name, uint32_t ggml_type, uint32_t n_dims,
+                         const uint64_t *dims, const void *data);
+/* Checks that every tensor the forward needs arrived, lays weights out for the kernels and
+ * allocates scratch for blocks of up to max_rows (1..LG_HIP_MAX_ROWS) verify rows. */
+int  lg_hip_model_commit(lg_hip_model *m, int max_rows);
+void lg_hip_model_destroy(lg_hip_model *m);
+
+/* ---- KV cache: f16 rings on the device (kvcache_init/free, include/model.h:79-80;
+ * src/cuda/model-cuda.cuh:998-1051).  Global layers hold max_seq rows, sliding layers
+ * lg_hip_ring_rows(window, max_seq); row of position p = p % rows. */
+int  lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out);
+void lg_hip_kv_destroy(lg_hip_kv *kv);
+int  lg_hip_ring_rows(int window, int max_seq);
+/* rows/width of an owning layer's K (== V) storage; *rows = 0 for a layer that shares. */
+int  lg_hip_kv_layout(const lg_hip_kv *kv, int layer, int *rows, int *width);
+/* Copy whole cache rows (binary16 bit patterns) from/to host memory: which = 0 K, 1 V. */
+int  lg_hip_kv_write(lg_hip_kv *kv, int layer, int which, int row0, int n_rows, const uint16_t *src);
+int  lg_hip_kv_read(const lg_hip_kv *kv, int layer, int which, int row0, int n_rows, uint16_t *dst);
+/* kvcache_save_prefix / kvcache_restore_prefix (include/model.h:82-92): first min(n, rows)
+ * rows of every owning layer, device to device. */
+int  lg_hip_kv_save_prefix(lg_hip_kv *kv, int n);
+int  lg_hip_kv_restore_prefix(lg_hip_kv *kv, int n);
+
+/* ---- the verify step: model_forward_spec (include/model.h:179-186,
+ * src/cuda/mtp-kernel.cuh:82-120).  toks[0] is the chosen token at position pos, toks[1..]
+ * the drafts; out[j] = greedy successor of toks[j] (first maximum of the soft-capped logits);
+ * *adv = 1 + number of leading drafts that held.  K/V rows pos..pos+n_rows-1 are written.
+ * Embedding lookup, the whole decoder, lm_head, argmax and the accept rule run on the device
+ * inside one captured graph; the host copies n_rows tokens in and n_rows+1 ints out. */
+int  lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n_rows, int pos,
+                         int32_t *out, int32_t *adv);
+/* model_prefill (include/model.h:121): positions pos0..pos0+n-1, cache writes only, no head.
+ * Runs as blocks of up to max_rows rows through the same kernels as the verify step. */
+int  lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int pos0);
+/* Post-output-norm hidden state of the last valid row of the latest verify step (n_embd
+ * floats): what the reference keeps in g_hidden / model.last_hidden for the draft head
+ * (src/cuda/mtp-kernel.cuh:117-118). */
+int  lg_hip_get_hidden(lg_hip_model *m, float *dst);
+/* Re-point that hidden state at row `row` of the latest step: for callers that accept rows by
+ * their own rule (the sampling hook, src/cuda/mtp-kernel.cuh:103-118). */
+int  lg_hip_set_hidden_row(lg_hip_model *m, int row);
+/* Soft-capped logits of row `row` of the latest step (n_vocab floats).  Only stored while the
+ * "store_logits" option is on (model_forward, include/model.h:98, needs them; the verify does not). */
+int  lg_hip_get_logits(lg_hip_model *m, int row, float *dst);
+/* Options: "store_logits" (0/1, default 0), "use_graph" (0/1, default 1). */
+int  lg_hip_set_option(lg_hip_model *m, const char *name, int value);
+
+/* ---- device-resident stepping: the same step with no host round trip between steps.
+ * A schedule is n_steps blocks of n_rows tokens built by the caller (drafts come from a draft
+ * head or, in the benchmark, are prepared in advance); each step verifies block `step`, writes
+ * its out[] and adv, then advances the device-resident position by adv and the step counter
+ * by one.  No reference counterpart: the reference synchronises every step
+ * (src/cuda/mtp-kernel.cuh:95,112). */
+int  lg_hip_schedule_load(lg_hip_model *m, const int32_t *toks, int n_steps, int n_rows, int pos0);
+int  lg_hip_schedule_run(lg_hip_model *m, lg_hip_kv *kv, int n_steps);   /* enqueues, does not wait */
+int  lg_hip_schedule_wait(lg_hip_model *m, int32_t *out, int32_t *adv, int32_t *final_pos);
+/* Times n_steps already-loaded steps with device events on the library's stream; *ms = total. */
+int  lg_hip_schedule_time(lg_hip_model *m, lg_hip_kv *kv, int n_steps, float *ms);
+
+/* ---- measurement: run one step un-captured with an event pair around every kernel and sum
+ * the durations per kernel class.  names/ms/launches/bytes are caller arrays of `cap` entries;
+ * returns the number of classes filled.  bytes[i] = weight + KV bytes the class must read per
+ * step (algorithmic, not measured). */
+int  lg_hip_profile_step(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n_rows, int pos,
+                         int repeats, const char **names, float *ms, int32_t *launches,
+                         double *bytes, int cap);
+
+/* ---- isolated kernels, host pointers in and out (parity tests of the parts) ----------------
+ * q4_0 x q8_0 matmul (matmul_q_spec, src/cuda/model-cuda-i8.cu:1592-1602): w = m rows of k/32
+ * 18-byte q4_0 blocks; x = rows x k floats, quantized on the device per 32 (d_quant_group,
+ * src/cuda/model-cuda.cuh:84-92).  Outputs (each may be NULL): out[rows][m] f32;
+ * dots[rows][m][k/32] int32 block dots; xq[rows][k] int8; xd[rows][k/32] f32 scales;
+ * xsum[rows][k/32] int32 sums.  *kernel_ms (may be NULL) = mean device time of `repeats` launches
+ * of the matmul kernel alone. */
+int  lg_hip_matmul_q4q8(const void *w, int k, int m, const float *x, int rows, float *out,
+                        int32_t *dots, int8_t *xq, float *xd, int32_t *xsum, int repeats, float *kernel_ms);
+/* Decode attention over an f16 ring (split_attn_kernel + combine_attn_kernel,
+ * src/cuda/model-cuda.cuh:527-608) for a block of `rows` queries at pos..pos+rows-1:
+ * q = rows x n_head x hd floats, already normed and rotated; kc/vc = seq rows of n_head_kv*hd
+ * binary16; window = 0 for a global layer.  out = rows x n_head x hd floats. */
+int  lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, int rows, int n_head,
+                      int n_head_kv, int hd, int seq, int window, int pos, float *out,
+                      int repeats, float *kernel_ms);
+/* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
+ * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
+size_t lg_hip_repacked_bytes(int k, int m);
+int    lg_hip_repack_q4_0(const void *src, int k, int m, void *dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LG_HIP_H */

@@ -1,0 +1,143 @@
+// lg_device.h — device-side building blocks of the verify step (gfx950, wave64).
+//
+// Numeric contract shared with the CPU oracle: every float reduction below has ONE defined
+// order, chosen to be natural for a 64-lane wavefront, and every elementary function comes
+// from include/lg_math.h.  Integer work (q8 quantization, q4_0 x q8 block dots) is exact.
+//   * row sum of squares: 64 lane partials, element i belongs to lane (i/4)%64, fma in
+//     ascending i, then an adjacent-pair binary tree over the lanes;
+//   * q4_0 x q8 matmul: 8 contiguous K segments per output, one lane each, serial fma over
+//     the segment's blocks, adjacent-pair tree over the 8 lanes;
+//   * attention: 32-key tiles aligned to absolute positions (see lg_kernels.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/lg_math.h"
+
+#define LG_WG        256      // threads per workgroup: 4 wavefronts
+#define LG_TILE      1152     // bytes of one weight tile: 64 lanes x 16 B of nibbles + 64 x 2 B of scales
+#define LG_TK        32       // keys per attention tile
+#define LG_MAXV      16       // float4 per lane of a residual row: n_embd <= 4096
+#define LG_HIP_MAX_ROWS_DEV 8   // widest draft block (same value as LG_HIP_MAX_ROWS in lg_hip.h)
+
+// Weight tile order (built on the host by lg_hip_repack_q4_0): an m x k q4_0 matrix is cut into
+// groups of 8 rows; row r of a group is cut into 8 segments of nit = k/256 blocks; tile (group,
+// it) holds, for lane = r*8 + c, the 16 nibble bytes and the f16 scale of block c*nit + it of
+// row r.  A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
+
+__device__ __forceinline__ float lg_wave_sum64(float v) {
+    v = v + __shfl_xor(v, 1);
+    v = v + __shfl_xor(v, 2);
+    v = v + __shfl_xor(v, 4);
+    v = v + __shfl_xor(v, 8);
+    v = v + __shfl_xor(v, 16);
+    v = v + __shfl_xor(v, 32);
+    return v;
+}
+__device__ __forceinline__ float lg_sum8(float v) {
+    v = v + __shfl_xor(v, 1);
+    v = v + __shfl_xor(v, 2);
+    v = v + __shfl_xor(v, 4);
+    return v;
+}
+__device__ __forceinline__ float lg_sum32(float v) {
+    v = v + __shfl_xor(v, 1);
+    v = v + __shfl_xor(v, 2);
+    v = v + __shfl_xor(v, 4);
+    v = v + __shfl_xor(v, 8);
+    v = v + __shfl_xor(v, 16);
+    return v;
+}
+__device__ __forceinline__ float lg_max_n(float v, int n) {       // n = 8 or 32 lanes
+    for (int o = 1; o < n; o <<= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ int lg_isum_n(int v, int n) {
+    for (int o = 1; o < n; o <<= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+__device__ __forceinline__ float lg_sumsq4(float4 v, float acc) {
+    acc = lg_fmaf(v.x, v.x, acc);
+    acc = lg_fmaf(v.y, v.y, acc);
+    acc = lg_fmaf(v.z, v.z, acc);
+    acc = lg_fmaf(v.w, v.w, acc);
+    return acc;
+}
+
+// q8 quantization of 32 consecutive values held as one float4 in each of 8 adjacent lanes:
+// amax, d = amax/127, id = 1/d (0 when d == 0), q = rint_even(x*id), sum of q.
+// Returns the 4 packed int8; *d_out / *sum_out are the same in all 8 lanes.
+__device__ __forceinline__ uint32_t lg_quant4_8lanes(float4 h, float *d_out, int *sum_out) {
+    float amax = fmaxf(fmaxf(fabsf(h.x), fabsf(h.y)), fmaxf(fabsf(h.z), fabsf(h.w)));
+    amax = lg_max_n(amax, 8);
+    const float d = amax / 127.0f;
+    const float id = d > 0.0f ? 1.0f / d : 0.0f;
+    const int q0 = (int)lg_rintf(h.x * id), q1 = (int)lg_rintf(h.y * id);
+    const int q2 = (int)lg_rintf(h.z * id), q3 = (int)lg_rintf(h.w * id);
+    *d_out = d;
+    *sum_out = lg_isum_n(q0 + q1 + q2 + q3, 8);
+    return (uint32_t)(q0 & 255) | ((uint32_t)(q1 & 255) << 8) | ((uint32_t)(q2 & 255) << 16) | ((uint32_t)(q3 & 255) << 24);
+}
+
+// Same for 32 values held one per lane in 32 adjacent lanes (half a wavefront).
+__device__ __forceinline__ int lg_quant1_32lanes(float h, float *d_out, int *sum_out) {
+    const float amax = lg_max_n(fabsf(h), 32);
+    const float d = amax / 127.0f;
+    const float id = d > 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)lg_rintf(h * id);
+    *d_out = d;
+    *sum_out = lg_isum_n(q, 32);
+    return q;
+}
+
+__device__ __forceinline__ float lg_h2f(uint16_t h) {
+    return __half2float(__ushort_as_half(h));
+}
+__device__ __forceinline__ uint16_t lg_f2h(float f) {
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// Four consecutive elements (e0 % 4 == 0) of row `row` of a tiled q4_0 matrix, dequantized.
+__device__ __forceinline__ float4 lg_tiled_deq4(const uint8_t *w, int nit, int row, int e0) {
+    const int b = e0 >> 5, o = e0 & 31;
+    const int c = b / nit, it = b - c * nit;
+    const uint8_t *tile = w + ((size_t)(row >> 3) * nit + it) * LG_TILE;
+    const int slot = (row & 7) * 8 + c;
+    const uint32_t qs = *(const uint32_t *)(tile + slot * 16 + (o & 15));
+    const float d = lg_h2f(*(const uint16_t *)(tile + 1024 + slot * 2));
+    const uint32_t nib = (o & 16) ? (qs >> 4) : qs;
+    float4 r;
+    r.x = d * (float)((int)(nib & 15) - 8);
+    r.y = d * (float)((int)((nib >> 8) & 15) - 8);
+    r.z = d * (float)((int)((nib >> 16) & 15) - 8);
+    r.w = d * (float)((int)((nib >> 24) & 15) - 8);
+    return r;
+}
+
+// One element of a q4_0 row in plain GGUF order (18-byte blocks).
+__device__ __forceinline__ float lg_q4_0_elem(const uint8_t *row, int e) {
+    const uint8_t *blk = row + (size_t)(e >> 5) * 18;
+    const float d = lg_h2f((uint16_t)(blk[0] | (blk[1] << 8)));
+    const int o = e & 31;
+    const int nib = (o & 16) ? (blk[2 + (o & 15)] >> 4) : (blk[2 + o] & 15);
+    return d * (float)(nib - 8);
+}
+
+// Inner product of one weight tile lane (16 nibble bytes = one q4_0 block) with the 32 int8 of
+// an activation block: sum(c*q) - 8*sum(q) == sum((c-8)*q), exact in int32.
+__device__ __forceinline__ int lg_block_dot(uint4 wq, const int8_t *act32, int act_sum) {
+    const int4 a0 = *(const int4 *)act32, a1 = *(const int4 *)(act32 + 16);
+    int dot = 0;
+    dot = __builtin_amdgcn_sdot4((int)(wq.x & 0x0F0F0F0Fu), a0.x, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)(wq.y & 0x0F0F0F0Fu), a0.y, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)(wq.z & 0x0F0F0F0Fu), a0.z, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)(wq.w & 0x0F0F0F0Fu), a0.w, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)((wq.x >> 4) & 0x0F0F0F0Fu), a1.x, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)((wq.y >> 4) & 0x0F0F0F0Fu), a1.y, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)((wq.z >> 4) & 0x0F0F0F0Fu), a1.z, dot, false);
+    dot = __builtin_amdgcn_sdot4((int)((wq.w >> 4) & 0x0F0F0F0Fu), a1.w, dot, false);
+    return dot - 8 * act_sum;
+}

@@ -1,0 +1,1016 @@
+// lg_hip.hip — C ABI of the gfx950 verify-step backend (declared in include/lg_hip.h).
+//
+// Host side: weight layout, scratch, the launch sequence of one step, graph capture, the
+// device-resident step schedule and the measurement helpers.  Device side: lg_kernels.h.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <map>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/lg_hip.h"
+#include "lg_kernels.h"
+
+static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
+
+// ---- errors -----------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+#define HIP_TRY(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) \
+    return fail(-100 - (int)e_, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); } while (0)
+
+extern "C" const char *lg_hip_last_error(void) { return g_err; }
+extern "C" int lg_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return n;
+}
+extern "C" int lg_hip_ring_rows(int window, int max_seq) {
+    int r = (window + 32 + 31) / 32 * 32;          // window + spare for a block of draft rows, tile multiple
+    return r < max_seq ? r : max_seq;
+}
+
+// ---- weight layout ----------------------------------------------------------------------------
+extern "C" size_t lg_hip_repacked_bytes(int k, int m) {
+    if (k <= 0 || m <= 0 || k % 256 || m % 8) return 0;
+    return (size_t)(m / 8) * (size_t)(k / 256) * LG_TILE;
+}
+
+// rows[i] points at virtual row i (k/32 blocks of 18 bytes each)
+static void repack_rows(const uint8_t *const *rows, int k, int m, uint8_t *dst) {
+    const int nit = k / 256, groups = m / 8;
+    auto work = [&](int g0, int g1) {
+        for (int g = g0; g < g1; ++g)
+            for (int it = 0; it < nit; ++it) {
+                uint8_t *tile = dst + ((size_t)g * nit + it) * LG_TILE;
+                for (int r = 0; r < 8; ++r)
+                    for (int c = 0; c < 8; ++c) {
+                        const uint8_t *blk = rows[g * 8 + r] + (size_t)(c * nit + it) * 18;
+                        memcpy(tile + (r * 8 + c) * 16, blk + 2, 16);
+                        memcpy(tile + 1024 + (r * 8 + c) * 2, blk, 2);
+                    }
+            }
+    };
+    unsigned hw = std::thread::hardware_concurrency();
+    int nt = (int)(hw ? (hw > 16 ? 16 : hw) : 4);
+    if ((size_t)groups * nit < 4096 || nt < 2) { work(0, groups); return; }
+    std::vector<std::thread> pool;
+    for (int t = 0; t < nt; ++t) pool.emplace_back(work, (int)((long long)groups * t / nt), (int)((long long)groups * (t + 1) / nt));
+    for (auto &th : pool) th.join();
+}
+
+extern "C" int lg_hip_repack_q4_0(const void *src, int k, int m, void *dst) {
+    if (!lg_hip_repacked_bytes(k, m)) return fail(-2, "repack: k=%d must be a multiple of 256 and m=%d of 8", k, m);
+    std::vector<const uint8_t *> rows((size_t)m);
+    for (int i = 0; i < m; ++i) rows[i] = (const uint8_t *)src + (size_t)i * (k / 32) * 18;
+    repack_rows(rows.data(), k, m, (uint8_t *)dst);
+    return 0;
+}
+
+// ---- objects ----------------------------------------------------------------------------------
+struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; };
+
+struct Layer {
+    uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
+    float *attn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *post_attn = nullptr, *ffn_norm = nullptr,
+          *post_ffw = nullptr, *post_norm = nullptr, *out_scale = nullptr;
+    int is_local = 0, hd = 0, nkv = 0, nff = 0, qd = 0, kd = 0, qkv_m = 0, k_off = 0, v_off = 0, owns = 0, src = 0;
+    const float *rope_tab = nullptr, *rope_ff = nullptr;
+};
+
+enum KClass { KC_PMP, KC_QKV, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
+              KC_FINALNORM, KC_HEAD, KC_ACCEPT, KC_COUNT };
+static const char *k_class_names[KC_COUNT] = { "ple_model_proj", "qkv", "attn_tiles", "attn_merge", "attn_output",
+    "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "final_norm", "lm_head", "accept" };
+
+struct Profile {
+    bool on = false;
+    std::vector<hipEvent_t> ev;        // pairs
+    std::vector<int> cls;
+};
+
+struct lg_hip_model {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    // config
+    int n_layer = 0, E = 0, H = 0, n_vocab = 0, window = 0, ple = 0, n_kv_start = 0, max_rows = 0;
+    float eps = 0, base = 0, base_swa = 0, softcap = 0;
+    std::vector<int> is_local, ffn_len, head_dim, n_head_kv;
+    std::map<std::string, HostTensor> host;
+    bool committed = false;
+    // weights
+    std::vector<Layer> L;
+    uint8_t *emb = nullptr, *pmp = nullptr, *pte = nullptr;
+    float *output_norm = nullptr, *rope_freqs = nullptr, *proj_norm = nullptr;
+    std::vector<void *> allocs;
+    std::map<std::pair<int, int>, float *> rope_tabs;      // (is_local, hd) -> table
+    size_t weight_bytes = 0;
+    // scratch
+    float *x[2] = { nullptr, nullptr }, *qkv = nullptr, *dout = nullptr, *pmp_raw = nullptr, *hidden_rows = nullptr,
+          *g_hidden = nullptr, *logits = nullptr, *pval = nullptr;
+    int8_t *aq = nullptr, *gq = nullptr, *pq = nullptr, *hq = nullptr;
+    float2 *ads = nullptr, *gds = nullptr, *pds = nullptr, *hds = nullptr;
+    int *pidx = nullptr;
+    StepCtl *ctl = nullptr;
+    int32_t *sched = nullptr, *out = nullptr, *adv = nullptr;
+    int sched_cap = 0, sched_steps = 0, sched_rows = 0;
+    int32_t *pin = nullptr;            // pinned host staging
+    int last_rows = 0, last_adv = 0;
+    int store_logits = 0, use_graph = 1;
+    std::map<std::string, hipGraphExec_t> graphs;
+    Profile prof;
+};
+
+struct lg_hip_kv {
+    lg_hip_model *m = nullptr;
+    int max_seq = 0, tiles_max = 0;
+    std::vector<int> seq, kv_dim;
+    std::vector<uint16_t *> k, v, px_k, px_v;
+    float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
+    unsigned id = 0;
+};
+static unsigned g_kv_ids = 0;
+
+template <typename T>
+static int dev_alloc(lg_hip_model *m, T **p, size_t n) {
+    HIP_TRY(hipMalloc((void **)p, n * sizeof(T) ? n * sizeof(T) : 16));
+    m->allocs.push_back((void *)*p);
+    return 0;
+}
+
+extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg_hip_model **out) {
+    if (!c || !out) return fail(-1, "model_create: null argument");
+    if (c->n_layer <= 0 || c->n_embd <= 0 || c->n_embd % 256 || c->n_embd > 256 * LG_MAXV || c->n_head <= 0 ||
+        c->n_vocab <= 0 || c->n_vocab % 32)
+        return fail(-2, "model_create: unsupported shape (n_embd %d must be a multiple of 256 and <= %d, n_vocab %d a multiple of 32)",
+                    c->n_embd, 256 * LG_MAXV, c->n_vocab);
+    if (c->n_embd_per_layer % 32) return fail(-2, "model_create: per-layer embedding width %d must be a multiple of 256 or 0", c->n_embd_per_layer);
+    if (lg_hip_device_count() <= device) return fail(-3, "model_create: no HIP device %d (the verify step has no CPU path)", device);
+    HIP_TRY(hipSetDevice(device));
+    lg_hip_model *m = new lg_hip_model();
+    m->device = device;
+    m->n_layer = c->n_layer; m->E = c->n_embd; m->H = c->n_head; m->n_vocab = c->n_vocab;
+    m->window = c->sliding_window; m->ple = c->n_embd_per_layer; m->n_kv_start = c->n_kv_start;
+    m->eps = c->rms_eps; m->base = c->rope_freq_base; m->base_swa = c->rope_freq_base_swa; m->softcap = c->logit_softcap;
+    m->is_local.assign(c->is_local, c->is_local + c->n_layer);
+    m->ffn_len.assign(c->ffn_len, c->ffn_len + c->n_layer);
+    m->head_dim.assign(c->head_dim, c->head_dim + c->n_layer);
+    m->n_head_kv.assign(c->n_head_kv, c->n_head_kv + c->n_layer);
+    hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
+    *out = m;
+    return 0;
+}
+
+extern "C" int lg_hip_model_tensor(lg_hip_model *m, const char *name, uint32_t type, uint32_t n_dims,
+                                   const uint64_t *dims, const void *data) {
+    if (!m || !name || !dims || !data || n_dims < 1 || n_dims > 4) return fail(-1, "model_tensor: bad argument");
+    if (m->committed) return fail(-4, "model_tensor: model already committed");
+    static const char *top[] = { "token_embd.weight", "output_norm.weight", "rope_freqs.weight",
+                                 "per_layer_token_embd.weight", "per_layer_model_proj.weight", "per_layer_proj_norm.weight" };
+    bool known = !strncmp(name, "blk.", 4);
+    for (const char *t : top) known = known || !strcmp(name, t);
+    if (!known) return 1;
+    HostTensor h;
+    h.type = type; h.n_dims = n_dims; h.data = data;
+    for (int i = 0; i < 4; ++i) h.dims[i] = i < (int)n_dims ? dims[i] : 1;
+    m->host[name] = h;
+    return 0;
+}
+
+static const HostTensor *find(lg_hip_model *m, const std::string &name) {
+    auto it = m->host.find(name);
+    return it == m->host.end() ? nullptr : &it->second;
+}
+static std::string lname(int L, const char *leaf) { return "blk." + std::to_string(L) + "." + leaf; }
+
+static int upload_vec(lg_hip_model *m, const std::string &name, size_t n, bool required, float **out) {
+    const HostTensor *t = find(m, name);
+    *out = nullptr;
+    if (!t) return required ? fail(-5, "model_commit: tensor %s is missing", name.c_str()) : 0;
+    size_t have = 1;
+    for (uint32_t i = 0; i < t->n_dims; ++i) have *= t->dims[i];
+    if (t->type != 0 || have != n) return fail(-6, "model_commit: %s must be f32 with %zu elements", name.c_str(), n);
+    if (dev_alloc(m, out, n)) return -7;
+    HIP_TRY(hipMemcpy(*out, t->data, n * 4, hipMemcpyHostToDevice));
+    m->weight_bytes += n * 4;
+    return 0;
+}
+
+struct RowSrc { const HostTensor *t; };
+static int check_mat(const HostTensor *t, const std::string &name, uint64_t k, uint64_t mrows) {
+    if (!t) return fail(-5, "model_commit: tensor %s is missing", name.c_str());
+    if (t->type != 2) return fail(-6, "model_commit: %s has ggml type %u; the verify path takes q4_0 matrices only", name.c_str(), t->type);
+    if (t->dims[0] != k || t->dims[1] != mrows) return fail(-6, "model_commit: %s is %llu x %llu, expected %llu x %llu", name.c_str(),
+        (unsigned long long)t->dims[0], (unsigned long long)t->dims[1], (unsigned long long)k, (unsigned long long)mrows);
+    if (k % 256 || mrows % 8) return fail(-6, "model_commit: %s needs row length %% 256 == 0 and rows %% 8 == 0", name.c_str());
+    return 0;
+}
+// upload a tiled matrix whose virtual rows are given by `rows`
+static int upload_tiled(lg_hip_model *m, const std::vector<const uint8_t *> &rows, int k, uint8_t **out,
+                        std::vector<uint8_t> &stage) {
+    const size_t bytes = lg_hip_repacked_bytes(k, (int)rows.size());
+    if (!bytes) return fail(-6, "model_commit: cannot tile a %zu x %d matrix", rows.size(), k);
+    stage.resize(bytes);
+    repack_rows(rows.data(), k, (int)rows.size(), stage.data());
+    if (dev_alloc(m, out, bytes)) return -7;
+    HIP_TRY(hipMemcpy(*out, stage.data(), bytes, hipMemcpyHostToDevice));
+    m->weight_bytes += bytes;
+    return 0;
+}
+static void push_rows(std::vector<const uint8_t *> &rows, const HostTensor *t, uint64_t r0, uint64_t n) {
+    const size_t rb = (size_t)(t->dims[0] / 32) * 18;
+    for (uint64_t r = r0; r < r0 + n; ++r) rows.push_back((const uint8_t *)t->data + r * rb);
+}
+
+static const float *rope_table(lg_hip_model *m, int is_local, int hd, int *rc) {
+    auto key = std::make_pair(is_local, hd);
+    auto it = m->rope_tabs.find(key);
+    if (it != m->rope_tabs.end()) return it->second;
+    std::vector<float> tab((size_t)hd / 2);
+    const float base = is_local ? m->base_swa : m->base;
+    for (int i = 0; i < hd / 2; ++i) tab[i] = powf(base, -2.0f * (float)i / (float)hd);   // src/cpu/model-cpu.c:90
+    float *d = nullptr;
+    if (hipMalloc((void **)&d, tab.size() * 4) != hipSuccess || hipMemcpy(d, tab.data(), tab.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
+        *rc = fail(-7, "model_commit: rope table upload failed");
+        return nullptr;
+    }
+    m->allocs.push_back(d);
+    m->rope_tabs[key] = d;
+    return d;
+}
+
+extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
+    if (!m) return fail(-1, "model_commit: null model");
+    if (m->committed) return fail(-4, "model_commit: already committed");
+    if (max_rows < 1 || max_rows > LG_HIP_MAX_ROWS) return fail(-2, "model_commit: max_rows %d outside 1..%d", max_rows, LG_HIP_MAX_ROWS);
+    HIP_TRY(hipSetDevice(m->device));
+    m->max_rows = max_rows;
+    const int E = m->E, H = m->H, nl = m->n_layer;
+    std::vector<uint8_t> stage;
+    int rc = 0;
+    {
+        const HostTensor *t = find(m, "token_embd.weight");
+        if ((rc = check_mat(t, "token_embd.weight", E, m->n_vocab))) return rc;
+        std::vector<const uint8_t *> rows;
+        push_rows(rows, t, 0, m->n_vocab);
+        if ((rc = upload_tiled(m, rows, E, &m->emb, stage))) return rc;
+    }
+    if ((rc = upload_vec(m, "output_norm.weight", E, true, &m->output_norm))) return rc;
+    int hd_global = 0;
+    for (int L = 0; L < nl; ++L) if (!m->is_local[L]) hd_global = m->head_dim[L];
+    if (find(m, "rope_freqs.weight") && hd_global)
+        if ((rc = upload_vec(m, "rope_freqs.weight", hd_global / 2, true, &m->rope_freqs))) return rc;
+    if (m->ple > 0 && find(m, "per_layer_token_embd.weight")) {
+        if (m->ple % 32) return fail(-2, "model_commit: per-layer width %d", m->ple);
+        const HostTensor *t = find(m, "per_layer_token_embd.weight");
+        const uint64_t total = (uint64_t)m->ple * nl;
+        if (t->type != 2 || t->dims[0] != total || t->dims[1] != (uint64_t)m->n_vocab)
+            return fail(-6, "model_commit: per_layer_token_embd.weight must be q4_0 %llu x %d", (unsigned long long)total, m->n_vocab);
+        const size_t bytes = (size_t)m->n_vocab * (total / 32) * 18;
+        if (dev_alloc(m, &m->pte, bytes)) return -7;
+        HIP_TRY(hipMemcpy(m->pte, t->data, bytes, hipMemcpyHostToDevice));
+        const HostTensor *p = find(m, "per_layer_model_proj.weight");
+        if ((rc = check_mat(p, "per_layer_model_proj.weight", E, total))) return rc;
+        std::vector<const uint8_t *> rows;
+        push_rows(rows, p, 0, total);
+        if ((rc = upload_tiled(m, rows, E, &m->pmp, stage))) return rc;
+        if ((rc = upload_vec(m, "per_layer_proj_norm.weight", m->ple, true, &m->proj_norm))) return rc;
+    } else m->ple = 0;
+
+    m->L.resize(nl);
+    int max_qkv = 0, max_ff = 0, max_qd = 0;
+    for (int L = 0; L < nl; ++L) {
+        Layer &y = m->L[L];
+        y.is_local = m->is_local[L]; y.hd = m->head_dim[L]; y.nkv = m->n_head_kv[L]; y.nff = m->ffn_len[L];
+        if (y.hd != 64 && y.hd != 128 && y.hd != 256 && y.hd != 512) return fail(-2, "model_commit: layer %d head size %d (64/128/256/512 are built)", L, y.hd);
+        if (y.nkv <= 0 || H % y.nkv || (H / y.nkv) * max_rows > 32) return fail(-2, "model_commit: layer %d: heads %d / kv heads %d with %d rows exceeds 32 queries per kv head", L, H, y.nkv, max_rows);
+        if (y.nff % 32) return fail(-2, "model_commit: layer %d feed-forward width %d must be a multiple of 32", L, y.nff);
+        y.qd = H * y.hd; y.kd = y.nkv * y.hd;
+        y.owns = L < m->n_kv_start;
+        y.src = y.owns ? L : m->n_kv_start - (y.is_local ? 2 : 1);          // src/cpu/model-cpu.c:175-179
+        if (y.src < 0) return fail(-2, "model_commit: layer %d has no layer to share KV with", L);
+        const HostTensor *q = find(m, lname(L, "attn_q.weight")), *k = find(m, lname(L, "attn_k.weight")),
+                         *v = find(m, lname(L, "attn_v.weight"));
+        if ((rc = check_mat(q, lname(L, "attn_q.weight"), E, y.qd))) return rc;
+        std::vector<const uint8_t *> rows;
+        push_rows(rows, q, 0, y.qd);
+        y.qkv_m = y.qd;
+        if (y.owns) {
+            if ((rc = check_mat(k, lname(L, "attn_k.weight"), E, y.kd))) return rc;
+            push_rows(rows, k, 0, y.kd);
+            y.k_off = y.qd; y.v_off = y.qd; y.qkv_m += y.kd;                // no attn_v: V = raw K projection
+            if (v) {
+                if ((rc = check_mat(v, lname(L, "attn_v.weight"), E, y.kd))) return rc;
+                push_rows(rows, v, 0, y.kd);
+                y.v_off = y.qd + y.kd; y.qkv_m += y.kd;
+            }
+        }
+        if ((rc = upload_tiled(m, rows, E, &y.wqkv, stage))) return rc;
+        rows.clear();
+        const HostTensor *o = find(m, lname(L, "attn_output.weight"));
+        if ((rc = check_mat(o, lname(L, "attn_output.weight"), y.qd, E))) return rc;
+        push_rows(rows, o, 0, E);
+        if ((rc = upload_tiled(m, rows, y.qd, &y.wo, stage))) return rc;
+        rows.clear();
+        const HostTensor *g = find(m, lname(L, "ffn_gate.weight")), *u = find(m, lname(L, "ffn_up.weight")),
+                         *d = find(m, lname(L, "ffn_down.weight"));
+        if ((rc = check_mat(g, lname(L, "ffn_gate.weight"), E, y.nff))) return rc;
+        if ((rc = check_mat(u, lname(L, "ffn_up.weight"), E, y.nff))) return rc;
+        if ((rc = check_mat(d, lname(L, "ffn_down.weight"), y.nff, E))) return rc;
+        for (int t = 0; t < y.nff / 32; ++t) { push_rows(rows, g, (uint64_t)t * 32, 32); push_rows(rows, u, (uint64_t)t * 32, 32); }
+        if ((rc = upload_tiled(m, rows, E, &y.wgu, stage))) return rc;
+        rows.clear();
+        push_rows(rows, d, 0, E);
+        if ((rc = upload_tiled(m, rows, y.nff, &y.wdown, stage))) return rc;
+        rows.clear();
+        if (m->ple) {
+            if (m->ple % 256) return fail(-2, "model_commit: per-layer width %d must be a multiple of 256", m->ple);
+            const HostTensor *ig = find(m, lname(L, "inp_gate.weight")), *pj = find(m, lname(L, "proj.weight"));
+            if ((rc = check_mat(ig, lname(L, "inp_gate.weight"), E, m->ple))) return rc;
+            if ((rc = check_mat(pj, lname(L, "proj.weight"), m->ple, E))) return rc;
+            push_rows(rows, ig, 0, m->ple);
+            if ((rc = upload_tiled(m, rows, E, &y.winp, stage))) return rc;
+            rows.clear();
+            push_rows(rows, pj, 0, E);
+            if ((rc = upload_tiled(m, rows, m->ple, &y.wproj, stage))) return rc;
+            if ((rc = upload_vec(m, lname(L, "post_norm.weight"), E, true, &y.post_norm))) return rc;
+        }
+        if ((rc = upload_vec(m, lname(L, "attn_norm.weight"), E, true, &y.attn_norm))) return rc;
+        if ((rc = upload_vec(m, lname(L, "attn_q_norm.weight"), y.hd, true, &y.q_norm))) return rc;
+        if ((rc = upload_vec(m, lname(L, "attn_k_norm.weight"), y.hd, y.owns, &y.k_norm))) return rc;
+        if ((rc = upload_vec(m, lname(L, "post_attention_norm.weight"), E, true, &y.post_attn))) return rc;
+        if ((rc = upload_vec(m, lname(L, "ffn_norm.weight"), E, true, &y.ffn_norm))) return rc;
+        if ((rc = upload_vec(m, lname(L, "post_ffw_norm.weight"), E, true, &y.post_ffw))) return rc;
+        if ((rc = upload_vec(m, lname(L, "layer_output_scale.weight"), 1, false, &y.out_scale))) return rc;
+        y.rope_tab = rope_table(m, y.is_local, y.hd, &rc);
+        if (!y.rope_tab) return rc;
+        y.rope_ff = y.is_local ? nullptr : m->rope_freqs;
+        if (y.qkv_m > max_qkv) max_qkv = y.qkv_m;
+        if (y.nff > max_ff) max_ff = y.nff;
+        if (y.qd > max_qd) max_qd = y.qd;
+    }
+    m->host.clear();
+    const size_t R = (size_t)max_rows;
+    if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
+        dev_alloc(m, &m->dout, R * E) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
+        dev_alloc(m, &m->aq, R * max_qd) || dev_alloc(m, &m->ads, R * max_qd / 32) ||
+        dev_alloc(m, &m->gq, R * max_ff) || dev_alloc(m, &m->gds, R * max_ff / 32) ||
+        dev_alloc(m, &m->hq, R * E) || dev_alloc(m, &m->hds, R * E / 32) ||
+        dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
+        dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
+        return -7;
+    if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple) || dev_alloc(m, &m->pds, R * m->ple / 32)))
+        return -7;
+    HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
+    HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
+    m->sched_cap = 4096;
+    if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
+        dev_alloc(m, &m->adv, (size_t)m->sched_cap))
+        return -7;
+    HIP_TRY(hipHostMalloc((void **)&m->pin, 256 * sizeof(int32_t), hipHostMallocDefault));
+    HIP_TRY(hipDeviceSynchronize());
+    m->committed = true;
+    return 0;
+}
+
+extern "C" void lg_hip_model_destroy(lg_hip_model *m) {
+    if (!m) return;
+    (void)hipSetDevice(m->device);
+    (void)hipDeviceSynchronize();
+    for (auto &g : m->graphs) (void)hipGraphExecDestroy(g.second);
+    for (void *p : m->allocs) (void)hipFree(p);
+    for (hipEvent_t e : m->prof.ev) (void)hipEventDestroy(e);
+    if (m->pin) (void)hipHostFree(m->pin);
+    if (m->stream) (void)hipStreamDestroy(m->stream);
+    delete m;
+}
+
+// ---- KV cache ---------------------------------------------------------------------------------
+extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
+    if (!m || !out || !m->committed) return fail(-1, "kv_create: model not committed");
+    if (max_seq < 1) return fail(-2, "kv_create: max_seq %d", max_seq);
+    HIP_TRY(hipSetDevice(m->device));
+    lg_hip_kv *kv = new lg_hip_kv();
+    kv->m = m; kv->max_seq = max_seq; kv->id = ++g_kv_ids;
+    const int nl = m->n_layer;
+    kv->seq.assign(nl, 0); kv->kv_dim.assign(nl, 0);
+    kv->k.assign(nl, nullptr); kv->v.assign(nl, nullptr); kv->px_k.assign(nl, nullptr); kv->px_v.assign(nl, nullptr);
+    int tiles = 1, max_hd = 0;
+    for (int L = 0; L < nl; ++L) {
+        const Layer &y = m->L[L];
+        kv->kv_dim[L] = y.kd;
+        if (y.hd > max_hd) max_hd = y.hd;
+        const bool ring = y.is_local && m->window > 0;
+        const int span = ring ? m->window + LG_HIP_MAX_ROWS : max_seq;       // keys any block can touch
+        int t = (span < max_seq ? span : max_seq) / 32 + 2;
+        if (t > tiles) tiles = t;
+        if (!y.owns) continue;
+        kv->seq[L] = ring ? lg_hip_ring_rows(m->window, max_seq) : max_seq;
+        const size_t bytes = (size_t)kv->seq[L] * y.kd * 2;
+        hipError_t e1 = hipMalloc((void **)&kv->k[L], bytes), e2 = hipMalloc((void **)&kv->v[L], bytes);
+        if (e1 != hipSuccess || e2 != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory at layer %d", L); }
+        (void)hipMemset(kv->k[L], 0, bytes); (void)hipMemset(kv->v[L], 0, bytes);
+    }
+    kv->tiles_max = tiles;
+    const size_t slots = (size_t)m->max_rows * m->H * tiles;
+    if (hipMalloc((void **)&kv->pm, slots * 4) != hipSuccess || hipMalloc((void **)&kv->pl, slots * 4) != hipSuccess ||
+        hipMalloc((void **)&kv->pacc, slots * max_hd * 4) != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory for attention partials"); }
+    HIP_TRY(hipDeviceSynchronize());
+    *out = kv;
+    return 0;
+}
+
+extern "C" void lg_hip_kv_destroy(lg_hip_kv *kv) {
+    if (!kv) return;
+    (void)hipSetDevice(kv->m->device);
+    (void)hipDeviceSynchronize();
+    // graphs captured for this cache hold its pointers
+    const std::string tag = "kv" + std::to_string(kv->id) + ":";
+    for (auto it = kv->m->graphs.begin(); it != kv->m->graphs.end();) {
+        if (it->first.compare(0, tag.size(), tag) == 0) { (void)hipGraphExecDestroy(it->second); it = kv->m->graphs.erase(it); }
+        else ++it;
+    }
+    for (size_t L = 0; L < kv->k.size(); ++L) {
+        (void)hipFree(kv->k[L]); (void)hipFree(kv->v[L]); (void)hipFree(kv->px_k[L]); (void)hipFree(kv->px_v[L]);
+    }
+    (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc);
+    delete kv;
+}
+
+extern "C" int lg_hip_kv_layout(const lg_hip_kv *kv, int layer, int *rows, int *width) {
+    if (!kv || layer < 0 || layer >= (int)kv->seq.size()) return fail(-1, "kv_layout: bad layer %d", layer);
+    if (rows) *rows = kv->seq[layer];
+    if (width) *width = kv->kv_dim[layer];
+    return 0;
+}
+static int kv_span(const lg_hip_kv *kv, int layer, int which, int row0, int n, size_t *off, size_t *bytes, uint16_t **base) {
+    if (!kv || layer < 0 || layer >= (int)kv->seq.size() || !kv->k[layer]) return fail(-1, "kv copy: layer %d owns no cache", layer);
+    if (row0 < 0 || n < 0 || row0 + n > kv->seq[layer]) return fail(-2, "kv copy: rows %d..%d outside 0..%d", row0, row0 + n, kv->seq[layer]);
+    *off = (size_t)row0 * kv->kv_dim[layer];
+    *bytes = (size_t)n * kv->kv_dim[layer] * 2;
+    *base = which ? kv->v[layer] : kv->k[layer];
+    return 0;
+}
+extern "C" int lg_hip_kv_write(lg_hip_kv *kv, int layer, int which, int row0, int n, const uint16_t *src) {
+    size_t off, bytes; uint16_t *base;
+    int rc = kv_span(kv, layer, which, row0, n, &off, &bytes, &base);
+    if (rc) return rc;
+    HIP_TRY(hipSetDevice(kv->m->device));
+    HIP_TRY(hipStreamSynchronize(kv->m->stream));
+    HIP_TRY(hipMemcpy(base + off, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+extern "C" int lg_hip_kv_read(const lg_hip_kv *kv, int layer, int which, int row0, int n, uint16_t *dst) {
+    size_t off, bytes; uint16_t *base;
+    int rc = kv_span(kv, layer, which, row0, n, &off, &bytes, &base);
+    if (rc) return rc;
+    HIP_TRY(hipSetDevice(kv->m->device));
+    HIP_TRY(hipStreamSynchronize(kv->m->stream));
+    HIP_TRY(hipMemcpy(dst, base + off, bytes, hipMemcpyDeviceToHost));
+    return 0;
+}
+extern "C" int lg_hip_kv_save_prefix(lg_hip_kv *kv, int n) {
+    if (!kv || n < 0) return fail(-1, "kv_save_prefix: bad argument");
+    HIP_TRY(hipSetDevice(kv->m->device));
+    HIP_TRY(hipStreamSynchronize(kv->m->stream));
+    for (size_t L = 0; L < kv->k.size(); ++L) {
+        if (!kv->k[L]) continue;
+        const int rows = n < kv->seq[L] ? n : kv->seq[L];
+        const size_t bytes = (size_t)rows * kv->kv_dim[L] * 2;
+        (void)hipFree(kv->px_k[L]); (void)hipFree(kv->px_v[L]);
+        kv->px_k[L] = kv->px_v[L] = nullptr;
+        if (!bytes) continue;
+        HIP_TRY(hipMalloc((void **)&kv->px_k[L], bytes));
+        HIP_TRY(hipMalloc((void **)&kv->px_v[L], bytes));
+        HIP_TRY(hipMemcpy(kv->px_k[L], kv->k[L], bytes, hipMemcpyDeviceToDevice));
+        HIP_TRY(hipMemcpy(kv->px_v[L], kv->v[L], bytes, hipMemcpyDeviceToDevice));
+    }
+    return 0;
+}
+extern "C" int lg_hip_kv_restore_prefix(lg_hip_kv *kv, int n) {
+    if (!kv || n < 0) return fail(-1, "kv_restore_prefix: bad argument");
+    HIP_TRY(hipSetDevice(kv->m->device));
+    for (size_t L = 0; L < kv->k.size(); ++L) {
+        if (!kv->px_k[L]) continue;
+        const int rows = n < kv->seq[L] ? n : kv->seq[L];
+        const size_t bytes = (size_t)rows * kv->kv_dim[L] * 2;
+        HIP_TRY(hipMemcpyAsync(kv->k[L], kv->px_k[L], bytes, hipMemcpyDeviceToDevice, kv->m->stream));
+        HIP_TRY(hipMemcpyAsync(kv->v[L], kv->px_v[L], bytes, hipMemcpyDeviceToDevice, kv->m->stream));
+    }
+    return 0;
+}
+
+// ---- launching --------------------------------------------------------------------------------
+static size_t lds_mm(int M, int k) { return (size_t)M * k + (size_t)M * (k / 32) * 8; }
+
+// Kernels that want more than the default dynamic LDS limit have it raised once per (kernel, size).
+template <typename K>
+static int set_lds(K kernel, size_t bytes) {
+    static std::map<const void *, size_t> raised;
+    if (bytes <= 48 * 1024) return 0;
+    if (bytes > 160 * 1024) return fail(-8, "kernel needs %zu bytes of LDS (160 KiB per workgroup)", bytes);
+    const void *fn = reinterpret_cast<const void *>(kernel);
+    auto it = raised.find(fn);
+    if (it != raised.end() && it->second >= bytes) return 0;
+    HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+    raised[fn] = bytes;
+    return 0;
+}
+
+struct Launcher {
+    lg_hip_model *m;
+    bool dry;              // only raise LDS limits, launch nothing (done once before a capture)
+    int rc = 0;
+    void begin(int cls) {
+        if (!m->prof.on || rc) return;
+        hipEvent_t a, b;
+        if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { rc = fail(-9, "event create failed"); return; }
+        m->prof.ev.push_back(a); m->prof.ev.push_back(b); m->prof.cls.push_back(cls);
+        (void)hipEventRecord(a, m->stream);
+    }
+    void end() {
+        if (m->prof.on && !rc) (void)hipEventRecord(m->prof.ev.back(), m->stream);
+        if (!rc) { hipError_t e = hipGetLastError(); if (e != hipSuccess) rc = fail(-100 - (int)e, "kernel launch failed: %s", hipGetErrorString(e)); }
+    }
+};
+
+#define LAUNCH(cls, kernel, grid, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { lx.begin(cls); \
+    hipLaunchKernelGGL(kernel, grid, dim3(LG_WG), lds, m->stream, __VA_ARGS__); lx.end(); } } while (0)
+
+// one block of M rows through the decoder (and the head when with_head)
+template <int M>
+static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry) {
+    Launcher lx{ m, dry };
+    const int E = m->E, H = m->H, nl = m->n_layer;
+    int cur = 0;                                   // x[cur] holds the residual
+    ActSrc base{};
+    base.E = E; base.eps = m->eps; base.toks = m->sched;
+    bool have_x = false;                           // false: rows are still token ids
+    const float *pend_dout = nullptr, *pend_w = nullptr, *pend_os = nullptr;   // sub-layer output waiting to be added
+
+    auto src_for = [&](const float *w_pre, bool write_x) {
+        ActSrc s = base;
+        if (!have_x) { s.emb = m->emb; s.emb_nit = E / 256; s.emb_scale = sqrtf((float)E); }
+        else s.x = m->x[cur];
+        s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os;
+        s.w_pre = w_pre;
+        if (write_x && (pend_dout || !have_x)) { s.x_out = m->x[cur ^ 1]; }
+        return s;
+    };
+    auto consumed = [&](const ActSrc &s) {         // after a prologue that wrote x_out
+        if (s.x_out) cur ^= 1;
+        have_x = true; pend_dout = pend_w = pend_os = nullptr;
+    };
+
+    if (m->ple) {
+        ActSrc s = src_for(nullptr, true);
+        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, nullptr, nullptr, nullptr };
+        LAUNCH(KC_PMP, (lg_k_mm<M, SRC_ACT, false>), dim3((a.m / 8 + 3) / 4), lds_mm(M, E), a, s, m->ctl);
+        consumed(s);
+    }
+    for (int L = 0; L < nl && !lx.rc; ++L) {
+        const Layer &y = m->L[L];
+        {   // q/k/v projections on rmsnorm(x) * attn_norm
+            ActSrc s = src_for(y.attn_norm, true);
+            MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, nullptr, nullptr, nullptr };
+            LAUNCH(KC_QKV, (lg_k_mm<M, SRC_ACT, false>), dim3((a.m / 8 + 3) / 4), lds_mm(M, E), a, s, m->ctl);
+            consumed(s);
+        }
+        {   // attention tiles + merge
+            const int G = H / y.nkv, nq = G * M, kst = y.hd + 8;
+            AttnArgs a{};
+            a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
+            a.H = H; a.nkv = y.nkv; a.hd = y.hd;
+            a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
+            a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd;
+            a.window = (y.is_local && m->window > 0) ? m->window : 0;
+            a.owns = y.owns; a.prerotated = 0; a.eps = m->eps;
+            a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max;
+            const size_t lds = (size_t)(nq + M) * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
+            LAUNCH(KC_ATTN, (lg_k_attn<M>), dim3(kv->tiles_max, y.nkv), lds, a, m->ctl);
+            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, a.window, m->aq, m->ads, nullptr };
+            LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), 0, g, m->ctl);
+        }
+        {   // attention output projection
+            MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, m->ads, nullptr };
+            LAUNCH(KC_O, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, y.qd), a, base, m->ctl);
+            pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
+        }
+        {   // feed-forward: gate/up + GeGLU, then down
+            ActSrc s = src_for(y.ffn_norm, true);
+            GegluArgs a{ y.wgu, E, y.nff, m->gq, m->gds };
+            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M>), dim3(y.nff / 32), lds_mm(M, E), a, s, m->ctl);
+            consumed(s);
+            MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, m->gds, nullptr };
+            LAUNCH(KC_DOWN, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, y.nff), d, base, m->ctl);
+            pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
+        }
+        if (m->ple) {   // per-layer embedding block
+            ActSrc s = src_for(nullptr, true);
+            PleGateArgs a{};
+            a.w = y.winp; a.k = E; a.ple = m->ple; a.pmp_raw = m->pmp_raw; a.layer = L; a.n_layer = nl;
+            a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
+            a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
+            a.pq = m->pq; a.pds = m->pds;
+            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), lds_mm(M, E) + (size_t)M * m->ple * 4, a, s, m->ctl);
+            consumed(s);
+            MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, m->pds, nullptr };
+            LAUNCH(KC_PLEPROJ, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, m->ple), p, base, m->ctl);
+            pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
+        }
+    }
+    if (with_head && !lx.rc) {
+        ActSrc s = src_for(m->output_norm, false);
+        s.h_out = m->hidden_rows;
+        QuantArgs q{ m->hq, m->hds };
+        LAUNCH(KC_FINALNORM, (lg_k_act_quant<M>), dim3(1), 0, q, s, m->ctl);
+        HeadArgs h{ m->emb, E, m->n_vocab, m->hq, m->hds, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
+        LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(m->n_vocab / 32), lds_mm(M, E), h);
+        AcceptArgs c{ m->pval, m->pidx, m->n_vocab / 32, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
+        LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), 0, c, m->ctl);
+    } else if (!lx.rc && !dry) {
+        hipLaunchKernelGGL(lg_k_advance, dim3(1), dim3(1), 0, m->stream, m->ctl, M);
+    }
+    return lx.rc;
+}
+
+static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head, bool dry = false) {
+    switch (rows) {
+        case 1: return enqueue_step<1>(m, kv, with_head, dry);
+        case 2: return enqueue_step<2>(m, kv, with_head, dry);
+        case 3: return enqueue_step<3>(m, kv, with_head, dry);
+        case 4: return enqueue_step<4>(m, kv, with_head, dry);
+        case 5: return enqueue_step<5>(m, kv, with_head, dry);
+        case 6: return enqueue_step<6>(m, kv, with_head, dry);
+        case 7: return enqueue_step<7>(m, kv, with_head, dry);
+        case 8: return enqueue_step<8>(m, kv, with_head, dry);
+    }
+    return fail(-2, "rows %d outside 1..%d", rows, LG_HIP_MAX_ROWS);
+}
+
+// launch one step, through a captured graph when enabled
+static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
+    if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "");
+    auto it = m->graphs.find(key);
+    if (it == m->graphs.end()) {
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        int rc = enqueue_step_rows(m, kv, rows, with_head, true);
+        if (rc) return rc;
+        HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        rc = enqueue_step_rows(m, kv, rows, with_head);
+        hipError_t e = hipStreamEndCapture(m->stream, &graph);
+        if (rc) { if (graph) (void)hipGraphDestroy(graph); return rc; }
+        if (e != hipSuccess) return fail(-100 - (int)e, "hipStreamEndCapture: %s", hipGetErrorString(e));
+        e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        if (e != hipSuccess) return fail(-100 - (int)e, "hipGraphInstantiate: %s", hipGetErrorString(e));
+        it = m->graphs.emplace(key, exec).first;
+    }
+    HIP_TRY(hipGraphLaunch(it->second, m->stream));
+    return 0;
+}
+
+static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int rows, int pos) {
+    if (!m || !kv || !toks || kv->m != m) return fail(-1, "bad model / cache / token pointer");
+    if (rows < 1 || rows > m->max_rows) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
+    if (pos < 0 || pos + rows > kv->max_seq) return fail(-2, "positions %d..%d do not fit a cache of %d", pos, pos + rows - 1, kv->max_seq);
+    for (int i = 0; i < n; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "token id %d outside the vocabulary of %d", toks[i], m->n_vocab);
+    return 0;
+}
+
+extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
+    if (!m || !name) return fail(-1, "set_option: null argument");
+    if (!strcmp(name, "store_logits")) m->store_logits = value != 0;
+    else if (!strcmp(name, "use_graph")) m->use_graph = value != 0;
+    else return fail(-2, "set_option: unknown option %s", name);
+    return 0;
+}
+
+static int load_block(lg_hip_model *m, const int32_t *toks, int rows, int pos) {
+    StepCtl c{ pos, 0, 0, 0 };
+    memcpy(m->pin, &c, sizeof c);
+    memcpy(m->pin + 8, toks, (size_t)rows * 4);
+    HIP_TRY(hipMemcpyAsync(m->ctl, m->pin, sizeof c, hipMemcpyHostToDevice, m->stream));
+    HIP_TRY(hipMemcpyAsync(m->sched, m->pin + 8, (size_t)rows * 4, hipMemcpyHostToDevice, m->stream));
+    return 0;
+}
+
+extern "C" int lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int rows, int pos,
+                                   int32_t *out, int32_t *adv) {
+    int rc = check_block(m, kv, toks, rows, rows, pos);
+    if (rc) return rc;
+    if (!out || !adv) return fail(-1, "forward_spec: null output");
+    HIP_TRY(hipSetDevice(m->device));
+    if ((rc = load_block(m, toks, rows, pos))) return rc;
+    if ((rc = launch_step(m, kv, rows, true))) return rc;
+    HIP_TRY(hipMemcpyAsync(m->pin + 32, m->out, (size_t)rows * 4, hipMemcpyDeviceToHost, m->stream));
+    HIP_TRY(hipMemcpyAsync(m->pin + 48, m->adv, 4, hipMemcpyDeviceToHost, m->stream));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    memcpy(out, m->pin + 32, (size_t)rows * 4);
+    *adv = m->pin[48];
+    m->last_rows = rows; m->last_adv = *adv;
+    return 0;
+}
+
+extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int pos0) {
+    if (n <= 0) return 0;
+    if (!m) return fail(-1, "prefill: null model");
+    HIP_TRY(hipSetDevice(m->device));
+    for (int done = 0; done < n;) {
+        const int rows = n - done < m->max_rows ? n - done : m->max_rows;
+        int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done);
+        if (rc) return rc;
+        if ((rc = load_block(m, toks + done, rows, pos0 + done))) return rc;
+        if ((rc = launch_step(m, kv, rows, false))) return rc;
+        HIP_TRY(hipStreamSynchronize(m->stream));       // the pinned staging is reused by the next block
+        done += rows;
+    }
+    return 0;
+}
+
+extern "C" int lg_hip_get_hidden(lg_hip_model *m, float *dst) {
+    if (!m || !dst) return fail(-1, "get_hidden: null argument");
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    HIP_TRY(hipMemcpy(dst, m->g_hidden, (size_t)m->E * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+extern "C" int lg_hip_set_hidden_row(lg_hip_model *m, int row) {
+    if (!m) return fail(-1, "set_hidden_row: null model");
+    if (row < 0 || row >= m->last_rows) return fail(-2, "set_hidden_row: row %d of a %d-row step", row, m->last_rows);
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipMemcpyAsync(m->g_hidden, m->hidden_rows + (size_t)row * m->E, (size_t)m->E * 4, hipMemcpyDeviceToDevice, m->stream));
+    return 0;
+}
+extern "C" int lg_hip_get_logits(lg_hip_model *m, int row, float *dst) {
+    if (!m || !dst) return fail(-1, "get_logits: null argument");
+    if (!m->store_logits) return fail(-4, "get_logits: the store_logits option is off");
+    if (row < 0 || row >= m->last_rows) return fail(-2, "get_logits: row %d of a %d-row step", row, m->last_rows);
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    HIP_TRY(hipMemcpy(dst, m->logits + (size_t)row * m->n_vocab, (size_t)m->n_vocab * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// ---- device-resident schedule -----------------------------------------------------------------
+extern "C" int lg_hip_schedule_load(lg_hip_model *m, const int32_t *toks, int n_steps, int rows, int pos0) {
+    if (!m || !toks || !m->committed) return fail(-1, "schedule_load: bad argument");
+    if (rows < 1 || rows > m->max_rows || n_steps < 1 || n_steps > m->sched_cap) return fail(-2, "schedule_load: %d steps of %d rows (limits %d, %d)", n_steps, rows, m->sched_cap, m->max_rows);
+    for (size_t i = 0; i < (size_t)n_steps * rows; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "schedule_load: token id %d outside the vocabulary", toks[i]);
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    HIP_TRY(hipMemcpy(m->sched, toks, (size_t)n_steps * rows * 4, hipMemcpyHostToDevice));
+    StepCtl c{ pos0, 0, 0, 0 };
+    HIP_TRY(hipMemcpy(m->ctl, &c, sizeof c, hipMemcpyHostToDevice));
+    m->sched_steps = n_steps; m->sched_rows = rows;
+    return 0;
+}
+extern "C" int lg_hip_schedule_run(lg_hip_model *m, lg_hip_kv *kv, int n_steps) {
+    if (!m || !kv || kv->m != m) return fail(-1, "schedule_run: bad argument");
+    if (n_steps < 1 || n_steps > m->sched_steps) return fail(-2, "schedule_run: %d steps requested, %d loaded", n_steps, m->sched_steps);
+    HIP_TRY(hipSetDevice(m->device));
+    for (int s = 0; s < n_steps; ++s) { int rc = launch_step(m, kv, m->sched_rows, true); if (rc) return rc; }
+    m->sched_steps -= n_steps;       // steps left to run
+    m->last_rows = m->sched_rows;
+    return 0;
+}
+extern "C" int lg_hip_schedule_wait(lg_hip_model *m, int32_t *out, int32_t *adv, int32_t *final_pos) {
+    if (!m) return fail(-1, "schedule_wait: null model");
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    StepCtl c;
+    HIP_TRY(hipMemcpy(&c, m->ctl, sizeof c, hipMemcpyDeviceToHost));
+    if (out) HIP_TRY(hipMemcpy(out, m->out, (size_t)c.step * m->sched_rows * 4, hipMemcpyDeviceToHost));
+    if (adv) HIP_TRY(hipMemcpy(adv, m->adv, (size_t)c.step * 4, hipMemcpyDeviceToHost));
+    if (final_pos) *final_pos = c.pos;
+    return c.step;
+}
+extern "C" int lg_hip_schedule_time(lg_hip_model *m, lg_hip_kv *kv, int n_steps, float *ms) {
+    if (!m || !ms) return fail(-1, "schedule_time: null argument");
+    HIP_TRY(hipSetDevice(m->device));
+    hipEvent_t a, b;
+    HIP_TRY(hipEventCreate(&a));
+    HIP_TRY(hipEventCreate(&b));
+    HIP_TRY(hipEventRecord(a, m->stream));
+    int rc = lg_hip_schedule_run(m, kv, n_steps);
+    if (!rc) {
+        (void)hipEventRecord(b, m->stream);
+        hipError_t e = hipEventSynchronize(b);
+        if (e != hipSuccess) rc = fail(-100 - (int)e, "hipEventSynchronize: %s", hipGetErrorString(e));
+        else (void)hipEventElapsedTime(ms, a, b);
+    }
+    (void)hipEventDestroy(a); (void)hipEventDestroy(b);
+    return rc;
+}
+
+// ---- measurement ------------------------------------------------------------------------------
+static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int rows, double *b) {
+    const double q = 18.0 / 32.0;                         // bytes per q4_0 weight
+    for (int i = 0; i < KC_COUNT; ++i) b[i] = 0;
+    if (m->ple) b[KC_PMP] = (double)m->E * m->ple * m->n_layer * q;
+    for (int L = 0; L < m->n_layer; ++L) {
+        const Layer &y = m->L[L];
+        b[KC_QKV] += (double)m->E * y.qkv_m * q;
+        b[KC_O] += (double)y.qd * m->E * q;
+        b[KC_GATEUP] += 2.0 * m->E * y.nff * q;
+        b[KC_DOWN] += (double)y.nff * m->E * q;
+        if (m->ple) { b[KC_PLEGATE] += (double)m->E * m->ple * q; b[KC_PLEPROJ] += (double)m->ple * m->E * q; }
+        const int window = (y.is_local && m->window > 0) ? m->window : 0;
+        const int last = pos + rows - 1, start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+        b[KC_ATTN] += 2.0 * (last - start + 1) * y.kd * 2.0;          // K and V rows, f16
+    }
+    b[KC_HEAD] = (double)m->E * m->n_vocab * q;
+    (void)kv;
+}
+
+extern "C" int lg_hip_profile_step(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int rows, int pos, int repeats,
+                                   const char **names, float *ms, int32_t *launches, double *bytes, int cap) {
+    int rc = check_block(m, kv, toks, rows, rows, pos);
+    if (rc) return rc;
+    if (cap < KC_COUNT || repeats < 1) return fail(-2, "profile_step: need room for %d classes", KC_COUNT);
+    HIP_TRY(hipSetDevice(m->device));
+    double acc[KC_COUNT] = { 0 };
+    int cnt[KC_COUNT] = { 0 };
+    for (int r = 0; r < repeats + 1; ++r) {              // first pass warms up and is dropped
+        if ((rc = load_block(m, toks, rows, pos))) return rc;
+        m->prof.on = true;
+        rc = enqueue_step_rows(m, kv, rows, true);
+        m->prof.on = false;
+        hipError_t e = hipStreamSynchronize(m->stream);
+        if (!rc && e != hipSuccess) rc = fail(-100 - (int)e, "profile_step: %s", hipGetErrorString(e));
+        for (size_t i = 0; i < m->prof.cls.size(); ++i) {
+            float t = 0;
+            if (!rc && r > 0 && hipEventElapsedTime(&t, m->prof.ev[2 * i], m->prof.ev[2 * i + 1]) == hipSuccess) { acc[m->prof.cls[i]] += t; cnt[m->prof.cls[i]]++; }
+        }
+        for (hipEvent_t ev : m->prof.ev) (void)hipEventDestroy(ev);
+        m->prof.ev.clear(); m->prof.cls.clear();
+        if (rc) return rc;
+    }
+    double b[KC_COUNT];
+    class_bytes(m, kv, pos, rows, b);
+    for (int i = 0; i < KC_COUNT; ++i) {
+        names[i] = k_class_names[i]; ms[i] = (float)(acc[i] / repeats); launches[i] = cnt[i] / repeats; bytes[i] = b[i];
+    }
+    m->last_rows = rows;
+    return KC_COUNT;
+}
+
+// ---- isolated kernels -------------------------------------------------------------------------
+struct Scratch {            // device buffers freed on scope exit
+    std::vector<void *> p;
+    ~Scratch() { for (void *q : p) (void)hipFree(q); }
+    template <typename T> int get(T **out, size_t n) {
+        HIP_TRY(hipMalloc((void **)out, n * sizeof(T) ? n * sizeof(T) : 16));
+        p.push_back(*out);
+        return 0;
+    }
+};
+
+template <int M>
+static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, const float *dx, float *dout, int32_t *ddots,
+                       int8_t *dq, float2 *dds, StepCtl *ctl, int repeats, float *kernel_ms) {
+    ActSrc s{};
+    const int n32 = M * (k / 32);
+    hipLaunchKernelGGL(lg_k_quant_flat, dim3((n32 * 8 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, st, dx, n32, dq, dds);
+    MmArgs a{ dw, k, mrows, dout, dq, dds, ddots };
+    const size_t lds = lds_mm(M, k);
+    int rc;
+    if (ddots) { if ((rc = set_lds(lg_k_mm<M, SRC_Q8, true>, lds))) return rc; }
+    if ((rc = set_lds(lg_k_mm<M, SRC_Q8, false>, lds))) return rc;
+    const dim3 grid((mrows / 8 + 3) / 4);
+    if (ddots) hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, true>), grid, dim3(LG_WG), lds, st, a, s, ctl);
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+    a.dots = nullptr;
+    hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, false>), grid, dim3(LG_WG), lds, st, a, s, ctl);       // warm-up, also the result
+    HIP_TRY(hipEventRecord(e0, st));
+    for (int r = 0; r < repeats; ++r) hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, false>), grid, dim3(LG_WG), lds, st, a, s, ctl);
+    HIP_TRY(hipEventRecord(e1, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    HIP_TRY(hipGetLastError());
+    float t = 0;
+    if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+    if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    return 0;
+}
+
+extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *x, int rows, float *out, int32_t *dots,
+                                  int8_t *xq, float *xd, int32_t *xsum, int repeats, float *kernel_ms) {
+    if (!w || !x) return fail(-1, "matmul: null input");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || !lg_hip_repacked_bytes(k, mrows) || lds_mm(rows, k) > 160 * 1024)
+        return fail(-2, "matmul: rows %d (1..%d), k %d (multiple of 256, rows*k*1.25 <= 160 KiB), m %d (multiple of 8)", rows, LG_HIP_MAX_ROWS, k, mrows);
+    if (lg_hip_device_count() < 1) return fail(-3, "matmul: no HIP device");
+    const int nb = k / 32;
+    std::vector<uint8_t> tiled(lg_hip_repacked_bytes(k, mrows));
+    int rc = lg_hip_repack_q4_0(w, k, mrows, tiled.data());
+    if (rc) return rc;
+    Scratch sc;
+    uint8_t *dw; float *dx, *dout; int32_t *ddots = nullptr; int8_t *dq; float2 *dds; StepCtl *ctl;
+    if (sc.get(&dw, tiled.size()) || sc.get(&dx, (size_t)rows * k) || sc.get(&dout, (size_t)rows * mrows) ||
+        sc.get(&dq, (size_t)rows * k) || sc.get(&dds, (size_t)rows * nb) || sc.get(&ctl, (size_t)1)) return -7;
+    if (dots && sc.get(&ddots, (size_t)rows * mrows * nb)) return -7;
+    HIP_TRY(hipMemcpy(dw, tiled.data(), tiled.size(), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dx, x, (size_t)rows * k * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    hipStream_t st;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    switch (rows) {
+#define CASE(M) case M: rc = matmul_rows<M>(st, dw, k, mrows, dx, dout, ddots, dq, dds, ctl, repeats, kernel_ms); break;
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+    }
+    (void)hipStreamDestroy(st);
+    if (rc) return rc;
+    if (out) HIP_TRY(hipMemcpy(out, dout, (size_t)rows * mrows * 4, hipMemcpyDeviceToHost));
+    if (dots) HIP_TRY(hipMemcpy(dots, ddots, (size_t)rows * mrows * nb * 4, hipMemcpyDeviceToHost));
+    if (xq) HIP_TRY(hipMemcpy(xq, dq, (size_t)rows * k, hipMemcpyDeviceToHost));
+    if (xd || xsum) {
+        std::vector<float2> ds((size_t)rows * nb);
+        HIP_TRY(hipMemcpy(ds.data(), dds, ds.size() * 8, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < ds.size(); ++i) {
+            if (xd) xd[i] = ds[i].x;
+            if (xsum) memcpy(&xsum[i], &ds[i].y, 4);
+        }
+    }
+    return 0;
+}
+
+template <int M>
+static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl, int tiles, int repeats, float *kernel_ms) {
+    const int G = a.H / a.nkv, nq = G * M, kst = a.hd + 8;
+    const size_t lds = (size_t)(nq + M) * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
+    int rc = set_lds(lg_k_attn<M>, lds);
+    if (rc) return rc;
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+    for (int r = 0; r < repeats + 1; ++r) {
+        if (r == 1) HIP_TRY(hipEventRecord(e0, st));
+        hipLaunchKernelGGL((lg_k_attn<M>), dim3(tiles, a.nkv), dim3(LG_WG), lds, st, a, ctl);
+        hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
+    }
+    HIP_TRY(hipEventRecord(e1, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    HIP_TRY(hipGetLastError());
+    float t = 0;
+    if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+    if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    return 0;
+}
+
+extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, int rows, int n_head, int n_head_kv,
+                                int hd, int seq, int window, int pos, float *out, int repeats, float *kernel_ms) {
+    if (!q || !kc || !vc || !out) return fail(-1, "attention: null argument");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || n_head_kv < 1 || n_head % n_head_kv || (n_head / n_head_kv) * rows > 32 ||
+        (hd != 64 && hd != 128 && hd != 256 && hd != 512) || pos < 0 || seq < 1)
+        return fail(-2, "attention: unsupported shape");
+    if (window > 0 ? seq < window + rows - 1 && seq < pos + rows : seq < pos + rows)
+        return fail(-2, "attention: a cache of %d rows cannot hold the keys of positions up to %d", seq, pos + rows - 1);
+    if (lg_hip_device_count() < 1) return fail(-3, "attention: no HIP device");
+    const int kd = n_head_kv * hd, qd = n_head * hd;
+    const int start0 = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int tiles = ((pos + rows - 1) >> 5) - (start0 >> 5) + 1;
+    Scratch sc;
+    float *dq, *dpm, *dpl, *dpacc, *dxf; uint16_t *dk, *dv; int8_t *dxq; float2 *dxds; StepCtl *ctl;
+    const size_t slots = (size_t)rows * n_head * tiles;
+    if (sc.get(&dq, (size_t)rows * qd) || sc.get(&dk, (size_t)seq * kd) || sc.get(&dv, (size_t)seq * kd) ||
+        sc.get(&dpm, slots) || sc.get(&dpl, slots) || sc.get(&dpacc, slots * hd) || sc.get(&dxf, (size_t)rows * qd) ||
+        sc.get(&dxq, (size_t)rows * qd) || sc.get(&dxds, (size_t)rows * qd / 32) || sc.get(&ctl, (size_t)1)) return -7;
+    HIP_TRY(hipMemcpy(dq, q, (size_t)rows * qd * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dk, kc, (size_t)seq * kd * 2, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dv, vc, (size_t)seq * kd * 2, hipMemcpyHostToDevice));
+    StepCtl c{ pos, 0, 0, 0 };
+    HIP_TRY(hipMemcpy(ctl, &c, sizeof c, hipMemcpyHostToDevice));
+    AttnArgs a{};
+    a.qkv = dq; a.ld = qd; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
+    a.kc = dk; a.vc = dv; a.seq = seq; a.kv_dim = kd; a.window = window; a.owns = 0; a.prerotated = 1; a.eps = 0;
+    a.pm = dpm; a.pl = dpl; a.pacc = dpacc; a.tiles_max = tiles;
+    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, dxq, dxds, dxf };
+    hipStream_t st;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    int rc = 0;
+    switch (rows) {
+#define CASE(M) case M: rc = attention_rows<M>(st, a, g, ctl, tiles, repeats, kernel_ms); break;
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+    }
+    (void)hipStreamDestroy(st);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpy(out, dxf, (size_t)rows * qd * 4, hipMemcpyDeviceToHost));
+    return 0;
+}

@@ -1,0 +1,66 @@
+/* session.c — see session.h. */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "session.h"
+
+int lg_model_forward_spec_n(struct model *m, struct kvcache *kv, const int *toks, int rows, int pos, int *out);
+
+struct lg_session { struct gguf_context *ctx; struct model m; struct kvcache kv; int has_kv; };
+
+struct lg_session *lg_session_open(const char *path) {
+    struct lg_session *s = calloc(1, sizeof *s);
+    if (!s) return NULL;
+    s->ctx = load_gguf(path);
+    if (!s->ctx || model_init(&s->m, s->ctx) != 0) { free_gguf(s->ctx); free(s); return NULL; }
+    return s;
+}
+void lg_session_close(struct lg_session *s) {
+    if (!s) return;
+    if (s->has_kv) kvcache_free(&s->kv);
+    model_free(&s->m);
+    free_gguf(s->ctx);
+    free(s);
+}
+int lg_session_kv(struct lg_session *s, int max_seq) {
+    if (s->has_kv) kvcache_free(&s->kv);
+    s->has_kv = kvcache_init(&s->kv, &s->m, max_seq) == 0;
+    return s->has_kv ? 0 : -1;
+}
+struct model   *lg_session_model(struct lg_session *s) { return &s->m; }
+struct kvcache *lg_session_kvcache(struct lg_session *s) { return s->has_kv ? &s->kv : NULL; }
+void lg_session_prefill(struct lg_session *s, const int *t, int n, int pos0) { model_prefill(&s->m, &s->kv, t, n, pos0); }
+int  lg_session_forward_next(struct lg_session *s, int token, int pos) { return model_forward_next(&s->m, &s->kv, token, pos); }
+void lg_session_forward(struct lg_session *s, int token, int pos, float *logits) { model_forward(&s->m, &s->kv, token, pos, logits); }
+int  lg_session_forward_spec(struct lg_session *s, const int *toks, int rows, int pos, int *out) {
+    return lg_model_forward_spec_n(&s->m, &s->kv, toks, rows, pos, out);
+}
+
+/* The generation loop of the reference (src/run.c:737-768) on token ids: prefill all but the last
+ * prompt token, pick the first token from the last one, then plain or block-speculative greedy
+ * steps; the speculative path falls back to plain steps when a block would not fit the cache
+ * (src/run.c:752) and never emits past n_gen. */
+int lg_session_generate(struct lg_session *s, const int *prompt, int n_prompt, int n_gen, int rows,
+                        const int *drafts, int *emitted, int *steps) {
+    if (n_prompt < 1 || !s->has_kv) return -1;
+    model_prefill(&s->m, &s->kv, prompt, n_prompt - 1, 0);
+    int pos = n_prompt - 1, g = 0, n_steps = 0;
+    int best = model_forward_next(&s->m, &s->kv, prompt[n_prompt - 1], pos++);
+    while (g < n_gen) {
+        emitted[g++] = best;
+        if (rows < 2 || g >= n_gen || pos + rows - 1 >= s->kv.max_seq) {
+            if (g < n_gen) { best = model_forward_next(&s->m, &s->kv, best, pos++); n_steps++; }
+            continue;
+        }
+        int toks[16], out[16];
+        toks[0] = best;
+        for (int j = 1; j < rows; j++) toks[j] = drafts ? drafts[g - 1 + j] : toks[j - 1];
+        int adv = lg_model_forward_spec_n(&s->m, &s->kv, toks, rows, pos, out);
+        n_steps++;
+        pos += adv;
+        for (int e = 1; e < adv && g < n_gen; e++) emitted[g++] = toks[e];
+        best = out[adv - 1];
+    }
+    if (steps) *steps = n_steps;
+    return g;
+}

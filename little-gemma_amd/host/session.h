@@ -1,0 +1,27 @@
+/* session.h — one loaded model + one KV cache behind plain function calls.
+ *
+ * What the reference's generate() does around the backend seam (src/run.c:711-745: load,
+ * model_init, kvcache_init, prefill, decode) for callers that hold token ids instead of text:
+ * run-hip's command line and the Python tests.  Everything goes through model.h.
+ */
+#ifndef LG_SESSION_H
+#define LG_SESSION_H
+#include "model.h"
+
+struct lg_session;
+struct lg_session *lg_session_open(const char *gguf_path);
+void lg_session_close(struct lg_session *s);
+int  lg_session_kv(struct lg_session *s, int max_seq);              /* (re)creates the cache */
+struct model   *lg_session_model(struct lg_session *s);
+struct kvcache *lg_session_kvcache(struct lg_session *s);
+void lg_session_prefill(struct lg_session *s, const int *tokens, int n, int pos0);
+int  lg_session_forward_next(struct lg_session *s, int token, int pos);
+void lg_session_forward(struct lg_session *s, int token, int pos, float *logits);
+int  lg_session_forward_spec(struct lg_session *s, const int *toks, int rows, int pos, int *out);
+/* Greedy generation of n_gen tokens after `prompt`, plain (rows = 1) or speculative with draft
+ * blocks of `rows` tokens taken from `drafts` (what a draft head would propose for each emitted
+ * position; NULL = repeat the last token, the reference's padding, src/run.c:58-63).
+ * Returns tokens emitted; *steps = target forwards/verify steps run. */
+int  lg_session_generate(struct lg_session *s, const int *prompt, int n_prompt, int n_gen, int rows,
+                         const int *drafts, int *emitted, int *steps);
+#endif
