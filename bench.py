@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""Benchmark of the MTP speculative-verify step on one MI355X.
+
+A "step" is one verify step: a block of M = K+1 rows (the chosen token and K drafts) through the
+whole E4B-shaped q4_0 decoder, lm_head, argmax and the accept rule, all on the device, with the
+position and the token schedule device-resident (no host round trip between steps).  Weights and
+the 2048-position KV cache are in HBM before the timed region.  The drafts are the model's own
+greedy continuation with the first mismatch drawn from a seeded Geometric(0.6), so the number of
+accepted tokens per step is known in advance and is checked.
+
+Prints one JSON line: verified tokens/s, the roofline figure of the dominant kernel (measured with
+device events on the library's stream), the whole-step HBM figure, and the CPU baseline (the
+reference's own CPU backend when its build is present, else this repository's restatement).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+lg = importlib.import_module("little-gemma_amd")
+
+HBM_PEAK_GBS = 8000.0
+CTX = 2048
+WORKLOADS = {
+    "e4b": ("E4B-shape q4_0 verify step (42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144, "
+            "5 sliding-512 : 1 global), ctx 2048", lg.synth.E4B),
+    "tiny": ("tiny 4-layer shape (plumbing check only: fits in cache, no bandwidth claim)", lg.synth.TINY),
+}
+
+
+def log(*a):
+    print("[bench]", *a, file=sys.stderr, flush=True)
+
+
+def seed_cache(gpu, info, layers, ctx, seed):
+    """Fill every owning layer with f16 values shaped like real rows: K ~ N(0, q/k-norm weight),
+    V ~ unit RMS.  Returns {layer: (K, V)} as uint16 arrays indexed by ring row."""
+    rng = np.random.default_rng(seed)
+    filled = {}
+    for L in range(info["n_layer"]):
+        rows, width = gpu.kv_layout(L)
+        if rows == 0:
+            continue
+        hd = layers[L]["head_dim"]
+        kstd = np.sqrt(1.28 / np.sqrt(hd))
+        n = min(rows, ctx)
+        K = np.zeros((rows, width), np.float16)
+        V = np.zeros((rows, width), np.float16)
+        K[:n] = (rng.standard_normal((n, width), np.float32) * kstd).astype(np.float16)
+        V[:n] = rng.standard_normal((n, width), np.float32).astype(np.float16)
+        if rows < ctx:      # ring: row r holds the latest position p < ctx with p % rows == r: any filled row is fine
+            pass
+        gpu.kv_write(L, 0, K.view(np.uint16))
+        gpu.kv_write(L, 1, V.view(np.uint16))
+        filled[L] = (K, V)
+    return filled
+
+
+def build_schedule(greedy, first_tok, rows, n_steps, n_vocab, seed, p=0.6):
+    """Blocks [chosen, d1..dK] along the greedy sequence; first mismatch ~ Geometric(p)."""
+    rng = np.random.default_rng(seed)
+    seq = [first_tok] + list(greedy)          # seq[i] = token at position pos0 + i
+    blocks, advs, at = [], [], 0
+    for _ in range(n_steps):
+        first_bad = int(rng.geometric(p))     # 1-based index of the first wrong draft
+        blk = [seq[at]]
+        for j in range(1, rows):
+            good = seq[at + j]
+            blk.append(good if j < first_bad else (good + 1 + int(rng.integers(0, n_vocab - 1))) % n_vocab)
+        adv = min(first_bad, rows)
+        blocks.append(blk)
+        advs.append(adv)
+        at += adv
+    return np.array(blocks, np.int32), np.array(advs, np.int32)
+
+
+def cpu_baseline(path, filled, info, layers, blocks, pos0, rows, budget_s):
+    from oracle import binding as ob
+    threads = os.cpu_count() or 1
+    threads = min(threads, int(os.environ.get("OMP_NUM_THREADS", threads)))
+    kind = "reference" if ob.ref_available(rows) else "port"
+    if kind == "reference":
+        m = ob.Reference(path, rows)
+        kv = m.kv_new(pos0 + len(blocks) * rows + 8)
+        views = m.kv_views(kv)
+    else:
+        m = ob.Oracle(path)
+        ob.lib().lgo_set_threads(threads)
+        kv = m.kv_new(pos0 + len(blocks) * rows + 8, ob.REF)
+        views = m.kv_views(kv)
+    # same cache contents as the GPU (f16-representable values, so f32 sliding rings hold the same numbers)
+    for L, (K, V) in views.items():
+        gk, gv = filled[L]
+        n_cpu = K.shape[0]
+        for p_ in range(max(0, pos0 - n_cpu), pos0):
+            src = p_ % gk.shape[0]
+            dst = p_ % n_cpu
+            if K.dtype == np.uint16:
+                K[dst] = gk[src].view(np.uint16); V[dst] = gv[src].view(np.uint16)
+            else:
+                K[dst] = gk[src].astype(np.float32); V[dst] = gv[src].astype(np.float32)
+    t0 = time.time()
+    toks_done = steps = 0
+    pos = pos0
+    for blk in blocks:
+        if kind == "reference":
+            adv, _ = m.forward_spec(kv, blk, pos)
+        else:
+            adv, _, _ = m.forward_spec(kv, blk, pos, ob.REF)
+        pos += adv
+        toks_done += adv
+        steps += 1
+        if time.time() - t0 > budget_s:
+            break
+    dt = time.time() - t0
+    m.kv_free(kv)
+    m.close()
+    return {"value": toks_done / dt, "unit": "verified tok/s", "cores": threads, "kind": kind,
+            "sample": f"{steps} verify steps of the same schedule ({toks_done} tokens) on the same GGUF and cache contents, {dt:.1f} s",
+            "ms_per_step": 1e3 * dt / steps}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--rows", type=int, default=5, help="verify rows M = K drafts + 1")
+    ap.add_argument("--workload", default="e4b", choices=sorted(WORKLOADS))
+    ap.add_argument("--model-dir", default=os.environ.get("LG_BENCH_DIR", "/tmp"))
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--seed", type=int, default=7)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU; the verify step is not sharded (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    rank = int(os.environ.get("RANK", "0"))
+    if rank != 0:
+        return
+    desc, spec = WORKLOADS[a.workload]
+    ctx = CTX if a.workload == "e4b" else 256
+    path = os.path.join(a.model_dir, f"lg_bench_{a.workload}_seed{spec['seed']}.gguf")
+    if not os.path.exists(path):
+        t0 = time.time()
+        lg.synth.write_model(path + ".tmp", **spec)
+        os.replace(path + ".tmp", path)
+        log(f"wrote {path} in {time.time() - t0:.1f}s")
+    total = a.steps + a.warmup
+    max_seq = ctx + (total + 2) * a.rows + 64
+    t0 = time.time()
+    gpu = lg.hiplib.HipBackend(path, max_seq, max_rows=max(a.rows, 1))
+    log(f"weights on the device in {time.time() - t0:.1f}s")
+
+    info, layers = gpu.info, gpu.layers
+    filled = seed_cache(gpu, info, layers, ctx, a.seed)
+    H = gpu.H
+    lg.hiplib.hip_check(H.lg_hip_kv_save_prefix(gpu.dkv, ctx), "kv_save_prefix")
+
+    # the model's own greedy continuation from the seeded cache (plain one-row decode)
+    first_tok = 1 + a.seed % (info["n_vocab"] - 1)
+    need = total * a.rows + a.rows + 1
+    t0 = time.time()
+    greedy, tok, pos = [], first_tok, ctx
+    for _ in range(need):
+        tok = gpu.forward_next(tok, pos)
+        greedy.append(tok)
+        pos += 1
+    decode_ms = 1e3 * (time.time() - t0) / need
+    log(f"plain decode: {need} tokens, {decode_ms:.3f} ms/token (host-synchronised)")
+    blocks, expect_adv = build_schedule(greedy, first_tok, a.rows, total, info["n_vocab"], a.seed)
+
+    # timed region: warm-up steps, then exactly --steps steps, device events on the library's stream
+    lg.hiplib.hip_check(H.lg_hip_kv_restore_prefix(gpu.dkv, ctx), "kv_restore_prefix")
+    gpu.schedule(blocks, ctx)
+    if a.warmup:
+        gpu.schedule_time(a.warmup)
+    wall0 = time.time()
+    ms = gpu.schedule_time(a.steps)
+    wall = time.time() - wall0
+    out, adv, final_pos = gpu.schedule_wait()
+    ok_adv = bool(np.array_equal(adv, expect_adv))
+    # greedy successors must reproduce the plain-decode sequence wherever they are valid
+    seq = [first_tok] + greedy
+    at, ok_tok = 0, True
+    for s in range(total):
+        for j in range(int(adv[s])):
+            ok_tok &= int(out[s, j]) == seq[at + j + 1]
+        at += int(adv[s])
+    timed_tokens = int(adv[a.warmup:].sum())
+    value = timed_tokens / (ms * 1e-3)
+
+    # per-kernel-class device time of one step (un-captured, event pair per launch)
+    prof = gpu.profile_step(blocks[0], ctx, repeats=3)
+    step_bytes = sum(c["bytes"] for c in prof)
+    dom = max((c for c in prof if c["bytes"] > 0), key=lambda c: c["ms"])
+    dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": dom_gbs / HBM_PEAK_GBS, "traffic": None,
+                "bytes_per_launch": dom["bytes"] / max(dom["launches"], 1), "ms_per_launch": dom["ms"] / max(dom["launches"], 1),
+                "launches_per_step": dom["launches"]}
+    step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9
+    line = {
+        "metric": "verified tok/s (E4B-shape q4_0, block-4, ctx 2048) + achieved HBM GB/s vs peak",
+        "value": value, "unit": "verified tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms / a.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 x int4 -> int32 block dots, f32 accumulate", "data": "synthetic",
+        "config": {"workload": desc, "verify_rows": a.rows, "drafts": a.rows - 1, "ctx": ctx,
+                   "mean_accepted_per_step": float(adv[a.warmup:].mean()), "first_mismatch": "Geometric(0.6), seeded"},
+        "roofline": roofline,
+        "step_hbm": {"bytes_per_step": step_bytes, "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": step_gbs / HBM_PEAK_GBS},
+        "kernel_classes": [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in c.items()} for c in prof],
+        "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
+                   "wall_ms_per_step": 1e3 * wall / a.steps, "plain_decode_ms_per_token_host_sync": decode_ms},
+    }
+    gpu.close()
+    if a.cpu_seconds > 0:
+        try:
+            line["cpu_baseline"] = cpu_baseline(path, filled, info, layers, blocks, ctx, a.rows, a.cpu_seconds)
+        except Exception as e:              # the baseline is reported, never allowed to break the GPU line
+            line["cpu_baseline"] = {"value": None, "error": repr(e)}
+    print(json.dumps(line), flush=True)
+    if not (ok_adv and ok_tok):
+        log("CHECK FAILED: verify output differs from plain decode / schedule")
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -16,6 +16,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HOST = os.path.join(HERE, "host")
 MAX_ROWS = 8
+INFO_KEYS = ("n_layer", "n_embd", "n_head", "n_vocab", "ple", "n_kv_start", "window", "n_ff", "n_head_kv",
+             "head_dim_swa", "head_dim_full", "n_ctx")
 
 f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
 i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
@@ -105,6 +107,8 @@ def load_backend():
     B.lg_session_model.restype = C.c_void_p
     B.lg_session_kvcache.argtypes = [C.c_void_p]
     B.lg_session_kvcache.restype = C.c_void_p
+    B.lg_session_info.argtypes = [C.c_void_p, i32p, C.c_int]
+    B.lg_session_layer.argtypes = [C.c_void_p, C.c_int, i32p]
     B.lg_session_prefill.argtypes = [C.c_void_p, i32p, C.c_int, C.c_int]
     B.lg_session_forward_next.argtypes = [C.c_void_p, C.c_int, C.c_int]
     B.lg_session_forward.argtypes = [C.c_void_p, C.c_int, C.c_int, f32p]
@@ -135,6 +139,14 @@ class HipBackend:
         if self.B.lg_session_kv(self.s, max_seq) != 0:
             raise HipError("kvcache_init failed")
         self.max_seq = max_seq
+        v = np.zeros(16, np.int32)
+        n = self.B.lg_session_info(self.s, v, 16)
+        self.info = dict(zip(INFO_KEYS, (int(x) for x in v[:n])))
+        self.layers = []
+        for i in range(self.info["n_layer"]):
+            o = np.zeros(4, np.int32)
+            self.B.lg_session_layer(self.s, i, o)
+            self.layers.append(dict(is_local=int(o[0]), head_dim=int(o[1]), n_head_kv=int(o[2]), ffn_len=int(o[3])))
         self.model = self.B.lg_session_model(self.s)
         self.dev = self.B.lg_model_device(self.model)
         self.dkv = self.B.lg_model_device_kv(self.B.lg_session_kvcache(self.s))

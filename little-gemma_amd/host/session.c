@@ -29,6 +29,19 @@ int lg_session_kv(struct lg_session *s, int max_seq) {
 }
 struct model   *lg_session_model(struct lg_session *s) { return &s->m; }
 struct kvcache *lg_session_kvcache(struct lg_session *s) { return s->has_kv ? &s->kv : NULL; }
+int lg_session_info(struct lg_session *s, int *out, int cap) {
+    const struct config *c = &s->m.cfg;
+    const int v[] = { c->n_layer, c->n_embd, c->n_head, c->n_vocab, c->n_embd_per_layer, c->n_kv_start,
+                      c->sliding_window, c->n_ff, c->n_head_kv, c->head_dim_swa, c->head_dim_full, c->n_ctx };
+    const int n = (int)(sizeof v / sizeof v[0]);
+    for (int i = 0; i < n && i < cap; i++) out[i] = v[i];
+    return n;
+}
+int lg_session_layer(struct lg_session *s, int L, int *out4) {
+    if (L < 0 || L >= s->m.cfg.n_layer) return -1;
+    out4[0] = s->m.is_local[L]; out4[1] = s->m.head_dim[L]; out4[2] = s->m.n_head_kv[L]; out4[3] = s->m.ffn_len[L];
+    return 0;
+}
 void lg_session_prefill(struct lg_session *s, const int *t, int n, int pos0) { model_prefill(&s->m, &s->kv, t, n, pos0); }
 int  lg_session_forward_next(struct lg_session *s, int token, int pos) { return model_forward_next(&s->m, &s->kv, token, pos); }
 void lg_session_forward(struct lg_session *s, int token, int pos, float *logits) { model_forward(&s->m, &s->kv, token, pos, logits); }

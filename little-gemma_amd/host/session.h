@@ -14,6 +14,10 @@ void lg_session_close(struct lg_session *s);
 int  lg_session_kv(struct lg_session *s, int max_seq);              /* (re)creates the cache */
 struct model   *lg_session_model(struct lg_session *s);
 struct kvcache *lg_session_kvcache(struct lg_session *s);
+/* n_layer, n_embd, n_head, n_vocab, ple, n_kv_start, window, n_ff, n_head_kv, head_dim_swa, head_dim_full, n_ctx */
+int  lg_session_info(struct lg_session *s, int *out, int cap);
+/* is_local, head_dim, n_head_kv, ffn_len of layer L */
+int  lg_session_layer(struct lg_session *s, int L, int *out4);
 void lg_session_prefill(struct lg_session *s, const int *tokens, int n, int pos0);
 int  lg_session_forward_next(struct lg_session *s, int token, int pos);
 void lg_session_forward(struct lg_session *s, int token, int pos, float *logits);

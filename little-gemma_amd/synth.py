@@ -20,7 +20,7 @@ DEFAULTS = dict(head_dim_full=0, n_ctx=8192, sliding_window=512, local_period=6,
 
 # 4 layers, d 512, 8 x 64 heads, 2 KV heads, FFN 2048, vocab 8192, sliding-128 / global alternating
 TINY = dict(DEFAULTS, n_layer=4, n_embd=512, n_head=8, n_head_kv=2, head_dim=64, n_ff=2048, n_vocab=8192,
-            sliding_window=128, local_period=2)
+            sliding_window=128, local_period=2, qk_norm=0.7)
 # the same with every optional piece switched on: PLE, shared-KV tail, V-less layers, output scale
 TINY_FULL = dict(TINY, n_layer=6, ple=256, shared_kv_layers=2, has_v=0, out_scale=0.9, head_dim_full=128)
 # E4B shape: 42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144; 5 sliding(512) : 1 global

@@ -1,0 +1,158 @@
+"""GPU parity of the parts, through the C ABI: the isolated q4_0 x q8 matmul (BASELINE config 2)
+and the decode attention over an f16 ring (config 3).  Bar: int32 block dots and every integer
+bit-exact; f32 outputs bit-identical to the oracle in this build's summation order and within
+1e-5 relative of float64."""
+import numpy as np
+import pytest
+
+from conftest import q4_0_codes, quant_q8_numpy, random_q4_0
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_matmul(ob, w, k, m, x):
+    L = ob.lib()
+    rows, nb = x.shape[0], k // 32
+    xq = np.zeros((rows, k), np.int8); xd = np.zeros((rows, nb), np.float32); xs = np.zeros((rows, nb), np.int32)
+    for j in range(rows):
+        L.lgo_quant_q8(x[j], k, xq[j], xd[j], xs[j])
+    out = np.zeros((rows, m), np.float32); dots = np.zeros((rows, m, nb), np.int32)
+    L.lgo_matmul_q4q8(w, k, m, xq, xd, rows, out, dots.ctypes.data, ob.ORDER_SEG8)
+    return xq, xd, xs, out, dots
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 5])
+def test_matmul_config2_full_size(lg, ob, gpu_required, rows):
+    """W 10240 x 2560 q4_0 (f16 scales ~N(0,0.01), codes uniform), X ~ N(0,1), M in {1,2,4,5}."""
+    m, k = 10240, 2560
+    rng = np.random.default_rng(100 + rows)
+    w = random_q4_0(rng, m, k)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    print(f"matmul m={m} k={k} rows={rows}", flush=True)
+    r = lg.hiplib.matmul_q4q8(w, k, m, x, want_dots=True)
+    xq, xd, xs, out, dots = oracle_matmul(ob, w, k, m, x)
+    nq, nd, ns = quant_q8_numpy(x)
+    assert np.array_equal(r["xq"], nq.reshape(rows, k)) and np.array_equal(r["xq"], xq)
+    assert np.array_equal(r["xd"].view(np.uint32), nd.reshape(rows, -1).view(np.uint32))
+    assert np.array_equal(r["xsum"], ns.reshape(rows, -1)) and np.array_equal(r["xsum"], xs)
+    # int32 block dots: bit-exact against the closed form sum((nibble-8)*q), all 10240*80*rows of them
+    dw, codes = q4_0_codes(w, m, k)
+    want_dots = np.einsum("ibe,jbe->jib", codes - 8, xq.reshape(rows, k // 32, 32).astype(np.int32))
+    assert np.array_equal(r["dots"], want_dots) and np.array_equal(r["dots"], dots)
+    # f32: bit-identical to the oracle's order, 1e-5 relative against float64
+    assert np.array_equal(r["out"].view(np.uint32), out.view(np.uint32))
+    want = np.einsum("jib,ib,jb->ji", want_dots.astype(np.float64), dw.astype(np.float64), xd.astype(np.float64))
+    assert np.abs(r["out"] - want).max() <= 1e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("m,k,rows", [(8, 256, 1), (2560, 10240, 5), (2048, 256, 8), (512, 3840, 3), (264, 15360, 8)])
+def test_matmul_edge_shapes(lg, ob, gpu_required, m, k, rows):
+    rng = np.random.default_rng(m + k)
+    w = random_q4_0(rng, m, k)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[0, :64] = 0.0                                      # zero groups: scale 0, no NaN
+    x[rows - 1, 32:64] = 1e-30
+    print(f"matmul m={m} k={k} rows={rows}", flush=True)
+    r = lg.hiplib.matmul_q4q8(w, k, m, x, want_dots=True)
+    xq, xd, xs, out, dots = oracle_matmul(ob, w, k, m, x)
+    assert np.array_equal(r["xq"], xq) and np.array_equal(r["xsum"], xs) and np.array_equal(r["dots"], dots)
+    assert np.array_equal(r["out"].view(np.uint32), out.view(np.uint32))
+    assert np.all(np.isfinite(r["out"]))
+
+
+def test_matmul_is_linear_in_the_scales(lg, gpu_required):
+    """Size-independent property: doubling every weight scale doubles every output exactly
+    (powers of two commute with rounding), negating codes around 8 negates it."""
+    m, k, rows = 512, 2560, 5
+    rng = np.random.default_rng(9)
+    w = random_q4_0(rng, m, k).reshape(m, k // 32, 18)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    base = lg.hiplib.matmul_q4q8(w.reshape(-1), k, m, x)["out"]
+    w2 = w.copy()
+    d = w2[:, :, :2].copy().view(np.float16)
+    w2[:, :, :2] = (d * np.float16(2)).view(np.uint8)
+    assert np.array_equal(lg.hiplib.matmul_q4q8(w2.reshape(-1), k, m, x)["out"], base * 2)
+    x2 = lg.hiplib.matmul_q4q8(w.reshape(-1), k, m, -x)["out"]
+    assert np.array_equal(x2, -base)
+
+
+def attention_f64(q, kc, vc, H, KV, hd, window, pos):
+    rows, seq = q.shape[0], kc.shape[0]
+    K = kc.view(np.float16).astype(np.float64).reshape(seq, KV, hd)
+    V = vc.view(np.float16).astype(np.float64).reshape(seq, KV, hd)
+    out = np.zeros((rows, H, hd))
+    for j in range(rows):
+        pj = pos + j
+        start = max(0, pj - window + 1) if window else 0
+        idx = [t % seq for t in range(start, pj + 1)]
+        for h in range(H):
+            kvh = h // (H // KV)
+            s = K[idx, kvh] @ q[j, h * hd:(h + 1) * hd].astype(np.float64)
+            p = np.exp(s - s.max()); p /= p.sum()
+            out[j, h] = p @ V[idx, kvh]
+    return out.reshape(rows, H * hd)
+
+
+def oracle_attention(ob, q, kc, vc, H, KV, hd, window, pos):
+    L = ob.lib()
+    rows, seq, kd = q.shape[0], kc.shape[0], KV * hd
+    out = np.zeros_like(q)
+    for j in range(rows):
+        pj = pos + j
+        start = max(0, pj - window + 1) if window else 0
+        for h in range(H):
+            o = np.zeros(hd, np.float32)
+            L.lgo_attention_f16(o, np.ascontiguousarray(q[j, h * hd:(h + 1) * hd]), kc.reshape(-1), vc.reshape(-1),
+                                hd, kd, h // (H // KV), seq, start, pj, 1, 1)
+            out[j, h * hd:(h + 1) * hd] = o
+    return out
+
+
+@pytest.mark.parametrize("seq,window,pos", [(4096 + 8, 0, 4091), (544, 512, 4091), (544, 512, 300), (4104, 0, 0), (160, 128, 31)])
+def test_attention_config3(lg, ob, gpu_required, seq, window, pos):
+    """8 query heads, 2 KV heads, head_dim 256, N(0,1) f16 K/V, 5 draft rows, causal among themselves:
+    context 4096 global, and the 512-window ring variant (plus a short context and position 0)."""
+    H, KV, hd, rows = 8, 2, 256, 5
+    rng = np.random.default_rng(seq + pos)
+    kc = rng.normal(0, 1, (seq, KV * hd)).astype(np.float16).view(np.uint16)
+    vc = rng.normal(0, 1, (seq, KV * hd)).astype(np.float16).view(np.uint16)
+    q = (rng.normal(0, 1, (rows, H * hd)) * 0.08).astype(np.float32)       # score std ~1.3, like a normed q.k
+    print(f"attention seq={seq} window={window} pos={pos}", flush=True)
+    out, _ = lg.hiplib.attention(q, kc, vc, H, KV, hd, window, pos)
+    want = oracle_attention(ob, q, kc, vc, H, KV, hd, window, pos)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    f64 = attention_f64(q, kc, vc, H, KV, hd, window, pos)
+    assert np.abs(out - f64).max() <= 1e-5 * max(1.0, np.abs(f64).max())
+    # causal mask among the draft rows: row j must not see rows > j.  Change the K/V of the last
+    # row's position and every earlier row's output stays bit-identical.
+    k2, v2 = kc.copy(), vc.copy()
+    last = (pos + rows - 1) % seq
+    k2[last] = rng.normal(0, 1, KV * hd).astype(np.float16).view(np.uint16)
+    v2[last] = rng.normal(0, 1, KV * hd).astype(np.float16).view(np.uint16)
+    out2, _ = lg.hiplib.attention(q, k2, v2, H, KV, hd, window, pos)
+    assert np.array_equal(out2[: rows - 1].view(np.uint32), out[: rows - 1].view(np.uint32))
+    assert not np.array_equal(out2[rows - 1], out[rows - 1])
+
+
+@pytest.mark.parametrize("H,KV,hd,rows", [(8, 2, 64, 8), (16, 8, 256, 4), (4, 4, 128, 1), (8, 2, 512, 2), (8, 8, 256, 5)])
+def test_attention_other_geometries(lg, ob, gpu_required, H, KV, hd, rows):
+    rng = np.random.default_rng(H * hd + rows)
+    seq, window, pos = 288, 256, 700
+    kc = rng.normal(0, 1, (seq, KV * hd)).astype(np.float16).view(np.uint16)
+    vc = rng.normal(0, 1, (seq, KV * hd)).astype(np.float16).view(np.uint16)
+    q = (rng.normal(0, 1, (rows, H * hd)) * 0.1).astype(np.float32)
+    print(f"attention H={H} KV={KV} hd={hd} rows={rows}", flush=True)
+    out, _ = lg.hiplib.attention(q, kc, vc, H, KV, hd, window, pos)
+    want = oracle_attention(ob, q, kc, vc, H, KV, hd, window, pos)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+
+
+def test_bad_arguments_are_refused(lg, gpu_required):
+    rng = np.random.default_rng(1)
+    with pytest.raises(lg.hiplib.HipError):
+        lg.hiplib.matmul_q4q8(random_q4_0(rng, 8, 256), 256, 8, np.zeros((9, 256), np.float32))      # 9 rows
+    with pytest.raises(lg.hiplib.HipError):
+        lg.hiplib.matmul_q4q8(np.zeros(12 * 18 * 8, np.uint8), 256, 12, np.zeros((1, 256), np.float32))   # rows % 8
+    with pytest.raises(lg.hiplib.HipError):
+        lg.hiplib.attention(np.zeros((2, 8 * 256), np.float32), np.zeros((64, 512), np.uint16), np.zeros((64, 512), np.uint16),
+                            8, 2, 256, 0, 100)                                                        # cache too short
