@@ -133,6 +133,7 @@ int  lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, in
                       int repeats, float *kernel_ms);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
+int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 */
 size_t lg_hip_repacked_bytes(int k, int m);
 int    lg_hip_repack_q4_0(const void *src, int k, int m, void *dst);
 

@@ -5,8 +5,9 @@
 // from include/lg_math.h.  Integer work (q8 quantization, q4_0 x q8 block dots) is exact.
 //   * row sum of squares: 64 lane partials, element i belongs to lane (i/4)%64, fma in
 //     ascending i, then an adjacent-pair binary tree over the lanes;
-//   * q4_0 x q8 matmul: 8 contiguous K segments per output, one lane each, serial fma over
-//     the segment's blocks, adjacent-pair tree over the 8 lanes;
+//   * q4_0 x q8 matmul: S contiguous K segments per output (S = 8, or 32 for rows of more than
+//     128 blocks), one lane each, serial fma over the segment's blocks, adjacent-pair tree over
+//     the S lanes;
 //   * attention: 32-key tiles aligned to absolute positions (see lg_kernels.h).
 #pragma once
 
@@ -22,10 +23,12 @@
 #define LG_MAXV      16       // float4 per lane of a residual row: n_embd <= 4096
 #define LG_HIP_MAX_ROWS_DEV 8   // widest draft block (same value as LG_HIP_MAX_ROWS in lg_hip.h)
 
-// Weight tile order (built on the host by lg_hip_repack_q4_0): an m x k q4_0 matrix is cut into
-// groups of 8 rows; row r of a group is cut into 8 segments of nit = k/256 blocks; tile (group,
-// it) holds, for lane = r*8 + c, the 16 nibble bytes and the f16 scale of block c*nit + it of
-// row r.  A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
+// Weight tile order (built on the host by lg_hip_repack_q4_0): a row of k/32 q4_0 blocks is cut
+// into S contiguous segments of nit blocks (S = lg_segments(k): 8, or 32 for rows of more than 128
+// blocks); the m x k matrix is cut into groups of 64/S rows; tile (group, it) holds, for
+// lane = r*S + c, the 16 nibble bytes and the f16 scale of block c*nit + it of row r of the group.
+// A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
+__host__ __device__ static inline int lg_segments(int k) { return (k >> 5) > 128 ? 32 : 8; }
 
 __device__ __forceinline__ float lg_wave_sum64(float v) {
     v = v + __shfl_xor(v, 1);
@@ -101,11 +104,11 @@ __device__ __forceinline__ uint16_t lg_f2h(float f) {
 }
 
 // Four consecutive elements (e0 % 4 == 0) of row `row` of a tiled q4_0 matrix, dequantized.
-__device__ __forceinline__ float4 lg_tiled_deq4(const uint8_t *w, int nit, int row, int e0) {
-    const int b = e0 >> 5, o = e0 & 31;
+__device__ __forceinline__ float4 lg_tiled_deq4(const uint8_t *w, int nit, int S, int row, int e0) {
+    const int b = e0 >> 5, o = e0 & 31, rw = 64 / S;
     const int c = b / nit, it = b - c * nit;
-    const uint8_t *tile = w + ((size_t)(row >> 3) * nit + it) * LG_TILE;
-    const int slot = (row & 7) * 8 + c;
+    const uint8_t *tile = w + ((size_t)(row / rw) * nit + it) * LG_TILE;
+    const int slot = (row % rw) * S + c;
     const uint32_t qs = *(const uint32_t *)(tile + slot * 16 + (o & 15));
     const float d = lg_h2f(*(const uint16_t *)(tile + 1024 + slot * 2));
     const uint32_t nib = (o & 16) ? (qs >> 4) : qs;
@@ -128,8 +131,7 @@ __device__ __forceinline__ float lg_q4_0_elem(const uint8_t *row, int e) {
 
 // Inner product of one weight tile lane (16 nibble bytes = one q4_0 block) with the 32 int8 of
 // an activation block: sum(c*q) - 8*sum(q) == sum((c-8)*q), exact in int32.
-__device__ __forceinline__ int lg_block_dot(uint4 wq, const int8_t *act32, int act_sum) {
-    const int4 a0 = *(const int4 *)act32, a1 = *(const int4 *)(act32 + 16);
+__device__ __forceinline__ int lg_block_dot(uint4 wq, int4 a0, int4 a1, int act_sum) {
     int dot = 0;
     dot = __builtin_amdgcn_sdot4((int)(wq.x & 0x0F0F0F0Fu), a0.x, dot, false);
     dot = __builtin_amdgcn_sdot4((int)(wq.y & 0x0F0F0F0Fu), a0.y, dot, false);

@@ -42,23 +42,27 @@ extern "C" int lg_hip_ring_rows(int window, int max_seq) {
 }
 
 // ---- weight layout ----------------------------------------------------------------------------
+extern "C" int lg_hip_segments(int k) { return lg_segments(k); }
+
 extern "C" size_t lg_hip_repacked_bytes(int k, int m) {
     if (k <= 0 || m <= 0 || k % 256 || m % 8) return 0;
-    return (size_t)(m / 8) * (size_t)(k / 256) * LG_TILE;
+    const int S = lg_segments(k);
+    if ((k / 32) % S) return 0;
+    return (size_t)(m / (64 / S)) * (size_t)(k / 32 / S) * LG_TILE;
 }
 
 // rows[i] points at virtual row i (k/32 blocks of 18 bytes each)
 static void repack_rows(const uint8_t *const *rows, int k, int m, uint8_t *dst) {
-    const int nit = k / 256, groups = m / 8;
+    const int S = lg_segments(k), rw = 64 / S, nit = k / 32 / S, groups = m / rw;
     auto work = [&](int g0, int g1) {
         for (int g = g0; g < g1; ++g)
             for (int it = 0; it < nit; ++it) {
                 uint8_t *tile = dst + ((size_t)g * nit + it) * LG_TILE;
-                for (int r = 0; r < 8; ++r)
-                    for (int c = 0; c < 8; ++c) {
-                        const uint8_t *blk = rows[g * 8 + r] + (size_t)(c * nit + it) * 18;
-                        memcpy(tile + (r * 8 + c) * 16, blk + 2, 16);
-                        memcpy(tile + 1024 + (r * 8 + c) * 2, blk, 2);
+                for (int r = 0; r < rw; ++r)
+                    for (int c = 0; c < S; ++c) {
+                        const uint8_t *blk = rows[g * rw + r] + (size_t)(c * nit + it) * 18;
+                        memcpy(tile + (r * S + c) * 16, blk + 2, 16);
+                        memcpy(tile + 1024 + (r * S + c) * 2, blk, 2);
                     }
             }
     };
@@ -71,7 +75,7 @@ static void repack_rows(const uint8_t *const *rows, int k, int m, uint8_t *dst) 
 }
 
 extern "C" int lg_hip_repack_q4_0(const void *src, int k, int m, void *dst) {
-    if (!lg_hip_repacked_bytes(k, m)) return fail(-2, "repack: k=%d must be a multiple of 256 and m=%d of 8", k, m);
+    if (!lg_hip_repacked_bytes(k, m)) return fail(-2, "repack: k=%d must be a multiple of 256 (1024 above 4096) and m=%d of 8", k, m);
     std::vector<const uint8_t *> rows((size_t)m);
     for (int i = 0; i < m; ++i) rows[i] = (const uint8_t *)src + (size_t)i * (k / 32) * 18;
     repack_rows(rows.data(), k, m, (uint8_t *)dst);
@@ -89,10 +93,10 @@ struct Layer {
     const float *rope_tab = nullptr, *rope_ff = nullptr;
 };
 
-enum KClass { KC_PMP, KC_QKV, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
-              KC_FINALNORM, KC_HEAD, KC_ACCEPT, KC_COUNT };
-static const char *k_class_names[KC_COUNT] = { "ple_model_proj", "qkv", "attn_tiles", "attn_merge", "attn_output",
-    "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "final_norm", "lm_head", "accept" };
+enum KClass { KC_ROWS, KC_PMP, KC_QKV, KC_QKVPOST, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
+              KC_HEAD, KC_ACCEPT, KC_COUNT };
+static const char *k_class_names[KC_COUNT] = { "rows_norm_quant", "ple_model_proj", "qkv", "qkv_post", "attn_tiles", "attn_merge",
+    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept" };
 
 struct Profile {
     bool on = false;
@@ -118,7 +122,7 @@ struct lg_hip_model {
     size_t weight_bytes = 0;
     // scratch
     float *x[2] = { nullptr, nullptr }, *qkv = nullptr, *dout = nullptr, *pmp_raw = nullptr, *hidden_rows = nullptr,
-          *g_hidden = nullptr, *logits = nullptr, *pval = nullptr;
+          *g_hidden = nullptr, *logits = nullptr, *pval = nullptr, *q_rot = nullptr;
     int8_t *aq = nullptr, *gq = nullptr, *pq = nullptr, *hq = nullptr;
     float2 *ads = nullptr, *gds = nullptr, *pds = nullptr, *hds = nullptr;
     int *pidx = nullptr;
@@ -364,7 +368,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     m->host.clear();
     const size_t R = (size_t)max_rows;
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
-        dev_alloc(m, &m->dout, R * E) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
+        dev_alloc(m, &m->dout, R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
         dev_alloc(m, &m->aq, R * max_qd) || dev_alloc(m, &m->ads, R * max_qd / 32) ||
         dev_alloc(m, &m->gq, R * max_ff) || dev_alloc(m, &m->gds, R * max_ff / 32) ||
         dev_alloc(m, &m->hq, R * E) || dev_alloc(m, &m->hds, R * E / 32) ||
@@ -546,8 +550,26 @@ struct Launcher {
     }
 };
 
-#define LAUNCH(cls, kernel, grid, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { lx.begin(cls); \
-    hipLaunchKernelGGL(kernel, grid, dim3(LG_WG), lds, m->stream, __VA_ARGS__); lx.end(); } } while (0)
+#define LAUNCH(cls, kernel, grid, block, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { lx.begin(cls); \
+    hipLaunchKernelGGL(kernel, grid, block, lds, lx.m->stream, __VA_ARGS__); lx.end(); } } while (0)
+
+// Plain matmul launch: picks the segment count from k and the workgroup shape from the row count
+// (small matrices get one wavefront per workgroup so that every CU has work).
+template <int M, bool DUMP>
+static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
+    const int S = lg_segments(a.k), rw = 64 / S, ngroups = a.m / rw;
+    const size_t lds = lds_mm(M, a.k);
+    if (S == 32) {
+        const int W = 4;
+        LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
+    } else if (ngroups >= 4096) {
+        const int W = 4;
+        LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
+    } else {
+        const int W = ngroups >= 1024 ? 2 : 1;
+        LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
+    }
+}
 
 // one block of M rows through the decoder (and the head when with_head)
 template <int M>
@@ -555,91 +577,90 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     Launcher lx{ m, dry };
     const int E = m->E, H = m->H, nl = m->n_layer;
     int cur = 0;                                   // x[cur] holds the residual
-    ActSrc base{};
-    base.E = E; base.eps = m->eps; base.toks = m->sched;
     bool have_x = false;                           // false: rows are still token ids
     const float *pend_dout = nullptr, *pend_w = nullptr, *pend_os = nullptr;   // sub-layer output waiting to be added
 
-    auto src_for = [&](const float *w_pre, bool write_x) {
-        ActSrc s = base;
-        if (!have_x) { s.emb = m->emb; s.emb_nit = E / 256; s.emb_scale = sqrtf((float)E); }
+    // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
+    auto rows = [&](const float *w_pre, float *h_out) {
+        RowArgs s{};
+        s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq; s.ds = m->hds;
+        if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os;
-        s.w_pre = w_pre;
-        if (write_x && (pend_dout || !have_x)) { s.x_out = m->x[cur ^ 1]; }
-        return s;
-    };
-    auto consumed = [&](const ActSrc &s) {         // after a prologue that wrote x_out
+        s.w_pre = w_pre; s.h_out = h_out;
+        if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
+        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M), dim3(64), 0, s, m->ctl);
         if (s.x_out) cur ^= 1;
         have_x = true; pend_dout = pend_w = pend_os = nullptr;
     };
 
     if (m->ple) {
-        ActSrc s = src_for(nullptr, true);
-        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, nullptr, nullptr, nullptr };
-        LAUNCH(KC_PMP, (lg_k_mm<M, SRC_ACT, false>), dim3((a.m / 8 + 3) / 4), lds_mm(M, E), a, s, m->ctl);
-        consumed(s);
+        rows(nullptr, nullptr);
+        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, m->hds, nullptr };
+        launch_mm<M, false>(lx, KC_PMP, a);
     }
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
-        {   // q/k/v projections on rmsnorm(x) * attn_norm
-            ActSrc s = src_for(y.attn_norm, true);
-            MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, nullptr, nullptr, nullptr };
-            LAUNCH(KC_QKV, (lg_k_mm<M, SRC_ACT, false>), dim3((a.m / 8 + 3) / 4), lds_mm(M, E), a, s, m->ctl);
-            consumed(s);
+        const int window = (y.is_local && m->window > 0) ? m->window : 0;
+        rows(y.attn_norm, nullptr);
+        {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
+            MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, m->hds, nullptr };
+            launch_mm<M, false>(lx, KC_QKV, a);
+            QkvPostArgs p{};
+            p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
+            p.H = H; p.nkv = y.nkv; p.hd = y.hd;
+            p.q_norm = y.q_norm; p.k_norm = y.k_norm; p.rope_tab = y.rope_tab; p.rope_ff = y.rope_ff;
+            p.q_rot = m->q_rot;
+            p.kc = y.owns ? kv->k[L] : nullptr; p.vc = y.owns ? kv->v[L] : nullptr;
+            p.seq = kv->seq[y.src]; p.kv_dim = y.kd; p.eps = m->eps;
+            LAUNCH(KC_QKVPOST, lg_k_qkv_post, dim3(H + (y.owns ? 2 * y.nkv : 0), M), dim3(64), 0, p, m->ctl);
         }
         {   // attention tiles + merge
             const int G = H / y.nkv, nq = G * M, kst = y.hd + 8;
             AttnArgs a{};
-            a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
-            a.H = H; a.nkv = y.nkv; a.hd = y.hd;
-            a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
-            a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd;
-            a.window = (y.is_local && m->window > 0) ? m->window : 0;
-            a.owns = y.owns; a.prerotated = 0; a.eps = m->eps;
+            a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
+            a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max;
-            const size_t lds = (size_t)(nq + M) * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
-            LAUNCH(KC_ATTN, (lg_k_attn<M>), dim3(kv->tiles_max, y.nkv), lds, a, m->ctl);
-            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, a.window, m->aq, m->ads, nullptr };
-            LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), 0, g, m->ctl);
+            const size_t lds = (size_t)nq * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
+            LAUNCH(KC_ATTN, (lg_k_attn<M>), dim3(kv->tiles_max, y.nkv), dim3(LG_WG), lds, a, m->ctl);
+            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, m->aq, m->ads, nullptr };
+            LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
         {   // attention output projection
             MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, m->ads, nullptr };
-            LAUNCH(KC_O, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, y.qd), a, base, m->ctl);
+            launch_mm<M, false>(lx, KC_O, a);
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
         }
         {   // feed-forward: gate/up + GeGLU, then down
-            ActSrc s = src_for(y.ffn_norm, true);
-            GegluArgs a{ y.wgu, E, y.nff, m->gq, m->gds };
-            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M>), dim3(y.nff / 32), lds_mm(M, E), a, s, m->ctl);
-            consumed(s);
+            rows(y.ffn_norm, nullptr);
+            GegluArgs a{ y.wgu, E, y.nff, m->hq, m->hds, m->gq, m->gds };
+            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M>), dim3(y.nff / 32), dim3(LG_WG), lds_mm(M, E), a);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, m->gds, nullptr };
-            LAUNCH(KC_DOWN, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, y.nff), d, base, m->ctl);
+            launch_mm<M, false>(lx, KC_DOWN, d);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
         }
         if (m->ple) {   // per-layer embedding block
-            ActSrc s = src_for(nullptr, true);
+            rows(nullptr, nullptr);
             PleGateArgs a{};
-            a.w = y.winp; a.k = E; a.ple = m->ple; a.pmp_raw = m->pmp_raw; a.layer = L; a.n_layer = nl;
+            a.w = y.winp; a.k = E; a.ple = m->ple; a.q_in = m->hq; a.ds_in = m->hds;
+            a.pmp_raw = m->pmp_raw; a.layer = L; a.n_layer = nl;
             a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
             a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
             a.pq = m->pq; a.pds = m->pds;
-            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), lds_mm(M, E) + (size_t)M * m->ple * 4, a, s, m->ctl);
-            consumed(s);
+            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E) + (size_t)M * 32 * 4, a, m->ctl);
             MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, m->pds, nullptr };
-            LAUNCH(KC_PLEPROJ, (lg_k_mm<M, SRC_Q8, false>), dim3((E / 8 + 3) / 4), lds_mm(M, m->ple), p, base, m->ctl);
+            launch_mm<M, false>(lx, KC_PLEPROJ, p);
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
         }
     }
     if (with_head && !lx.rc) {
-        ActSrc s = src_for(m->output_norm, false);
-        s.h_out = m->hidden_rows;
-        QuantArgs q{ m->hq, m->hds };
-        LAUNCH(KC_FINALNORM, (lg_k_act_quant<M>), dim3(1), 0, q, s, m->ctl);
-        HeadArgs h{ m->emb, E, m->n_vocab, m->hq, m->hds, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
-        LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(m->n_vocab / 32), lds_mm(M, E), h);
-        AcceptArgs c{ m->pval, m->pidx, m->n_vocab / 32, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
-        LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), 0, c, m->ctl);
+        rows(m->output_norm, m->hidden_rows);
+        const int passes = 4;
+        const int grid = (m->n_vocab / 8 + passes * 8 - 1) / (passes * 8);
+        HeadArgs h{ m->emb, E, m->n_vocab, passes, m->hq, m->hds, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
+        LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(grid), dim3(LG_WG), lds_mm(M, E), h);
+        AcceptArgs c{ m->pval, m->pidx, grid, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
+        LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), dim3(LG_WG), 0, c, m->ctl);
     } else if (!lx.rc && !dry) {
         hipLaunchKernelGGL(lg_k_advance, dim3(1), dim3(1), 0, m->stream, m->ctl, M);
     }
@@ -834,6 +855,7 @@ static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int
         b[KC_ATTN] += 2.0 * (last - start + 1) * y.kd * 2.0;          // K and V rows, f16
     }
     b[KC_HEAD] = (double)m->E * m->n_vocab * q;
+    b[KC_ROWS] = 0;
     (void)kv;
 }
 
@@ -882,23 +904,21 @@ struct Scratch {            // device buffers freed on scope exit
 
 template <int M>
 static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, const float *dx, float *dout, int32_t *ddots,
-                       int8_t *dq, float2 *dds, StepCtl *ctl, int repeats, float *kernel_ms) {
-    ActSrc s{};
+                       int8_t *dq, float2 *dds, StepCtl *, int repeats, float *kernel_ms) {
     const int n32 = M * (k / 32);
     hipLaunchKernelGGL(lg_k_quant_flat, dim3((n32 * 8 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, st, dx, n32, dq, dds);
     MmArgs a{ dw, k, mrows, dout, dq, dds, ddots };
-    const size_t lds = lds_mm(M, k);
-    int rc;
-    if (ddots) { if ((rc = set_lds(lg_k_mm<M, SRC_Q8, true>, lds))) return rc; }
-    if ((rc = set_lds(lg_k_mm<M, SRC_Q8, false>, lds))) return rc;
-    const dim3 grid((mrows / 8 + 3) / 4);
-    if (ddots) hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, true>), grid, dim3(LG_WG), lds, st, a, s, ctl);
+    lg_hip_model shim;                       // the launcher only needs a stream and the profiling switch
+    shim.stream = st;
+    Launcher lx{ &shim, false };
+    if (ddots) launch_mm<M, true>(lx, 0, a);
     hipEvent_t e0, e1;
     HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
     a.dots = nullptr;
-    hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, false>), grid, dim3(LG_WG), lds, st, a, s, ctl);       // warm-up, also the result
+    launch_mm<M, false>(lx, 0, a);           // warm-up, also the result
     HIP_TRY(hipEventRecord(e0, st));
-    for (int r = 0; r < repeats; ++r) hipLaunchKernelGGL((lg_k_mm<M, SRC_Q8, false>), grid, dim3(LG_WG), lds, st, a, s, ctl);
+    for (int r = 0; r < repeats; ++r) launch_mm<M, false>(lx, 0, a);
+    if (lx.rc) return lx.rc;
     HIP_TRY(hipEventRecord(e1, st));
     HIP_TRY(hipStreamSynchronize(st));
     HIP_TRY(hipGetLastError());
@@ -953,7 +973,7 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
 template <int M>
 static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl, int tiles, int repeats, float *kernel_ms) {
     const int G = a.H / a.nkv, nq = G * M, kst = a.hd + 8;
-    const size_t lds = (size_t)(nq + M) * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
+    const size_t lds = (size_t)nq * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
     int rc = set_lds(lg_k_attn<M>, lds);
     if (rc) return rc;
     hipEvent_t e0, e1;
@@ -997,8 +1017,8 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     StepCtl c{ pos, 0, 0, 0 };
     HIP_TRY(hipMemcpy(ctl, &c, sizeof c, hipMemcpyHostToDevice));
     AttnArgs a{};
-    a.qkv = dq; a.ld = qd; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
-    a.kc = dk; a.vc = dv; a.seq = seq; a.kv_dim = kd; a.window = window; a.owns = 0; a.prerotated = 1; a.eps = 0;
+    a.q = dq; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
+    a.kc = dk; a.vc = dv; a.seq = seq; a.kv_dim = kd; a.window = window;
     a.pm = dpm; a.pl = dpl; a.pacc = dpacc; a.tiles_max = tiles;
     MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, dxq, dxds, dxf };
     hipStream_t st;

@@ -1,0 +1,106 @@
+/* run-hip — the reference CLI's generation path on the gfx950 backend, for token ids.
+ *
+ * The reference's `run` takes text (-p) and a draft-head file (-mtp) and prints text
+ * (src/run.c:697-842).  Tokenizer, chat template and the draft head are outside this build, so
+ * run-hip keeps the flags and the loop (prefill, first token, plain or block-LG_MTP_N speculative
+ * greedy steps, the same stderr statistics lines) but takes the prompt as token ids and, for
+ * -mtp, a file of draft token ids in place of a draft head:
+ *
+ *   run-hip -m model.gguf -p 12,7,99,4 [-n 256] [-mtp drafts.txt | -mtp self]
+ *
+ * -mtp self runs the plain path first and replays its own output as (perfect) drafts: the check
+ * the reference does by hand — output with and without -mtp must be byte-identical
+ * (docs/mtp.md:16-19) — as one command.  Output: generated token ids on stdout, one line.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+
+#include "model.h"
+#include "session.h"
+
+static double now_sec(void) {                       /* wall clock, like src/run.c:42-46 */
+    struct timespec ts;
+    timespec_get(&ts, TIME_UTC);
+    return (double)ts.tv_sec + 1e-9 * (double)ts.tv_nsec;
+}
+
+static int parse_ids(const char *s, int *out, int cap) {
+    int n = 0;
+    while (*s && n < cap) {
+        char *end;
+        long v = strtol(s, &end, 10);
+        if (end == s) break;
+        out[n++] = (int)v;
+        s = end;
+        while (*s == ',' || *s == ' ' || *s == '\n') s++;
+    }
+    return n;
+}
+
+int main(int argc, char **argv) {
+    const char *model = NULL, *prompt = NULL, *mtp = NULL;
+    int n_gen = 256;
+    for (int i = 1; i < argc; i++) {
+        if (!strcmp(argv[i], "-m") && i + 1 < argc) model = argv[++i];
+        else if (!strcmp(argv[i], "-p") && i + 1 < argc) prompt = argv[++i];
+        else if (!strcmp(argv[i], "-mtp") && i + 1 < argc) mtp = argv[++i];
+        else if (!strcmp(argv[i], "-n") && i + 1 < argc) n_gen = atoi(argv[++i]);
+    }
+    if (!model || !prompt) {
+        printf("Usage: %s -m <model.gguf> -p <id,id,...> [-n N] [-mtp <draft-ids.txt> | -mtp self]\n"
+               "       (built with LG_MTP_N=%d: speculative blocks verify %d tokens per step)\n", argv[0], LG_MTP_N, LG_MTP_N);
+        return 1;
+    }
+    static int ids[8192];
+    int n_prompt = parse_ids(prompt, ids, 8192);
+    if (n_prompt < 1 || n_gen < 1) { fprintf(stderr, "run-hip: empty prompt\n"); return 1; }
+    struct lg_session *s = lg_session_open(model);
+    if (!s) { fprintf(stderr, "run-hip: cannot load %s\n", model); return 1; }
+    config_print(&lg_session_model(s)->cfg);
+    const int max_seq = n_prompt + n_gen + 1;                       /* src/run.c:715 */
+    int *emitted = calloc((size_t)n_gen, sizeof(int)), *drafts = NULL, *plain = NULL;
+    if (!emitted) return 1;
+
+    if (mtp) {
+        drafts = calloc((size_t)n_gen + 64, sizeof(int));
+        if (!drafts) return 1;
+        if (!strcmp(mtp, "self")) {
+            plain = calloc((size_t)n_gen, sizeof(int));
+            if (!plain || lg_session_kv(s, max_seq) != 0) return 1;
+            int steps;
+            lg_session_generate(s, ids, n_prompt, n_gen, 1, NULL, plain, &steps);
+            memcpy(drafts, plain, (size_t)n_gen * sizeof(int));
+        } else {
+            FILE *f = fopen(mtp, "r");
+            if (!f) { perror(mtp); return 1; }
+            static char buf[1 << 20];
+            size_t got = fread(buf, 1, sizeof buf - 1, f);
+            buf[got] = 0;
+            fclose(f);
+            parse_ids(buf, drafts, n_gen);
+        }
+    }
+    if (lg_session_kv(s, max_seq) != 0) { fprintf(stderr, "run-hip: kvcache_init failed\n"); return 1; }
+    int steps = 0;
+    double t0 = now_sec();
+    int g = lg_session_generate(s, ids, n_prompt, n_gen, mtp ? LG_MTP_N : 1, drafts, emitted, &steps);
+    double dt = now_sec() - t0;
+    for (int i = 0; i < g; i++) printf("%s%d", i ? "," : "", emitted[i]);
+    printf("\n");
+    fprintf(stderr, "gen:    %d tokens in %.2fs (%.2f tok/s), prompt %d tokens included\n", g, dt, g / (dt > 0 ? dt : 1e-9), n_prompt);
+    if (mtp) {
+        int accepted = g - 1 - steps > 0 ? g - 1 - steps : 0;
+        fprintf(stderr, "mtp:    %d verify/decode steps for %d tokens (block %d, %.2f tokens per step, %d drafts accepted)\n",
+                steps, g, LG_MTP_N, steps ? (double)(g - 1) / steps : 0.0, accepted);
+    }
+    int rc = 0;
+    if (plain) {
+        rc = memcmp(plain, emitted, (size_t)g * sizeof(int)) != 0;
+        fprintf(stderr, "check:  -mtp output %s plain greedy output\n", rc ? "DIFFERS FROM" : "is byte-identical to");
+    }
+    free(emitted); free(drafts); free(plain);
+    lg_session_close(s);
+    return rc;
+}

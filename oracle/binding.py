@@ -12,7 +12,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 REF, I8, I8_LIBM = 0, 1, 2
-ORDER_SEG8, ORDER_CUDA32 = 0, 1
+ORDER_SEG, ORDER_CUDA32 = 0, 1
 _lib = None
 _ref = {}
 

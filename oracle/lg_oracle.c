@@ -81,13 +81,17 @@ int32_t lgo_block_dot(const unsigned char *blk, const int8_t *q) {
     return acc;
 }
 
+/* K segments of this build's matmul order: 8, or 32 for rows of more than 128 blocks (the
+ * wide ffn_down rows), so that every lane's serial chain stays short. */
+int lgo_segments(int k) { return k / 32 > 128 ? 32 : 8; }
+
 /* ---- q4_0 x q8 matmul.  out[j*m+i] = sum_b (xd[j][b]*dw[i][b]) * dot(i,j,b)
  * (src/cuda/model-cuda-i8.cu:813-903); `order` picks how the f32 terms are summed. */
 void lgo_matmul_q4q8(const void *w, int k, int m, const int8_t *xq, const float *xd, int rows,
                      float *out, int32_t *dots, int order) {
-    const int nb = k / 32;
+    const int nb = k / 32, S = lgo_segments(k);
     const unsigned char *base = w;
-    if (order == LGO_ORDER_SEG8 && nb % 8) { fprintf(stderr, "lgo_matmul_q4q8: k=%d not a multiple of 256\n", k); abort(); }
+    if (order == LGO_ORDER_SEG && nb % S) { fprintf(stderr, "lgo_matmul_q4q8: k=%d not a multiple of %d\n", k, 32 * S); abort(); }
     #pragma omp parallel for schedule(static)
     for (int i = 0; i < m; i++) {
         const unsigned char *row = base + (size_t)i * nb * LG_Q4_0_BYTES;
@@ -95,9 +99,9 @@ void lgo_matmul_q4q8(const void *w, int k, int m, const int8_t *xq, const float 
             const int8_t *aq = xq + (size_t)j * k;
             const float *ad = xd + (size_t)j * nb;
             float lane[32];
-            if (order == LGO_ORDER_SEG8) {
-                const int per = nb / 8;
-                for (int s = 0; s < 8; s++) {
+            if (order == LGO_ORDER_SEG) {
+                const int per = nb / S;
+                for (int s = 0; s < S; s++) {
                     float p = 0.0f;
                     for (int b = s * per; b < (s + 1) * per; b++) {
                         const unsigned char *blk = row + (size_t)b * LG_Q4_0_BYTES;
@@ -108,7 +112,7 @@ void lgo_matmul_q4q8(const void *w, int k, int m, const int8_t *xq, const float 
                     }
                     lane[s] = p;
                 }
-                out[(size_t)j * m + i] = tree_sum(lane, 8);
+                out[(size_t)j * m + i] = tree_sum(lane, S);
             } else {
                 for (int l = 0; l < 32; l++) lane[l] = 0.0f;
                 for (int b = 0; b < nb; b++) {
@@ -549,7 +553,7 @@ struct qact { int8_t *q; float *d; };
 static void quant_into(struct qact *a, const float *x, int n) { lgo_quant_q8(x, n, a->q, a->d, NULL); }
 static void mm(const struct gguf_tensor *w, int k, int mrows, const struct qact *a, float *out) {
     if (w->type != GGML_TYPE_Q4_0) { fprintf(stderr, "oracle: matmul weight %s is %s, only q4_0 is on the int8 path\n", w->name, ggml_type_name(w->type)); abort(); }
-    lgo_matmul_q4q8(w->data, k, mrows, a->q, a->d, 1, out, NULL, LGO_ORDER_SEG8);
+    lgo_matmul_q4q8(w->data, k, mrows, a->q, a->d, 1, out, NULL, LGO_ORDER_SEG);
 }
 
 static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos, int exact, float *logits, float *hidden) {

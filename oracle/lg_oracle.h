@@ -24,7 +24,8 @@ enum lgo_mode {
 
 /* f32 combine order of the q4_0 x q8 matmul */
 enum lgo_order {
-    LGO_ORDER_SEG8   = 0,  /* this build: 8 contiguous K segments, serial fma inside, adjacent tree */
+    LGO_ORDER_SEG    = 0,  /* this build: lgo_segments(k) contiguous K segments, serial fma inside each,
+                              adjacent-pair tree across them */
     LGO_ORDER_CUDA32 = 1,  /* reference: 32 lane-strided partials + shfl_down tree
                               (src/cuda/model-cuda-i8.cu:830-845,897-902) */
 };
@@ -40,6 +41,7 @@ void    lgo_rope(float *v, int d, int pos, const float *freq_tab, const float *f
 /* one (query head) attention over an f16 ring: keys start..pos, row of position p = p % seq */
 void    lgo_attention_f16(float *out, const float *q, const uint16_t *kc, const uint16_t *vc,
                           int hd, int kv_dim, int kvh, int seq, int start, int pos, int tiled, int exact);
+int     lgo_segments(int k);
 int     lgo_accept(const int *toks, const int *out, int rows);
 float   lgo_expf(float x); float lgo_tanhf(float x); void lgo_sincosf(float x, float *s, float *c);
 float   lgo_gelu(float x, int exact);

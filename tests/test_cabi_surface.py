@@ -37,24 +37,27 @@ def test_backend_library_defines_the_model_h_symbols(lg):
 
 
 def test_repack_layout_against_numpy(lg):
-    """Tile (group g, it): lane r*8+c holds block c*nit+it of row 8g+r — 16 nibble bytes, then scales."""
+    """Tile (group g, it): lane r*S+c holds block c*nit+it of row g*(64/S)+r — 16 nibble bytes, then scales."""
     H = lg.hiplib.load_hip()
     rng = np.random.default_rng(8)
-    for m, k in ((16, 256), (24, 2560), (8, 512)):
+    for m, k in ((16, 256), (24, 2560), (8, 512), (8, 10240), (16, 15360)):
         w = random_q4_0(rng, m, k)
-        nb, nit = k // 32, k // 256
+        nb = k // 32
+        S = H.lg_hip_segments(k)
+        assert S == (32 if nb > 128 else 8)
+        rw, nit = 64 // S, nb // S
         n = H.lg_hip_repacked_bytes(k, m)
-        assert n == (m // 8) * nit * 1152 == w.size                  # same bytes, reordered
+        assert n == (m // rw) * nit * 1152 == w.size                 # same bytes, reordered
         out = np.zeros(n, np.uint8)
         assert H.lg_hip_repack_q4_0(w, k, m, out) == 0
         blocks = w.reshape(m, nb, 18)
-        tiles = out.reshape(m // 8, nit, 1152)
-        for g in range(m // 8):
+        tiles = out.reshape(m // rw, nit, 1152)
+        for g in range(m // rw):
             for it in range(nit):
-                for r in range(8):
-                    for c in range(8):
-                        blk = blocks[g * 8 + r, c * nit + it]
-                        lane = r * 8 + c
+                for r in range(rw):
+                    for c in range(S):
+                        blk = blocks[g * rw + r, c * nit + it]
+                        lane = r * S + c
                         assert np.array_equal(tiles[g, it, lane * 16:lane * 16 + 16], blk[2:])
                         assert np.array_equal(tiles[g, it, 1024 + lane * 2:1024 + lane * 2 + 2], blk[:2])
     assert H.lg_hip_repacked_bytes(100, 8) == 0 and H.lg_hip_repacked_bytes(256, 12) == 0
@@ -64,6 +67,8 @@ def test_repack_layout_against_numpy(lg):
 
 def test_ring_rows_agree_with_the_oracle(lg, ob):
     H, L = lg.hiplib.load_hip(), ob.lib()
+    for k in (256, 2560, 4096, 4352, 10240):
+        assert H.lg_hip_segments(k) == L.lgo_segments(k)
     for window, max_seq in ((128, 4096), (512, 2300), (1024, 8300), (512, 400), (7, 64)):
         assert H.lg_hip_ring_rows(window, max_seq) == L.lgo_ring_rows(window, max_seq)
 

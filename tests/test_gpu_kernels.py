@@ -17,7 +17,7 @@ def oracle_matmul(ob, w, k, m, x):
     for j in range(rows):
         L.lgo_quant_q8(x[j], k, xq[j], xd[j], xs[j])
     out = np.zeros((rows, m), np.float32); dots = np.zeros((rows, m, nb), np.int32)
-    L.lgo_matmul_q4q8(w, k, m, xq, xd, rows, out, dots.ctypes.data, ob.ORDER_SEG8)
+    L.lgo_matmul_q4q8(w, k, m, xq, xd, rows, out, dots.ctypes.data, ob.ORDER_SEG)
     return xq, xd, xs, out, dots
 
 

@@ -82,7 +82,7 @@ def test_matmul_q4q8_against_float64(ob, m, k, rows):
     dots_want = np.einsum("ibe,jbe->jib", codes - 8, xq.reshape(rows, nb, 32).astype(np.int32))
     want = np.einsum("jib,ib,jb->ji", dots_want.astype(np.float64), dw.astype(np.float64), xd.astype(np.float64))
     outs = {}
-    for order in (ob.ORDER_SEG8, ob.ORDER_CUDA32):
+    for order in (ob.ORDER_SEG, ob.ORDER_CUDA32):
         out = np.zeros((rows, m), np.float32); dots = np.zeros((rows, m, nb), np.int32)
         L.lgo_matmul_q4q8(w, k, m, xq, xd, rows, out, dots.ctypes.data, order)
         assert np.array_equal(dots, dots_want)                         # int32 block dots: exact
@@ -90,12 +90,12 @@ def test_matmul_q4q8_against_float64(ob, m, k, rows):
         assert np.abs(out - want).max() <= 1e-5 * scale
         outs[order] = out
     # the two summation orders are the same mathematics: they differ by rounding only
-    assert np.abs(outs[ob.ORDER_SEG8] - outs[ob.ORDER_CUDA32]).max() <= 2e-6 * np.abs(want).max()
+    assert np.abs(outs[ob.ORDER_SEG] - outs[ob.ORDER_CUDA32]).max() <= 2e-6 * np.abs(want).max()
     # transposition / indexing check: the f32-activation matmul on the dequantized operands agrees to q8 noise
     xdeq = (xq.reshape(rows, nb, 32).astype(np.float32) * xd[:, :, None]).reshape(rows, k)
     ref = np.zeros(m, np.float32)
     L.lgo_matmul_f32(w, 2, k, m, np.ascontiguousarray(xdeq[0]), ref)
-    assert np.abs(ref - outs[ob.ORDER_SEG8][0]).max() <= 1e-4 * np.abs(want).max()
+    assert np.abs(ref - outs[ob.ORDER_SEG][0]).max() <= 1e-4 * np.abs(want).max()
 
 
 def test_rmsnorm_both_orders(ob):
