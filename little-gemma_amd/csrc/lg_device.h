@@ -3,7 +3,7 @@
 // Numeric contract shared with the CPU oracle: every float reduction below has ONE defined
 // order, chosen to be natural for a 64-lane wavefront, and every elementary function comes
 // from include/lg_math.h.  Integer work (q8 quantization, q4_0 x q8 block dots) is exact.
-//   * row sum of squares: 64 lane partials, element i belongs to lane (i/4)%64, fma in
+//   * row sum of squares: 256 lane partials, element i belongs to lane (i/4)%256, fma in
 //     ascending i, then an adjacent-pair binary tree over the lanes;
 //   * q4_0 x q8 matmul: S contiguous K segments per output (S = 8, or 32 for rows of more than
 //     128 blocks), one lane each, serial fma over the segment's blocks, adjacent-pair tree over
@@ -30,35 +30,69 @@
 // A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
 __host__ __device__ static inline int lg_segments(int k) { return (k >> 5) > 128 ? 32 : 8; }
 
-__device__ __forceinline__ float lg_wave_sum64(float v) {
-    v = v + __shfl_xor(v, 1);
-    v = v + __shfl_xor(v, 2);
-    v = v + __shfl_xor(v, 4);
-    v = v + __shfl_xor(v, 8);
-    v = v + __shfl_xor(v, 16);
-    v = v + __shfl_xor(v, 32);
+// Cross-lane exchange for the reductions.  Within a row of 16 lanes DPP moves data in one VALU
+// instruction; the partner patterns (swap inside pairs, swap pairs inside quads, mirror 8, mirror
+// 16) differ from xor-butterflies only in which lane of the already-uniform sub-group supplies the
+// value, so sums come out in the same adjacent-pair tree order (addition is commutative) and
+// max / integer sums are order-free anyway.
+template <int CTRL>
+__device__ __forceinline__ float lg_dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int lg_dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+#define LG_DPP_SWAP1   0xB1     // quad_perm [1,0,3,2]
+#define LG_DPP_SWAP2   0x4E     // quad_perm [2,3,0,1]
+#define LG_DPP_MIRROR8 0x141    // row_half_mirror
+#define LG_DPP_MIRROR16 0x140   // row_mirror
+
+__device__ __forceinline__ float lg_sum8(float v) {
+    v = v + lg_dpp_f<LG_DPP_SWAP1>(v);
+    v = v + lg_dpp_f<LG_DPP_SWAP2>(v);
+    v = v + lg_dpp_f<LG_DPP_MIRROR8>(v);
     return v;
 }
-__device__ __forceinline__ float lg_sum8(float v) {
-    v = v + __shfl_xor(v, 1);
-    v = v + __shfl_xor(v, 2);
-    v = v + __shfl_xor(v, 4);
+__device__ __forceinline__ float lg_sum16(float v) {
+    v = lg_sum8(v);
+    v = v + lg_dpp_f<LG_DPP_MIRROR16>(v);
     return v;
 }
 __device__ __forceinline__ float lg_sum32(float v) {
-    v = v + __shfl_xor(v, 1);
-    v = v + __shfl_xor(v, 2);
-    v = v + __shfl_xor(v, 4);
-    v = v + __shfl_xor(v, 8);
+    v = lg_sum16(v);
     v = v + __shfl_xor(v, 16);
     return v;
 }
-__device__ __forceinline__ float lg_max_n(float v, int n) {       // n = 8 or 32 lanes
-    for (int o = 1; o < n; o <<= 1) v = fmaxf(v, __shfl_xor(v, o));
+__device__ __forceinline__ float lg_wave_sum64(float v) {
+    v = lg_sum32(v);
+    v = v + __shfl_xor(v, 32);
     return v;
 }
-__device__ __forceinline__ int lg_isum_n(int v, int n) {
-    for (int o = 1; o < n; o <<= 1) v += __shfl_xor(v, o);
+template <int S>
+__device__ __forceinline__ float lg_sum_seg(float v) {       // S = 8 or 32 adjacent lanes
+    if (S == 8) return lg_sum8(v);
+    return lg_sum32(v);
+}
+__device__ __forceinline__ float lg_max8(float v) {
+    v = fmaxf(v, lg_dpp_f<LG_DPP_SWAP1>(v));
+    v = fmaxf(v, lg_dpp_f<LG_DPP_SWAP2>(v));
+    v = fmaxf(v, lg_dpp_f<LG_DPP_MIRROR8>(v));
+    return v;
+}
+__device__ __forceinline__ float lg_max_n(float v, int n) {       // n = 8, 32 or 64 lanes
+    v = lg_max8(v);
+    if (n >= 16) v = fmaxf(v, lg_dpp_f<LG_DPP_MIRROR16>(v));
+    if (n >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+    if (n >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ int lg_isum_n(int v, int n) {          // n = 8 or 32 lanes
+    v += lg_dpp_i<LG_DPP_SWAP1>(v);
+    v += lg_dpp_i<LG_DPP_SWAP2>(v);
+    v += lg_dpp_i<LG_DPP_MIRROR8>(v);
+    if (n >= 16) v += lg_dpp_i<LG_DPP_MIRROR16>(v);
+    if (n >= 32) v += __shfl_xor(v, 16);
     return v;
 }
 

@@ -171,6 +171,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     m->ffn_len.assign(c->ffn_len, c->ffn_len + c->n_layer);
     m->head_dim.assign(c->head_dim, c->head_dim + c->n_layer);
     m->n_head_kv.assign(c->n_head_kv, c->n_head_kv + c->n_layer);
+    if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
     *out = m;
@@ -299,7 +300,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         Layer &y = m->L[L];
         y.is_local = m->is_local[L]; y.hd = m->head_dim[L]; y.nkv = m->n_head_kv[L]; y.nff = m->ffn_len[L];
         if (y.hd != 64 && y.hd != 128 && y.hd != 256 && y.hd != 512) return fail(-2, "model_commit: layer %d head size %d (64/128/256/512 are built)", L, y.hd);
-        if (y.nkv <= 0 || H % y.nkv || (H / y.nkv) * max_rows > 32) return fail(-2, "model_commit: layer %d: heads %d / kv heads %d with %d rows exceeds 32 queries per kv head", L, H, y.nkv, max_rows);
+        if (y.nkv <= 0 || H % y.nkv || H / y.nkv > 8) return fail(-2, "model_commit: layer %d: %d query heads per kv head (at most 8 are built)", L, H / y.nkv);
         if (y.nff % 32) return fail(-2, "model_commit: layer %d feed-forward width %d must be a multiple of 32", L, y.nff);
         y.qd = H * y.hd; y.kd = y.nkv * y.hd;
         y.owns = L < m->n_kv_start;
@@ -340,7 +341,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if ((rc = upload_tiled(m, rows, y.nff, &y.wdown, stage))) return rc;
         rows.clear();
         if (m->ple) {
-            if (m->ple % 256) return fail(-2, "model_commit: per-layer width %d must be a multiple of 256", m->ple);
+            if (m->ple != 256) return fail(-2, "model_commit: per-layer width %d (256 is built)", m->ple);
             const HostTensor *ig = find(m, lname(L, "inp_gate.weight")), *pj = find(m, lname(L, "proj.weight"));
             if ((rc = check_mat(ig, lname(L, "inp_gate.weight"), E, m->ple))) return rc;
             if ((rc = check_mat(pj, lname(L, "proj.weight"), m->ple, E))) return rc;
@@ -589,7 +590,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os;
         s.w_pre = w_pre; s.h_out = h_out;
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
-        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M), dim3(64), 0, s, m->ctl);
+        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M), dim3(LG_WG), 0, s, m->ctl);
         if (s.x_out) cur ^= 1;
         have_x = true; pend_dout = pend_w = pend_os = nullptr;
     };
@@ -616,13 +617,13 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             LAUNCH(KC_QKVPOST, lg_k_qkv_post, dim3(H + (y.owns ? 2 * y.nkv : 0), M), dim3(64), 0, p, m->ctl);
         }
         {   // attention tiles + merge
-            const int G = H / y.nkv, nq = G * M, kst = y.hd + 8;
+            const int G = H / y.nkv, kst = y.hd + 8;
             AttnArgs a{};
             a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max;
-            const size_t lds = (size_t)nq * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
-            LAUNCH(KC_ATTN, (lg_k_attn<M>), dim3(kv->tiles_max, y.nkv), dim3(LG_WG), lds, a, m->ctl);
+            const size_t lds = (size_t)G * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
+            LAUNCH(KC_ATTN, lg_k_attn, dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), lds, a, m->ctl);
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, m->aq, m->ads, nullptr };
             LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
@@ -647,7 +648,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
             a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
             a.pq = m->pq; a.pds = m->pds;
-            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E) + (size_t)M * 32 * 4, a, m->ctl);
+            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E), a, m->ctl);
             MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, m->pds, nullptr };
             launch_mm<M, false>(lx, KC_PLEPROJ, p);
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
@@ -972,15 +973,15 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
 
 template <int M>
 static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl, int tiles, int repeats, float *kernel_ms) {
-    const int G = a.H / a.nkv, nq = G * M, kst = a.hd + 8;
-    const size_t lds = (size_t)nq * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)nq * 32 * 4 + (size_t)nq * 4;
-    int rc = set_lds(lg_k_attn<M>, lds);
+    const int G = a.H / a.nkv, kst = a.hd + 8;
+    const size_t lds = (size_t)G * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
+    int rc = set_lds(lg_k_attn, lds);
     if (rc) return rc;
     hipEvent_t e0, e1;
     HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
     for (int r = 0; r < repeats + 1; ++r) {
         if (r == 1) HIP_TRY(hipEventRecord(e0, st));
-        hipLaunchKernelGGL((lg_k_attn<M>), dim3(tiles, a.nkv), dim3(LG_WG), lds, st, a, ctl);
+        hipLaunchKernelGGL(lg_k_attn, dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
         hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
     }
     HIP_TRY(hipEventRecord(e1, st));
@@ -996,7 +997,7 @@ static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl,
 extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, int rows, int n_head, int n_head_kv,
                                 int hd, int seq, int window, int pos, float *out, int repeats, float *kernel_ms) {
     if (!q || !kc || !vc || !out) return fail(-1, "attention: null argument");
-    if (rows < 1 || rows > LG_HIP_MAX_ROWS || n_head_kv < 1 || n_head % n_head_kv || (n_head / n_head_kv) * rows > 32 ||
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || n_head_kv < 1 || n_head % n_head_kv || n_head / n_head_kv > 8 ||
         (hd != 64 && hd != 128 && hd != 256 && hd != 512) || pos < 0 || seq < 1)
         return fail(-2, "attention: unsupported shape");
     if (window > 0 ? seq < window + rows - 1 && seq < pos + rows : seq < pos + rows)

@@ -43,44 +43,55 @@ struct RowArgs {
     float          eps;
 };
 
+// Sum over the 256 lanes of a workgroup in adjacent-pair tree order; every thread gets the result.
+__device__ __forceinline__ float lg_block_sum256(float v, float *scratch4) {
+    v = lg_wave_sum64(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (scratch4[0] + scratch4[1]) + (scratch4[2] + scratch4[3]);
+}
+
+#define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
-__global__ __launch_bounds__(64) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
-    const int lane = threadIdx.x, j = blockIdx.x;
-    const int E = s.E, nv = E >> 8;
-    float4 xv[LG_MAXV], dv[LG_MAXV], wpost[LG_MAXV], wpre[LG_MAXV];
+__global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
+    __shared__ float red[4];
+    const int t = threadIdx.x, j = blockIdx.x;
+    const int E = s.E, nq = E >> 2;                          // float4 quads in a row; thread t owns quads t + 256*v
+    float4 xv[LG_ROWV], dv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
     // issue every load up front: one memory round trip for the whole row
     if (s.emb) {
         const int tok = s.toks[ctl->step * M + j];
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) {
-            const float4 t = lg_tiled_deq4(s.emb, s.emb_nit, s.emb_seg, tok, 256 * v + 4 * lane);
-            xv[v] = make_float4(t.x * s.emb_scale, t.y * s.emb_scale, t.z * s.emb_scale, t.w * s.emb_scale);
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+            const float4 e = lg_tiled_deq4(s.emb, s.emb_nit, s.emb_seg, tok, 4 * (t + 256 * v));
+            xv[v] = make_float4(e.x * s.emb_scale, e.y * s.emb_scale, e.z * s.emb_scale, e.w * s.emb_scale);
         }
     } else {
         const float4 *xr = (const float4 *)(s.x + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) xv[v] = xr[64 * v + lane];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) xv[v] = xr[t + 256 * v];
     }
     if (s.dout) {
         const float4 *dr = (const float4 *)(s.dout + (size_t)j * E), *wr = (const float4 *)s.w_post;
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) { dv[v] = dr[64 * v + lane]; wpost[v] = wr[64 * v + lane]; }
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { dv[v] = dr[t + 256 * v]; wpost[v] = wr[t + 256 * v]; }
     }
     if (s.w_pre) {
         const float4 *wr = (const float4 *)s.w_pre;
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) wpre[v] = wr[64 * v + lane];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) wpre[v] = wr[t + 256 * v];
     }
     if (s.dout) {
         float ss = 0.0f;
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) ss = lg_sumsq4(dv[v], ss);
-        ss = lg_wave_sum64(ss);
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
+        ss = lg_block_sum256(ss, red);
         const float sc = 1.0f / sqrtf(ss / (float)E + s.eps);
         const bool has_os = s.os != nullptr;
         const float osv = has_os ? s.os[0] : 1.0f;
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) {
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
             const float4 w = wpost[v];
             float4 r;
             r.x = xv[v].x + dv[v].x * sc * w.x;  r.y = xv[v].y + dv[v].y * sc * w.y;
@@ -92,16 +103,16 @@ __global__ __launch_bounds__(64) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
     if (s.x_out) {
         float4 *xo = (float4 *)(s.x_out + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) xo[64 * v + lane] = xv[v];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) xo[t + 256 * v] = xv[v];
     }
     if (s.w_pre) {
         float ss = 0.0f;
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) ss = lg_sumsq4(xv[v], ss);
-        ss = lg_wave_sum64(ss);
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(xv[v], ss);
+        ss = lg_block_sum256(ss, red);
         const float sc = 1.0f / sqrtf(ss / (float)E + s.eps);
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) {
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
             const float4 w = wpre[v];
             xv[v] = make_float4(xv[v].x * sc * w.x, xv[v].y * sc * w.y, xv[v].z * sc * w.z, xv[v].w * sc * w.w);
         }
@@ -109,16 +120,18 @@ __global__ __launch_bounds__(64) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
     if (s.h_out) {
         float4 *ho = (float4 *)(s.h_out + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_MAXV; ++v) if (v < nv) ho[64 * v + lane] = xv[v];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ho[t + 256 * v] = xv[v];
     }
     uint32_t *qrow = (uint32_t *)(s.q + (size_t)j * E);
     float2 *drow = s.ds + (size_t)j * (E >> 5);
     #pragma unroll
-    for (int v = 0; v < LG_MAXV; ++v) if (v < nv) {
+    for (int v = 0; v < LG_ROWV; ++v) {
+        // nq is a multiple of 64, so a whole wavefront is either inside the row or outside it
+        if (t + 256 * v >= nq) break;
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
-        qrow[64 * v + lane] = packed;
-        if ((lane & 7) == 0) drow[(64 * v + lane) >> 3] = make_float2(d, __int_as_float(sum));
+        qrow[t + 256 * v] = packed;
+        if ((t & 7) == 0) drow[(t + 256 * v) >> 3] = make_float2(d, __int_as_float(sum));
     }
 }
 
@@ -135,45 +148,69 @@ __global__ __launch_bounds__(LG_WG) void lg_k_quant_flat(const float *x, int n32
 }
 
 // Copy M already-quantized rows (int8 + {scale,sum}) from global memory into LDS.
+// Eight loads are issued before the first store (named temporaries, not an array, and a scheduling
+// barrier between the two halves), so a workgroup pays about one memory round trip per 8 elements
+// per thread instead of one per element.  Indices past the end are clamped to the last element,
+// which is then copied more than once with the same value: no branches.
+template <typename T>
+__device__ __forceinline__ void lg_copy_batched(const T *src, T *dst, int n) {
+    const int nt = blockDim.x;
+    for (int i0 = threadIdx.x; i0 < n; i0 += 8 * nt) {
+        const int last = n - 1;
+        const int a0 = min(i0, last), a1 = min(i0 + nt, last), a2 = min(i0 + 2 * nt, last), a3 = min(i0 + 3 * nt, last);
+        const int a4 = min(i0 + 4 * nt, last), a5 = min(i0 + 5 * nt, last), a6 = min(i0 + 6 * nt, last), a7 = min(i0 + 7 * nt, last);
+        const T t0 = src[a0], t1 = src[a1], t2 = src[a2], t3 = src[a3], t4 = src[a4], t5 = src[a5], t6 = src[a6], t7 = src[a7];
+        __builtin_amdgcn_sched_barrier(0);
+        dst[a0] = t0; dst[a1] = t1; dst[a2] = t2; dst[a3] = t3; dst[a4] = t4; dst[a5] = t5; dst[a6] = t6; dst[a7] = t7;
+    }
+}
 template <int M>
 __device__ __forceinline__ void lg_load_q8(const int8_t *q, const float2 *ds, int k, int8_t *lq, float2 *lds_ds) {
-    const int n16 = M * k / 16, nt = blockDim.x;
-    const uint4 *src = (const uint4 *)q;
-    uint4 *dst = (uint4 *)lq;
-    for (int i = threadIdx.x; i < n16; i += nt) dst[i] = src[i];
-    const int nd = M * (k >> 5);
-    for (int i = threadIdx.x; i < nd; i += nt) lds_ds[i] = ds[i];
+    lg_copy_batched<uint4>((const uint4 *)q, (uint4 *)lq, M * k / 16);
+    lg_copy_batched<float2>(ds, lds_ds, M * (k >> 5));
 }
 
 // ---------------------------------------------------------------------------------------------
 // G row groups against M q8 activation rows held in LDS.  A row is cut into S contiguous K
 // segments (S = 8, or 32 for rows longer than 128 blocks); lane = r*S + c owns row r of the group
 // (64/S rows per group) and segment c, and walks the segment's nit blocks with a serial fma chain.
-// The G groups share every activation load (gate with up, or two neighbouring groups).  On return
-// every lane of a row holds that row's M results (adjacent-pair tree over the S lanes done).
+// The G groups share every activation load (gate with up, or two neighbouring groups).
+// Weights are fetched in chunks of LG_U tiles per group; the first chunk is requested before the
+// activations are staged (weights depend on nothing), each later chunk while the previous one is
+// being consumed.
+#define LG_U 5
+template <int G>
+struct WChunk { uint4 q[G][LG_U]; uint32_t s[G][LG_U]; };
+
+template <int G>
+__device__ __forceinline__ void lg_mm_fetch(WChunk<G> &w, const uint8_t *const (&wg)[G], int it0, int nit, int lane) {
+    #pragma unroll
+    for (int u = 0; u < LG_U; ++u)
+        #pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;                 // clamp: never read past the group
+            w.q[g][u] = *(const uint4 *)(wg[g] + (size_t)it * LG_TILE + lane * 16);
+            w.s[g][u] = *(const uint16_t *)(wg[g] + (size_t)it * LG_TILE + 1024 + lane * 2);
+        }
+}
+
+// On return every lane of a row holds that row's M results (adjacent-pair tree over the S lanes done).
+// `first` must hold the chunk of tiles 0..LG_U-1.
 template <int M, int S, int G, bool DUMP>
-__device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], int nit, const int8_t *act,
+__device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChunk<G> &first, int nit, const int8_t *act,
                                              const float2 *actds, int k, float (&acc)[G][M], int lane,
                                              int32_t *dots, int m, const int (&row)[G]) {
-    constexpr int U = 5;                                   // tiles in flight per group
     const int c = lane & (S - 1), nb = k >> 5;
     #pragma unroll
     for (int g = 0; g < G; ++g)
         #pragma unroll
         for (int j = 0; j < M; ++j) acc[g][j] = 0.0f;
-    for (int it0 = 0; it0 < nit; it0 += U) {
-        uint4 wq[G][U];
-        uint16_t ws[G][U];
+    WChunk<G> cur = first;
+    for (int it0 = 0; it0 < nit; it0 += LG_U) {
+        WChunk<G> nxt;
+        if (it0 + LG_U < nit) lg_mm_fetch<G>(nxt, wg, it0 + LG_U, nit, lane);
         #pragma unroll
-        for (int u = 0; u < U; ++u)
-            #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const int it = it0 + u < nit ? it0 + u : nit - 1;             // clamp: no out-of-range load
-                wq[g][u] = *(const uint4 *)(wg[g] + (size_t)it * LG_TILE + lane * 16);
-                ws[g][u] = *(const uint16_t *)(wg[g] + (size_t)it * LG_TILE + 1024 + lane * 2);
-            }
-        #pragma unroll
-        for (int u = 0; u < U; ++u) {
+        for (int u = 0; u < LG_U; ++u) {
             if (it0 + u >= nit) break;
             const int b = c * nit + it0 + u;
             #pragma unroll
@@ -182,30 +219,28 @@ __device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], int 
                 const int4 a0 = *(const int4 *)(act + (size_t)j * k + b * 32), a1 = *(const int4 *)(act + (size_t)j * k + b * 32 + 16);
                 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const int dot = lg_block_dot(wq[g][u], a0, a1, __float_as_int(ds.y));
+                    const int dot = lg_block_dot(cur.q[g][u], a0, a1, __float_as_int(ds.y));
                     if (DUMP) dots[((size_t)j * m + row[g]) * nb + b] = dot;
-                    acc[g][j] = lg_fmaf(ds.x * lg_h2f(ws[g][u]), (float)dot, acc[g][j]);
+                    acc[g][j] = lg_fmaf(ds.x * lg_h2f((uint16_t)cur.s[g][u]), (float)dot, acc[g][j]);
                 }
             }
         }
+        if (it0 + LG_U < nit) cur = nxt;
     }
     #pragma unroll
     for (int g = 0; g < G; ++g)
         #pragma unroll
-        for (int j = 0; j < M; ++j) {
-            float v = acc[g][j];
-            #pragma unroll
-            for (int o = 1; o < S; o <<= 1) v = v + __shfl_xor(v, o);
-            acc[g][j] = v;
-        }
+        for (int j = 0; j < M; ++j) acc[g][j] = lg_sum_seg<S>(acc[g][j]);
 }
 
+// acc[j] for a lane-dependent j without indexing the register array (an indexed access would
+// move the accumulators to scratch memory): bitwise select over the M candidates.
 template <int M>
 __device__ __forceinline__ float lg_pick(const float (&acc)[M], int j) {
-    float v = acc[0];
+    uint32_t v = 0;
     #pragma unroll
-    for (int t = 1; t < M; ++t) v = j == t ? acc[t] : v;
-    return v;
+    for (int t = 0; t < M; ++t) v |= __float_as_uint(acc[t]) & (uint32_t)-(int)(j == t);
+    return __uint_as_float(v);
 }
 
 struct MmArgs {
@@ -218,19 +253,16 @@ struct MmArgs {
 };
 
 // Plain matmul: out[j][i] f32.  blockDim = 64*W wavefronts, each wavefront takes G neighbouring
-// row groups (G*64/S rows) per pass; grid covers ceil(m / (W*G*64/S)) passes.
+// row groups (G*64/S rows); grid covers ceil(groups / (W*G)) workgroups.
 template <int M, int S, int G, bool DUMP>
-__global__ __launch_bounds__(LG_WG) void lg_k_mm(MmArgs a) {
+__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm(MmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
-    __syncthreads();
     constexpr int RW = 64 / S;                                // rows per group
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int nit = (a.k >> 5) / S, ngroups = a.m / RW;
     const int g0 = (blockIdx.x * nw + wave) * G;
-    if (g0 >= ngroups) return;
     const uint8_t *wg[G];
     int row[G];
     #pragma unroll
@@ -239,8 +271,13 @@ __global__ __launch_bounds__(LG_WG) void lg_k_mm(MmArgs a) {
         wg[g] = a.w + (size_t)gi * nit * LG_TILE;
         row[g] = gi * RW + lane / S;
     }
+    WChunk<G> first;
+    lg_mm_fetch<G>(first, wg, 0, nit, lane);
+    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    __syncthreads();
+    if (g0 >= ngroups) return;
     float acc[G][M];
-    lg_mm_groups<M, S, G, DUMP>(wg, nit, lq, lds, a.k, acc, lane, a.dots, a.m, row);
+    lg_mm_groups<M, S, G, DUMP>(wg, first, nit, lq, lds, a.k, acc, lane, a.dots, a.m, row);
     const int c = lane & (S - 1);
     if (c < M) {
         #pragma unroll
@@ -260,20 +297,22 @@ struct GegluArgs {
     float2        *gds;      // [M][n_ff/32]
 };
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_mm_geglu(GegluArgs a) {
+__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_geglu(GegluArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
     __shared__ float gbuf[LG_HIP_MAX_ROWS_DEV][32];
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
-    __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
     const int t = blockIdx.x;                               // 32-wide slice of n_ff
     const size_t gstride = (size_t)nit * LG_TILE;
     const uint8_t *wg[2] = { a.w + ((size_t)t * 8 + wave) * gstride, a.w + ((size_t)t * 8 + 4 + wave) * gstride };
     const int row[2] = { 0, 0 };
+    WChunk<2> first;
+    lg_mm_fetch<2>(first, wg, 0, nit, lane);
+    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    __syncthreads();
     float acc[2][M];
-    lg_mm_groups<M, 8, 2, false>(wg, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
+    lg_mm_groups<M, 8, 2, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
     const int c = lane & 7, r = lane >> 3;
     if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * lg_pick<M>(acc[1], c);
     __syncthreads();
@@ -304,44 +343,38 @@ struct PleGateArgs {
     float2        *pds;      // [M][ple/32]
 };
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_mm_plegate(PleGateArgs a, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const StepCtl *ctl) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
-    float *ipl = (float *)(lds + (size_t)M * (a.k >> 5));        // [M][32]: this workgroup's slice
     __shared__ float gbuf[LG_HIP_MAX_ROWS_DEV][32];
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    __shared__ float ipl[LG_HIP_MAX_ROWS_DEV][32];           // this workgroup's 32 elements of ipl, per row
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
     const int ple = a.ple;
-    for (int j = wave; j < M; j += LG_WG / 64) {              // one wavefront per row: slice norm
-        const float *pr = a.pmp_raw + (size_t)j * a.n_layer * ple + (size_t)a.layer * ple;
-        float ss = 0.0f;
-        for (int v = 0; 256 * v < ple; ++v) {
-            const int e0 = 256 * v + 4 * lane;
-            if (e0 < ple) {
-                float4 p = *(const float4 *)(pr + e0);
-                p = make_float4(p.x * a.pscale, p.y * a.pscale, p.z * a.pscale, p.w * a.pscale);
-                ss = lg_sumsq4(p, ss);
-            }
-        }
-        ss = lg_wave_sum64(ss);
-        const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
-        if (lane < 32) {
-            const int e = blockIdx.x * 32 + lane;
-            const int tok = a.toks[ctl->step * M + j];
-            const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
-            const float p = pr[e] * a.pscale * sc * a.proj_norm[e];
-            const float tk = lg_q4_0_elem(trow, a.layer * ple + e) * a.tscale;
-            ipl[j * 32 + lane] = (p + tk) * a.rsqrt2;
-        }
-    }
-    __syncthreads();
     const uint8_t *wg[1] = { a.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
     const int row[1] = { 0 };
+    WChunk<1> first;
+    lg_mm_fetch<1>(first, wg, 0, nit, lane);
+    // ipl slice: all loads of a row issued together (projection slice, token row bytes, norm weight)
+    for (int j = wave; j < M; j += LG_WG / 64) {
+        const float *pr = a.pmp_raw + (size_t)j * a.n_layer * ple + (size_t)a.layer * ple;
+        const int tok = a.toks[ctl->step * M + j];
+        const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
+        const int e = blockIdx.x * 32 + (lane & 31);
+        const float4 p4 = 4 * lane < ple ? *(const float4 *)(pr + 4 * lane) : make_float4(0, 0, 0, 0);
+        const float pe = pr[e], wn = a.proj_norm[e];
+        const float tk = lg_q4_0_elem(trow, a.layer * ple + e) * a.tscale;
+        const float4 p = make_float4(p4.x * a.pscale, p4.y * a.pscale, p4.z * a.pscale, p4.w * a.pscale);
+        const float ss = lg_wave_sum64(lg_sumsq4(p, 0.0f));                 // ple <= 256: one quad per lane
+        const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
+        if (lane < 32) ipl[j][lane] = (pe * a.pscale * sc * wn + tk) * a.rsqrt2;
+    }
+    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    __syncthreads();
     float acc[1][M];
-    lg_mm_groups<M, 8, 1, false>(wg, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
+    lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
     const int c = lane & 7, r = lane >> 3;
-    if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * ipl[c * 32 + wave * 8 + r];
+    if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * ipl[c][wave * 8 + r];
     __syncthreads();
     for (int j = threadIdx.x >> 5; j < M; j += LG_WG / 32) {
         const int i = threadIdx.x & 31;
@@ -364,7 +397,7 @@ struct HeadArgs {
     float *pval; int *pidx; // [gridDim.x][M]
 };
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_mm_head(HeadArgs a) {
+__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_head(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
@@ -382,7 +415,9 @@ __global__ __launch_bounds__(LG_WG) void lg_k_mm_head(HeadArgs a) {
         const uint8_t *wg[2] = { a.w + (size_t)g0 * nit * LG_TILE, a.w + (size_t)(g0 + 1) * nit * LG_TILE };
         const int row[2] = { g0 * 8 + r, g0 * 8 + 8 + r };
         float acc[2][M];
-        lg_mm_groups<M, 8, 2, false>(wg, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
+        WChunk<2> first;
+        lg_mm_fetch<2>(first, wg, 0, nit, lane);
+        lg_mm_groups<M, 8, 2, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
         if (c < M) {
             #pragma unroll
             for (int g = 0; g < 2; ++g) {
@@ -495,22 +530,23 @@ __global__ __launch_bounds__(64) void lg_k_qkv_post(QkvPostArgs a, const StepCtl
     const int head = isq ? job : (job - a.H) % a.nkv;
     const float *src = a.qkv + (size_t)j * a.ld + (isq ? (size_t)head * hd : (size_t)(isv ? a.v_off : a.k_off) + (size_t)head * hd);
     const float *w = isq ? a.q_norm : (isv ? nullptr : a.k_norm);
-    float4 xv[2];
-    float ss = 0.0f;
+    float4 xv[2], wv[2];
+    float ss0 = 0.0f, ss1 = 0.0f;                            // lanes l and l+64 of the 256-lane sum order
     #pragma unroll
     for (int v = 0; v < 2; ++v) {
         const int e0 = 256 * v + 4 * lane;
-        if (e0 < hd) { xv[v] = *(const float4 *)(src + e0); ss = lg_sumsq4(xv[v], ss); }
+        if (e0 < hd) { xv[v] = *(const float4 *)(src + e0); if (w) wv[v] = *(const float4 *)(w + e0); }
     }
-    ss = lg_wave_sum64(ss);
+    if (4 * lane < hd) ss0 = lg_sumsq4(xv[0], 0.0f);
+    if (256 + 4 * lane < hd) ss1 = lg_sumsq4(xv[1], 0.0f);
+    const float ss = lg_wave_sum64(ss0) + lg_wave_sum64(ss1);
     const float sc = 1.0f / sqrtf(ss / (float)hd + a.eps);
     #pragma unroll
     for (int v = 0; v < 2; ++v) {
         const int e0 = 256 * v + 4 * lane;
         if (e0 >= hd) continue;
         float4 r;
-        if (w) { const float4 ww = *(const float4 *)(w + e0);
-                 r = make_float4(xv[v].x * sc * ww.x, xv[v].y * sc * ww.y, xv[v].z * sc * ww.z, xv[v].w * sc * ww.w); }
+        if (w) r = make_float4(xv[v].x * sc * wv[v].x, xv[v].y * sc * wv[v].y, xv[v].z * sc * wv[v].z, xv[v].w * sc * wv[v].w);
         else r = make_float4(xv[v].x * sc, xv[v].y * sc, xv[v].z * sc, xv[v].w * sc);
         vec[e0] = r.x; vec[e0 + 1] = r.y; vec[e0 + 2] = r.z; vec[e0 + 3] = r.w;
     }
@@ -537,9 +573,8 @@ __global__ __launch_bounds__(64) void lg_k_qkv_post(QkvPostArgs a, const StepCtl
 
 // ---------------------------------------------------------------------------------------------
 // Attention.  Keys are processed in tiles of 32 aligned to absolute positions (tile n covers
-// positions 32n..32n+31).  One workgroup per (kv head, tile): it stages the tile's K and V rows in
-// LDS once for the gqa*M (head,row) queries that share the kv head, and writes for each query the
-// tile's partial softmax (max, sum, V-accumulator).
+// positions 32n..32n+31); for each (head, draft row, tile) a partial softmax (max, sum,
+// V-accumulator) is written, merged afterwards in ascending tile order.
 // Defined order: score = (a0+a1)+(a2+a3), a_c = fma chain over dims i%4==c; m = max over valid
 // keys; e = exp(s-m); l = adjacent tree over the 32 key slots; acc[d] = fma chain over valid
 // slots ascending.
@@ -550,105 +585,114 @@ struct AttnArgs {
     int seq, kv_dim, window; // ring rows, row width, 0 = global
     float *pm, *pl, *pacc;   // partials: [M*H][tiles_max], [M*H][tiles_max][hd]
     int tiles_max;
+    __device__ __forceinline__ uint4 kc4(size_t off) const { return *(const uint4 *)(kc + off); }
+    __device__ __forceinline__ uint4 vc4(size_t off) const { return *(const uint4 *)(vc + off); }
 };
 
 __device__ __forceinline__ int lg_win_start(int pos, int window) {
     return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
 }
 
-template <int M>
+// One workgroup per (tile, kv head, draft row): the G = H/nkv query heads of the kv head's group.
+// The score of (query g, key slot) is split over two lanes of the same wavefront (lane and lane^32):
+// each runs two of the four partial chains, and the halves meet as (a0+a1)+(a2+a3).
 __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int hd = a.hd, G = a.H / a.nkv, nq = G * M;
+    const int hd = a.hd, G = a.H / a.nkv;
     const int kst = hd + 8;                                   // padded K/V tile row (halves)
-    float *qs = (float *)smem;                                // [nq][hd]
-    uint16_t *kt = (uint16_t *)(qs + (size_t)nq * hd);        // [32][kst]
+    float *qs = (float *)smem;                                // [G][hd]
+    uint16_t *kt = (uint16_t *)(qs + (size_t)G * hd);         // [32][kst]
     uint16_t *vt = kt + 32 * kst;                             // [32][kst]
-    float *es = (float *)(vt + 32 * kst);                     // [nq][32]
-    uint32_t *vmask = (uint32_t *)(es + nq * 32);             // [nq]
-    const int pos = ctl->pos, kvh = blockIdx.y;
-    const int start0 = lg_win_start(pos, a.window), last_needed = pos + M - 1;
-    const int n = (start0 >> 5) + blockIdx.x;
-    if (n > (last_needed >> 5)) return;
+    float *es = (float *)(vt + 32 * kst);                     // [G][32]
+    uint32_t *vmask = (uint32_t *)(es + G * 32);              // [G]
+    const int kvh = blockIdx.y, j = blockIdx.z;
+    const int pos0 = ctl->pos, pj = pos0 + j;
+    const int startj = lg_win_start(pj, a.window);
+    const int n = (lg_win_start(pos0, a.window) >> 5) + blockIdx.x;
+    if (n < (startj >> 5) || n > (pj >> 5)) return;           // tile outside this row's keys
     const int t0 = n << 5;
-    // queries of this kv head's group, K/V tile rows
-    for (int idx = threadIdx.x; idx < nq * (hd >> 2); idx += LG_WG) {
-        const int qi = idx / (hd >> 2), e0 = (idx - qi * (hd >> 2)) << 2;
-        const int j = qi / G, head = kvh * G + qi % G;
-        *(float4 *)(qs + (size_t)qi * hd + e0) = *(const float4 *)(a.q + (size_t)j * a.H * hd + (size_t)head * hd + e0);
-    }
-    for (int idx = threadIdx.x; idx < 32 * (hd >> 3); idx += LG_WG) {
-        const int sl = idx / (hd >> 3), e0 = (idx - sl * (hd >> 3)) << 3;
-        const int t = t0 + sl;
-        uint4 kk = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-        if (t >= start0 && t <= last_needed) {
-            const size_t off = (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd + e0;
-            kk = *(const uint4 *)(a.kc + off);
-            vv = *(const uint4 *)(a.vc + off);
+    {   // stage q (G heads of this row) and the tile's K/V rows; loads are issued in groups ahead of
+        // the LDS stores (named temporaries + scheduling barrier, see lg_copy_batched)
+        const float *qrow = a.q + (size_t)j * a.H * hd + (size_t)kvh * G * hd;
+        lg_copy_batched<float4>((const float4 *)qrow, (float4 *)qs, G * (hd >> 2));
+        const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
+        for (int i0 = threadIdx.x; i0 < nk8; i0 += 4 * LG_WG) {
+            // element u of the batch: LDS offset (halves) in `lo`, cache offset in `go`, validity in `ok`
+            auto place = [&](int u, int &lo, size_t &go, bool &ok) {
+                const int idx = min(i0 + u * LG_WG, nk8 - 1);
+                const int sl = idx / per_row, e0 = (idx - sl * per_row) << 3, t = t0 + sl;
+                ok = t >= startj && t <= pj;
+                lo = sl * kst + e0;
+                go = (size_t)((ok ? t : pj) % a.seq) * a.kv_dim + (size_t)kvh * hd + e0;
+            };
+            int l0, l1, l2, l3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3;
+            place(0, l0, g0, ok0); place(1, l1, g1, ok1); place(2, l2, g2, ok2); place(3, l3, g3, ok3);
+            const uint4 k0 = a.kc4(g0), k1 = a.kc4(g1), k2 = a.kc4(g2), k3 = a.kc4(g3);
+            const uint4 v0 = a.vc4(g0), v1 = a.vc4(g1), v2 = a.vc4(g2), v3 = a.vc4(g3);
+            __builtin_amdgcn_sched_barrier(0);
+            auto keep = [](uint4 v, bool ok) {               // zero the rows no query of this block may see
+                const uint32_t mk = ok ? 0xFFFFFFFFu : 0u;
+                return make_uint4(v.x & mk, v.y & mk, v.z & mk, v.w & mk);
+            };
+            *(uint4 *)(kt + l0) = keep(k0, ok0);  *(uint4 *)(vt + l0) = keep(v0, ok0);
+            *(uint4 *)(kt + l1) = keep(k1, ok1);  *(uint4 *)(vt + l1) = keep(v1, ok1);
+            *(uint4 *)(kt + l2) = keep(k2, ok2);  *(uint4 *)(vt + l2) = keep(v2, ok2);
+            *(uint4 *)(kt + l3) = keep(k3, ok3);  *(uint4 *)(vt + l3) = keep(v3, ok3);
         }
-        *(uint4 *)(kt + sl * kst + e0) = kk;
-        *(uint4 *)(vt + sl * kst + e0) = vv;
     }
     __syncthreads();
-    // scores, tile max, exp, tile sum.  Thread = (key slot, query group of 8).
-    {
-        const int sl = threadIdx.x & 31, qg = threadIdx.x >> 5, t = t0 + sl;
-        for (int qi = qg; qi < nq; qi += LG_WG / 32) {
-            const int j = qi / G, pj = pos + j;
-            const bool valid = t >= lg_win_start(pj, a.window) && t <= pj;
-            float s = -INFINITY;
-            if (valid) {
-                const float *qv = qs + (size_t)qi * hd;
-                const uint16_t *kr = kt + sl * kst;
-                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-                for (int i = 0; i < hd; i += 8) {
-                    const float4 q4 = *(const float4 *)(qv + i), q5 = *(const float4 *)(qv + i + 4);
-                    const uint4 k4 = *(const uint4 *)(kr + i);
-                    a0 = lg_fmaf(q4.x, lg_h2f((uint16_t)(k4.x & 0xFFFF)), a0);
-                    a1 = lg_fmaf(q4.y, lg_h2f((uint16_t)(k4.x >> 16)), a1);
-                    a2 = lg_fmaf(q4.z, lg_h2f((uint16_t)(k4.y & 0xFFFF)), a2);
-                    a3 = lg_fmaf(q4.w, lg_h2f((uint16_t)(k4.y >> 16)), a3);
-                    a0 = lg_fmaf(q5.x, lg_h2f((uint16_t)(k4.z & 0xFFFF)), a0);
-                    a1 = lg_fmaf(q5.y, lg_h2f((uint16_t)(k4.z >> 16)), a1);
-                    a2 = lg_fmaf(q5.z, lg_h2f((uint16_t)(k4.w & 0xFFFF)), a2);
-                    a3 = lg_fmaf(q5.w, lg_h2f((uint16_t)(k4.w >> 16)), a3);
-                }
-                s = (a0 + a1) + (a2 + a3);
+    {   // scores, tile max, exp, tile sum
+        const int sl = threadIdx.x & 31, part = threadIdx.x >> 5, t = t0 + sl;
+        const bool valid = t >= startj && t <= pj;
+        for (int unit = part; unit < 2 * G; unit += LG_WG / 32) {
+            const int g = unit >> 1, hf = unit & 1;
+            const float *qv = qs + (size_t)g * hd + 2 * hf;
+            const uint16_t *kr = kt + sl * kst + 2 * hf;
+            float ax = 0.0f, ay = 0.0f;                       // chains 2hf and 2hf+1
+            for (int i = 0; i < hd; i += 8) {
+                const float2 q0 = *(const float2 *)(qv + i), q1 = *(const float2 *)(qv + i + 4);
+                const uint32_t k0 = *(const uint32_t *)(kr + i), k1 = *(const uint32_t *)(kr + i + 4);
+                ax = lg_fmaf(q0.x, lg_h2f((uint16_t)(k0 & 0xFFFF)), ax);
+                ay = lg_fmaf(q0.y, lg_h2f((uint16_t)(k0 >> 16)), ay);
+                ax = lg_fmaf(q1.x, lg_h2f((uint16_t)(k1 & 0xFFFF)), ax);
+                ay = lg_fmaf(q1.y, lg_h2f((uint16_t)(k1 >> 16)), ay);
             }
+            const float mine = ax + ay, other = __shfl_xor(mine, 32);
+            float s = hf ? other + mine : mine + other;       // (a0+a1) + (a2+a3)
+            if (!valid) s = -INFINITY;
             const float mx = lg_max_n(s, 32);
             const float e = valid ? lg_expf(s - mx) : 0.0f;
             const float l = lg_sum32(e);
             const unsigned long long bal = __ballot(valid);
             const uint32_t mask = (uint32_t)(threadIdx.x & 32 ? bal >> 32 : bal);
-            es[qi * 32 + sl] = e;
-            if (sl == 0) {
-                vmask[qi] = mask;
-                if (mask) {
-                    const int head = kvh * G + qi % G;
-                    const size_t pi = ((size_t)j * a.H + head) * a.tiles_max + blockIdx.x;
+            if (hf == 0) {
+                es[g * 32 + sl] = e;
+                if (sl == 0) {
+                    vmask[g] = mask;
+                    const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
                     a.pm[pi] = mx; a.pl[pi] = l;
                 }
             }
         }
     }
     __syncthreads();
-    // acc[d] = sum over valid slots of e * V[slot][d]
-    {
-        const int parts = hd >= LG_WG ? 1 : LG_WG / hd;       // thread groups splitting the queries
-        const int qpart = hd >= LG_WG ? 0 : threadIdx.x / hd;
-        for (int d = hd >= LG_WG ? threadIdx.x : threadIdx.x % hd; d < hd; d += LG_WG) {
-            for (int qi = qpart; qi < nq; qi += parts) {
-                const uint32_t mask = vmask[qi];
-                if (!mask) continue;
-                float acc = 0.0f;
-                #pragma unroll 8
-                for (int sl = 0; sl < 32; ++sl)
-                    if (mask >> sl & 1) acc = lg_fmaf(es[qi * 32 + sl], lg_h2f(vt[sl * kst + d]), acc);
-                const int j = qi / G, head = kvh * G + qi % G;
-                const size_t pi = ((size_t)j * a.H + head) * a.tiles_max + blockIdx.x;
-                a.pacc[pi * hd + d] = acc;
-            }
+    // acc[d] = sum over valid slots of e * V[slot][d]; thread = (head g, 4 dims)
+    for (int unit = threadIdx.x; unit < G * (hd >> 2); unit += LG_WG) {
+        const int g = unit / (hd >> 2), d0 = (unit - g * (hd >> 2)) << 2;
+        const uint32_t mask = vmask[g];
+        float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        #pragma unroll 8
+        for (int sl = 0; sl < 32; ++sl) {
+            if (!(mask >> sl & 1)) continue;
+            const float e = es[g * 32 + sl];
+            const uint2 v4 = *(const uint2 *)(vt + sl * kst + d0);
+            acc.x = lg_fmaf(e, lg_h2f((uint16_t)(v4.x & 0xFFFF)), acc.x);
+            acc.y = lg_fmaf(e, lg_h2f((uint16_t)(v4.x >> 16)), acc.y);
+            acc.z = lg_fmaf(e, lg_h2f((uint16_t)(v4.y & 0xFFFF)), acc.z);
+            acc.w = lg_fmaf(e, lg_h2f((uint16_t)(v4.y >> 16)), acc.w);
         }
+        const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
+        *(float4 *)(a.pacc + pi * hd + d0) = acc;
     }
 }
 

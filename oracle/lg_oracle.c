@@ -150,14 +150,15 @@ void lgo_matmul_f32(const void *w, uint32_t type, int k, int m, const float *x, 
 
 /* ---- rmsnorm: x * (1/sqrt(mean(x^2)+eps)) * w   (src/cpu/model-cpu.c:78-83,100-105).
  * tree = 0: serial sum like the reference CPU; tree = 1: this build's order
- * (64 lane partials, element i belongs to lane (i/4)%64, fma, adjacent tree). w may be NULL. */
+ * (256 lane partials, element i belongs to lane (i/4)%256, fma in ascending i, adjacent-pair
+ * tree over the lanes). w may be NULL. */
 void lgo_rmsnorm(float *out, const float *x, const float *w, int n, float eps, int tree) {
     float ss = 0.0f;
     if (!tree) for (int i = 0; i < n; i++) ss += x[i] * x[i];
     else {
-        float lane[64] = { 0 };
-        for (int i = 0; i < n; i++) lane[(i >> 2) & 63] = lg_fmaf(x[i], x[i], lane[(i >> 2) & 63]);
-        ss = tree_sum(lane, 64);
+        float lane[256] = { 0 };
+        for (int i = 0; i < n; i++) lane[(i >> 2) & 255] = lg_fmaf(x[i], x[i], lane[(i >> 2) & 255]);
+        ss = tree_sum(lane, 256);
     }
     float s = 1.0f / sqrtf(ss / (float)n + eps);
     if (w) for (int i = 0; i < n; i++) out[i] = x[i] * s * w[i];
