@@ -30,6 +30,23 @@
 // A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
 __host__ __device__ static inline int lg_segments(int k) { return (k >> 5) > 128 ? 32 : 8; }
 
+// Order of a q8 activation row in memory.  A matmul lane (row r, segment c) needs, at step `it`,
+// block c*nit + it of the row; lanes c = 0..S-1 therefore want blocks that lie nit apart.  Rows are
+// stored so that these are neighbours: the 16-byte unit w of the natural order (block b = w/2, half
+// = w%2) lives at unit it*2S + half*S + c, and the block's {scale,sum} pair at it*S + c, with
+// c = b / nit, it = b % nit.  A wavefront's LDS reads are then consecutive 16-byte units (no bank
+// conflicts), and producers write this order directly.
+struct ActLayout { int S, nit; };
+__host__ __device__ static inline ActLayout lg_act_layout(int k) { const int S = lg_segments(k); return { S, (k >> 5) / S }; }
+__host__ __device__ static inline int lg_act_unit(ActLayout a, int w) {
+    const int b = w >> 1, c = b / a.nit, it = b - c * a.nit;
+    return it * 2 * a.S + (w & 1) * a.S + c;
+}
+__host__ __device__ static inline int lg_act_block(ActLayout a, int b) {
+    const int c = b / a.nit, it = b - c * a.nit;
+    return it * a.S + c;
+}
+
 // Cross-lane exchange for the reductions.  Within a row of 16 lanes DPP moves data in one VALU
 // instruction; the partner patterns (swap inside pairs, swap pairs inside quads, mirror 8, mirror
 // 16) differ from xor-butterflies only in which lane of the already-uniform sub-group supplies the

@@ -123,8 +123,7 @@ struct lg_hip_model {
     // scratch
     float *x[2] = { nullptr, nullptr }, *qkv = nullptr, *dout = nullptr, *pmp_raw = nullptr, *hidden_rows = nullptr,
           *g_hidden = nullptr, *logits = nullptr, *pval = nullptr, *q_rot = nullptr;
-    int8_t *aq = nullptr, *gq = nullptr, *pq = nullptr, *hq = nullptr;
-    float2 *ads = nullptr, *gds = nullptr, *pds = nullptr, *hds = nullptr;
+    int8_t *aq = nullptr, *gq = nullptr, *pq = nullptr, *hq = nullptr;     // q8 activation buffers (values + {scale,sum})
     int *pidx = nullptr;
     StepCtl *ctl = nullptr;
     int32_t *sched = nullptr, *out = nullptr, *adv = nullptr;
@@ -370,13 +369,11 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     const size_t R = (size_t)max_rows;
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
         dev_alloc(m, &m->dout, R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
-        dev_alloc(m, &m->aq, R * max_qd) || dev_alloc(m, &m->ads, R * max_qd / 32) ||
-        dev_alloc(m, &m->gq, R * max_ff) || dev_alloc(m, &m->gds, R * max_ff / 32) ||
-        dev_alloc(m, &m->hq, R * E) || dev_alloc(m, &m->hds, R * E / 32) ||
+        dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4) ||
         dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
         dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
-    if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple) || dev_alloc(m, &m->pds, R * m->ple / 32)))
+    if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4)))
         return -7;
     HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
     HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
@@ -584,7 +581,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
     auto rows = [&](const float *w_pre, float *h_out) {
         RowArgs s{};
-        s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq; s.ds = m->hds;
+        s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq;
         if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os;
@@ -597,7 +594,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
 
     if (m->ple) {
         rows(nullptr, nullptr);
-        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, m->hds, nullptr };
+        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, nullptr };
         launch_mm<M, false>(lx, KC_PMP, a);
     }
     for (int L = 0; L < nl && !lx.rc; ++L) {
@@ -605,7 +602,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         const int window = (y.is_local && m->window > 0) ? m->window : 0;
         rows(y.attn_norm, nullptr);
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
-            MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, m->hds, nullptr };
+            MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
             launch_mm<M, false>(lx, KC_QKV, a);
             QkvPostArgs p{};
             p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
@@ -624,41 +621,43 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max;
             const size_t lds = (size_t)G * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
             LAUNCH(KC_ATTN, lg_k_attn, dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), lds, a, m->ctl);
-            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, m->aq, m->ads, nullptr };
+            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, m->aq, nullptr };
             LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
         {   // attention output projection
-            MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, m->ads, nullptr };
+            MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, nullptr };
             launch_mm<M, false>(lx, KC_O, a);
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
         }
         {   // feed-forward: gate/up + GeGLU, then down
             rows(y.ffn_norm, nullptr);
-            GegluArgs a{ y.wgu, E, y.nff, m->hq, m->hds, m->gq, m->gds };
-            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M>), dim3(y.nff / 32), dim3(LG_WG), lds_mm(M, E), a);
-            MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, m->gds, nullptr };
+            GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
+            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M, 4>), dim3(y.nff / 32), dim3(256), lds_mm(M, E), a);
+            MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
             launch_mm<M, false>(lx, KC_DOWN, d);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
         }
         if (m->ple) {   // per-layer embedding block
             rows(nullptr, nullptr);
             PleGateArgs a{};
-            a.w = y.winp; a.k = E; a.ple = m->ple; a.q_in = m->hq; a.ds_in = m->hds;
+            a.w = y.winp; a.k = E; a.ple = m->ple; a.q_in = m->hq;
             a.pmp_raw = m->pmp_raw; a.layer = L; a.n_layer = nl;
             a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
             a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
-            a.pq = m->pq; a.pds = m->pds;
+            a.pq = m->pq;
             LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E), a, m->ctl);
-            MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, m->pds, nullptr };
+            MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, nullptr };
             launch_mm<M, false>(lx, KC_PLEPROJ, p);
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
         }
     }
     if (with_head && !lx.rc) {
         rows(m->output_norm, m->hidden_rows);
-        const int passes = 4;
-        const int grid = (m->n_vocab / 8 + passes * 8 - 1) / (passes * 8);
-        HeadArgs h{ m->emb, E, m->n_vocab, passes, m->hq, m->hds, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
+        int grid = 512;                                  // two workgroups per CU, each walks `passes` blocks of 64 rows
+        int passes = (m->n_vocab / 64 + grid - 1) / grid;
+        if (passes < 1) passes = 1;
+        grid = (m->n_vocab / 64 + passes - 1) / passes;
+        HeadArgs h{ m->emb, E, m->n_vocab, passes, m->hq, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
         LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(grid), dim3(LG_WG), lds_mm(M, E), h);
         AcceptArgs c{ m->pval, m->pidx, grid, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
         LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), dim3(LG_WG), 0, c, m->ctl);
@@ -905,10 +904,10 @@ struct Scratch {            // device buffers freed on scope exit
 
 template <int M>
 static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, const float *dx, float *dout, int32_t *ddots,
-                       int8_t *dq, float2 *dds, StepCtl *, int repeats, float *kernel_ms) {
+                       int8_t *dq, int repeats, float *kernel_ms) {
     const int n32 = M * (k / 32);
-    hipLaunchKernelGGL(lg_k_quant_flat, dim3((n32 * 8 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, st, dx, n32, dq, dds);
-    MmArgs a{ dw, k, mrows, dout, dq, dds, ddots };
+    hipLaunchKernelGGL(lg_k_quant_flat, dim3((n32 * 8 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, st, dx, M, k, dq);
+    MmArgs a{ dw, k, mrows, dout, dq, ddots };
     lg_hip_model shim;                       // the launcher only needs a stream and the profiling switch
     shim.stream = st;
     Launcher lx{ &shim, false };
@@ -941,17 +940,16 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     int rc = lg_hip_repack_q4_0(w, k, mrows, tiled.data());
     if (rc) return rc;
     Scratch sc;
-    uint8_t *dw; float *dx, *dout; int32_t *ddots = nullptr; int8_t *dq; float2 *dds; StepCtl *ctl;
+    uint8_t *dw; float *dx, *dout; int32_t *ddots = nullptr; int8_t *dq;
     if (sc.get(&dw, tiled.size()) || sc.get(&dx, (size_t)rows * k) || sc.get(&dout, (size_t)rows * mrows) ||
-        sc.get(&dq, (size_t)rows * k) || sc.get(&dds, (size_t)rows * nb) || sc.get(&ctl, (size_t)1)) return -7;
+        sc.get(&dq, (size_t)rows * k * 5 / 4)) return -7;
     if (dots && sc.get(&ddots, (size_t)rows * mrows * nb)) return -7;
     HIP_TRY(hipMemcpy(dw, tiled.data(), tiled.size(), hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(dx, x, (size_t)rows * k * 4, hipMemcpyHostToDevice));
-    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
     hipStream_t st;
     HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
     switch (rows) {
-#define CASE(M) case M: rc = matmul_rows<M>(st, dw, k, mrows, dx, dout, ddots, dq, dds, ctl, repeats, kernel_ms); break;
+#define CASE(M) case M: rc = matmul_rows<M>(st, dw, k, mrows, dx, dout, ddots, dq, repeats, kernel_ms); break;
         CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
 #undef CASE
     }
@@ -959,14 +957,23 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     if (rc) return rc;
     if (out) HIP_TRY(hipMemcpy(out, dout, (size_t)rows * mrows * 4, hipMemcpyDeviceToHost));
     if (dots) HIP_TRY(hipMemcpy(dots, ddots, (size_t)rows * mrows * nb * 4, hipMemcpyDeviceToHost));
-    if (xq) HIP_TRY(hipMemcpy(xq, dq, (size_t)rows * k, hipMemcpyDeviceToHost));
+    // the device keeps activation rows in the matmul's own order (lg_act_layout); hand them back in natural order
+    const ActLayout lay = lg_act_layout(k);
+    if (xq) {
+        std::vector<int8_t> dev((size_t)rows * k);
+        HIP_TRY(hipMemcpy(dev.data(), dq, dev.size(), hipMemcpyDeviceToHost));
+        for (int j = 0; j < rows; ++j)
+            for (int w = 0; w < k / 16; ++w) memcpy(xq + (size_t)j * k + (size_t)w * 16, dev.data() + (size_t)j * k + (size_t)lg_act_unit(lay, w) * 16, 16);
+    }
     if (xd || xsum) {
         std::vector<float2> ds((size_t)rows * nb);
-        HIP_TRY(hipMemcpy(ds.data(), dds, ds.size() * 8, hipMemcpyDeviceToHost));
-        for (size_t i = 0; i < ds.size(); ++i) {
-            if (xd) xd[i] = ds[i].x;
-            if (xsum) memcpy(&xsum[i], &ds[i].y, 4);
-        }
+        HIP_TRY(hipMemcpy(ds.data(), dq + (size_t)rows * k, ds.size() * 8, hipMemcpyDeviceToHost));
+        for (int j = 0; j < rows; ++j)
+            for (int b = 0; b < nb; ++b) {
+                const float2 v = ds[(size_t)j * nb + lg_act_block(lay, b)];
+                if (xd) xd[(size_t)j * nb + b] = v.x;
+                if (xsum) memcpy(&xsum[(size_t)j * nb + b], &v.y, 4);
+            }
     }
     return 0;
 }
@@ -1007,11 +1014,11 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     const int start0 = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     const int tiles = ((pos + rows - 1) >> 5) - (start0 >> 5) + 1;
     Scratch sc;
-    float *dq, *dpm, *dpl, *dpacc, *dxf; uint16_t *dk, *dv; int8_t *dxq; float2 *dxds; StepCtl *ctl;
+    float *dq, *dpm, *dpl, *dpacc, *dxf; uint16_t *dk, *dv; int8_t *dxq; StepCtl *ctl;
     const size_t slots = (size_t)rows * n_head * tiles;
     if (sc.get(&dq, (size_t)rows * qd) || sc.get(&dk, (size_t)seq * kd) || sc.get(&dv, (size_t)seq * kd) ||
         sc.get(&dpm, slots) || sc.get(&dpl, slots) || sc.get(&dpacc, slots * hd) || sc.get(&dxf, (size_t)rows * qd) ||
-        sc.get(&dxq, (size_t)rows * qd) || sc.get(&dxds, (size_t)rows * qd / 32) || sc.get(&ctl, (size_t)1)) return -7;
+        sc.get(&dxq, (size_t)rows * qd * 5 / 4) || sc.get(&ctl, (size_t)1)) return -7;
     HIP_TRY(hipMemcpy(dq, q, (size_t)rows * qd * 4, hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(dk, kc, (size_t)seq * kd * 2, hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(dv, vc, (size_t)seq * kd * 2, hipMemcpyHostToDevice));
@@ -1021,7 +1028,7 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     a.q = dq; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
     a.kc = dk; a.vc = dv; a.seq = seq; a.kv_dim = kd; a.window = window;
     a.pm = dpm; a.pl = dpl; a.pacc = dpacc; a.tiles_max = tiles;
-    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, dxq, dxds, dxf };
+    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, dxq, dxf };
     hipStream_t st;
     HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
     int rc = 0;

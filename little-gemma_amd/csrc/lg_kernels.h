@@ -35,8 +35,7 @@ struct RowArgs {
     float         *h_out;    // [M][E] normed rows before quantization, or nullptr
     const uint8_t *emb;      // tiled token_embd: rows are token lookups scaled by emb_scale
     const int32_t *toks;     // token schedule base ([n_steps][M])
-    int8_t        *q;        // [M][E] q8 values
-    float2        *ds;       // [M][E/32] {scale, sum}
+    int8_t        *q;        // q8 activation buffer: [M][E] values, then [M][E/32] {scale, sum}
     int            emb_nit, emb_seg;
     float          emb_scale;
     int            E;
@@ -52,6 +51,13 @@ __device__ __forceinline__ float lg_block_sum256(float v, float *scratch4) {
     return (scratch4[0] + scratch4[1]) + (scratch4[2] + scratch4[3]);
 }
 
+// A q8 activation buffer holds the M rows of int8 values ([M][k], order of lg_act_layout(k))
+// immediately followed by their per-32 {scale, sum} pairs ([M][k/32] float2): one contiguous
+// region of M*k*5/4 bytes, copied to LDS in one go.
+template <int M>
+__device__ __forceinline__ const float2 *lg_q8_ds(const int8_t *q, int k) { return (const float2 *)(q + (size_t)M * k); }
+template <int M>
+__device__ __forceinline__ float2 *lg_q8_ds(int8_t *q, int k) { return (float2 *)(q + (size_t)M * k); }
 #define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
@@ -123,28 +129,34 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ho[t + 256 * v] = xv[v];
     }
     uint32_t *qrow = (uint32_t *)(s.q + (size_t)j * E);
-    float2 *drow = s.ds + (size_t)j * (E >> 5);
+    float2 *drow = lg_q8_ds<M>(s.q, E) + (size_t)j * (E >> 5);
+    const ActLayout lay = lg_act_layout(E);
     #pragma unroll
     for (int v = 0; v < LG_ROWV; ++v) {
         // nq is a multiple of 64, so a whole wavefront is either inside the row or outside it
         if (t + 256 * v >= nq) break;
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
-        qrow[t + 256 * v] = packed;
-        if ((t & 7) == 0) drow[(t + 256 * v) >> 3] = make_float2(d, __int_as_float(sum));
+        const int quad = t + 256 * v;                        // 4 values = a quarter of a 16-byte unit
+        qrow[lg_act_unit(lay, quad >> 2) * 4 + (quad & 3)] = packed;
+        if ((t & 7) == 0) drow[lg_act_block(lay, quad >> 3)] = make_float2(d, __int_as_float(sum));
     }
 }
 
-// Plain q8 quantization of n32 groups of 32 floats (no norm): 8 lanes per group.
-__global__ __launch_bounds__(LG_WG) void lg_k_quant_flat(const float *x, int n32, int8_t *q, float2 *ds) {
-    const int g = (blockIdx.x * LG_WG + threadIdx.x) >> 3, l = threadIdx.x & 7;
-    const bool live = g < n32;
+// Plain q8 quantization of rows x k floats (no norm): 8 lanes per group of 32, output in the
+// activation row order of lg_act_layout(k).
+__global__ __launch_bounds__(LG_WG) void lg_k_quant_flat(const float *x, int rows, int k, int8_t *q) {
+    float2 *ds = (float2 *)(q + (size_t)rows * k);
+    const int g = (blockIdx.x * LG_WG + threadIdx.x) >> 3, l = threadIdx.x & 7, nb = k >> 5;
+    const bool live = g < rows * nb;
     const float4 h = live ? ((const float4 *)x)[(size_t)g * 8 + l] : make_float4(0, 0, 0, 0);
     float d; int sum;
     const uint32_t packed = lg_quant4_8lanes(h, &d, &sum);
     if (!live) return;
-    ((uint32_t *)q)[(size_t)g * 8 + l] = packed;
-    if (l == 0) ds[g] = make_float2(d, __int_as_float(sum));
+    const int j = g / nb, b = g - j * nb;
+    const ActLayout lay = lg_act_layout(k);
+    ((uint32_t *)(q + (size_t)j * k))[lg_act_unit(lay, b * 2 + (l >> 2)) * 4 + (l & 3)] = packed;
+    if (l == 0) ds[(size_t)j * nb + lg_act_block(lay, b)] = make_float2(d, __int_as_float(sum));
 }
 
 // Copy M already-quantized rows (int8 + {scale,sum}) from global memory into LDS.
@@ -165,9 +177,8 @@ __device__ __forceinline__ void lg_copy_batched(const T *src, T *dst, int n) {
     }
 }
 template <int M>
-__device__ __forceinline__ void lg_load_q8(const int8_t *q, const float2 *ds, int k, int8_t *lq, float2 *lds_ds) {
-    lg_copy_batched<uint4>((const uint4 *)q, (uint4 *)lq, M * k / 16);
-    lg_copy_batched<float2>(ds, lds_ds, M * (k >> 5));
+__device__ __forceinline__ void lg_load_q8(const int8_t *q, int k, int8_t *lq) {
+    lg_copy_batched<uint4>((const uint4 *)q, (uint4 *)lq, M * k * 5 / 64);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -212,11 +223,12 @@ __device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChu
         #pragma unroll
         for (int u = 0; u < LG_U; ++u) {
             if (it0 + u >= nit) break;
-            const int b = c * nit + it0 + u;
+            const int it = it0 + u, b = c * nit + it;        // b: block of the natural order (for DUMP)
             #pragma unroll
             for (int j = 0; j < M; ++j) {
-                const float2 ds = actds[j * nb + b];
-                const int4 a0 = *(const int4 *)(act + (size_t)j * k + b * 32), a1 = *(const int4 *)(act + (size_t)j * k + b * 32 + 16);
+                const float2 ds = actds[j * nb + it * S + c];
+                const int8_t *au = act + (size_t)j * k + (size_t)(it * 2 * S + c) * 16;
+                const int4 a0 = *(const int4 *)au, a1 = *(const int4 *)(au + S * 16);
                 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     const int dot = lg_block_dot(cur.q[g][u], a0, a1, __float_as_int(ds.y));
@@ -247,8 +259,7 @@ struct MmArgs {
     const uint8_t *w;        // tiled weights
     int            k, m;     // row length, rows
     float         *out;      // [M][m]
-    const int8_t  *q_in;     // [M][k] q8 input rows
-    const float2  *ds_in;    // [M][k/32]
+    const int8_t  *q_in;     // q8 activation buffer of the M input rows
     int32_t       *dots;     // DUMP only: [M][m][k/32]
 };
 
@@ -273,7 +284,7 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm(MmArgs a) {
     }
     WChunk<G> first;
     lg_mm_fetch<G>(first, wg, 0, nit, lane);
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    lg_load_q8<M>(a.q_in, a.k, lq);
     __syncthreads();
     if (g0 >= ngroups) return;
     float acc[G][M];
@@ -292,36 +303,52 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm(MmArgs a) {
 struct GegluArgs {
     const uint8_t *w;        // tiled [2*n_ff][k], virtual row order: 32 gate, 32 up, 32 gate, ...
     int            k, n_ff;
-    const int8_t  *q_in; const float2 *ds_in;
-    int8_t        *gq;       // [M][n_ff]
-    float2        *gds;      // [M][n_ff/32]
+    const int8_t  *q_in;
+    int8_t        *gq;       // q8 activation buffer of the result, width n_ff
 };
-template <int M>
-__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_geglu(GegluArgs a) {
+// WV = 4: wavefront w computes gate AND up rows 8w..8w+7 (shared activation loads);
+// WV = 8: wavefronts 0-3 compute the gate rows, 4-7 the up rows (twice the wavefronts per CU to
+// hide latency, at the price of reading the activations twice from LDS).
+template <int M, int WV>
+__global__ __launch_bounds__(64 * WV, 2) void lg_k_mm_geglu(GegluArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
-    __shared__ float gbuf[LG_HIP_MAX_ROWS_DEV][32];
+    __shared__ float gbuf[2][LG_HIP_MAX_ROWS_DEV][32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
     const int t = blockIdx.x;                               // 32-wide slice of n_ff
     const size_t gstride = (size_t)nit * LG_TILE;
-    const uint8_t *wg[2] = { a.w + ((size_t)t * 8 + wave) * gstride, a.w + ((size_t)t * 8 + 4 + wave) * gstride };
-    const int row[2] = { 0, 0 };
-    WChunk<2> first;
-    lg_mm_fetch<2>(first, wg, 0, nit, lane);
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
-    __syncthreads();
-    float acc[2][M];
-    lg_mm_groups<M, 8, 2, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
     const int c = lane & 7, r = lane >> 3;
-    if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * lg_pick<M>(acc[1], c);
+    if (WV == 4) {
+        const uint8_t *wg[2] = { a.w + ((size_t)t * 8 + wave) * gstride, a.w + ((size_t)t * 8 + 4 + wave) * gstride };
+        const int row[2] = { 0, 0 };
+        WChunk<2> first;
+        lg_mm_fetch<2>(first, wg, 0, nit, lane);
+        lg_load_q8<M>(a.q_in, a.k, lq);
+        __syncthreads();
+        float acc[2][M];
+        lg_mm_groups<M, 8, 2, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
+        if (c < M) gbuf[0][c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * lg_pick<M>(acc[1], c);
+    } else {
+        const uint8_t *wg[1] = { a.w + ((size_t)t * 8 + wave) * gstride };      // groups 0-3 gate, 4-7 up
+        const int row[1] = { 0 };
+        WChunk<1> first;
+        lg_mm_fetch<1>(first, wg, 0, nit, lane);
+        lg_load_q8<M>(a.q_in, a.k, lq);
+        __syncthreads();
+        float acc[1][M];
+        lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
+        if (c < M) gbuf[wave >> 2][c][(wave & 3) * 8 + r] = lg_pick<M>(acc[0], c);
+    }
     __syncthreads();
-    for (int j = threadIdx.x >> 5; j < M; j += LG_WG / 32) {       // half-wavefront per row, one value per lane
+    for (int j = threadIdx.x >> 5; j < M; j += 2 * WV) {         // half-wavefront per row, one value per lane
         const int i = threadIdx.x & 31;
+        const float g = WV == 4 ? gbuf[0][j][i] : lg_gelu(gbuf[0][j][i]) * gbuf[1][j][i];
         float d; int sum;
-        const int q = lg_quant1_32lanes(gbuf[j][i], &d, &sum);
-        a.gq[(size_t)j * a.n_ff + t * 32 + i] = (int8_t)q;
-        if (i == 0) a.gds[(size_t)j * (a.n_ff >> 5) + t] = make_float2(d, __int_as_float(sum));
+        const int q = lg_quant1_32lanes(g, &d, &sum);
+        const ActLayout lay = lg_act_layout(a.n_ff);          // order the ffn_down matmul reads
+        a.gq[(size_t)j * a.n_ff + lg_act_unit(lay, t * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
+        if (i == 0) lg_q8_ds<M>(a.gq, a.n_ff)[(size_t)j * (a.n_ff >> 5) + lg_act_block(lay, t)] = make_float2(d, __int_as_float(sum));
     }
 }
 
@@ -332,15 +359,14 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_geglu(GegluArgs a) {
 struct PleGateArgs {
     const uint8_t *w;        // tiled inp_gate [ple][E]
     int            k, ple;
-    const int8_t  *q_in; const float2 *ds_in;
+    const int8_t  *q_in;
     const float   *pmp_raw;  // [M][n_layer*ple] raw projection
     int            layer, n_layer;
     const float   *proj_norm;     // [ple]
     const uint8_t *pte;      // per_layer_token_embd, plain q4_0 rows of n_layer*ple
     const int32_t *toks;
     float          pscale, tscale, rsqrt2, eps;
-    int8_t        *pq;       // [M][ple]
-    float2        *pds;      // [M][ple/32]
+    int8_t        *pq;       // q8 activation buffer of the result, width ple
 };
 template <int M>
 __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const StepCtl *ctl) {
@@ -369,7 +395,7 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const
         const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
         if (lane < 32) ipl[j][lane] = (pe * a.pscale * sc * wn + tk) * a.rsqrt2;
     }
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    lg_load_q8<M>(a.q_in, a.k, lq);
     __syncthreads();
     float acc[1][M];
     lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
@@ -380,8 +406,9 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const
         const int i = threadIdx.x & 31;
         float d; int sum;
         const int q = lg_quant1_32lanes(gbuf[j][i], &d, &sum);
-        a.pq[(size_t)j * ple + blockIdx.x * 32 + i] = (int8_t)q;
-        if (i == 0) a.pds[(size_t)j * (ple >> 5) + blockIdx.x] = make_float2(d, __int_as_float(sum));
+        const ActLayout lay = lg_act_layout(ple);
+        a.pq[(size_t)j * ple + lg_act_unit(lay, blockIdx.x * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
+        if (i == 0) lg_q8_ds<M>(a.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, blockIdx.x)] = make_float2(d, __int_as_float(sum));
     }
 }
 
@@ -391,7 +418,7 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const
 // workgroup and row goes to global memory.
 struct HeadArgs {
     const uint8_t *w; int k, n_vocab, passes;
-    const int8_t *q_in; const float2 *ds_in;
+    const int8_t *q_in;
     float softcap;
     float *logits;          // [M][n_vocab] or nullptr
     float *pval; int *pidx; // [gridDim.x][M]
@@ -403,7 +430,7 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_head(HeadArgs a) {
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
     __shared__ float sv[4][LG_HIP_MAX_ROWS_DEV];
     __shared__ int si[4][LG_HIP_MAX_ROWS_DEV];
-    lg_load_q8<M>(a.q_in, a.ds_in, a.k, lq, lds);
+    lg_load_q8<M>(a.q_in, a.k, lq);
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
     const int c = lane & 7, r = lane >> 3, ngroups = a.n_vocab >> 3;
@@ -700,7 +727,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
 struct MergeArgs {
     const float *pm, *pl, *pacc; int tiles_max;
     int H, hd, window;
-    int8_t *xq; float2 *xds;   // [M][H*hd] q8 of the attention output (input of attn_output)
+    int8_t *xq;                // q8 activation buffer of the attention output, width H*hd (input of attn_output)
     float *xf;                 // optional f32 copy [M][H*hd]
 };
 template <int M>
@@ -754,10 +781,11 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
         float dq; int sum;
         const int q = lg_quant1_32lanes(r, &dq, &sum);
         if (d < hd) {
-            const size_t e = (size_t)j * qd + (size_t)head * hd + d;
-            a.xq[e] = (int8_t)q;
-            if ((d & 31) == 0) a.xds[e >> 5] = make_float2(dq, __int_as_float(sum));
-            if (a.xf) a.xf[e] = r;
+            const int e = head * hd + d;                       // element of the row, natural order
+            const ActLayout lay = lg_act_layout(qd);          // order the attn_output matmul reads
+            a.xq[(size_t)j * qd + lg_act_unit(lay, e >> 4) * 16 + (e & 15)] = (int8_t)q;
+            if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[(size_t)j * (qd >> 5) + lg_act_block(lay, e >> 5)] = make_float2(dq, __int_as_float(sum));
+            if (a.xf) a.xf[(size_t)j * qd + e] = r;
         }
     }
 }
