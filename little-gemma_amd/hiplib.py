@@ -36,7 +36,7 @@ def build():
     """Compile the HIP library for gfx950 and the C backend on top of it."""
     subprocess.run(["make", "-C", CSRC, "-B", "liblg_hip.so"], check=True, stdout=subprocess.DEVNULL,
                    stderr=subprocess.DEVNULL)
-    subprocess.run(["make", "-C", HOST, "-B", "liblg_host.so", "liblg_modelhip.so"], check=True,
+    subprocess.run(["make", "-C", HOST, "-B", "liblg_host.so", "liblg_modelhip.so", "run-hip"], check=True,
                    stdout=subprocess.DEVNULL)
 
 

@@ -14,11 +14,12 @@
  *   lgo_forward(LGO_REF)           bit-identical logits and tokens against the reference's own CPU
  *                                  backend built from its sources (oracle/_ref), and against the
  *                                  committed fixtures those runs produced (tests/golden)
- *   lgo_forward(LGO_I8 / _LIBM)    built from the pinned primitives above; the reference's CUDA int8 path
- *                                  it restates cannot run without an NVIDIA device, so the composition
- *                                  (quantization points, op order) is pinned by agreement with LGO_REF
- *                                  when quantization is made lossless (test_i8_reduces_to_ref) and by
- *                                  the measured LGO_REF gap staying inside the q8 noise band.
+ *   lgo_forward(LGO_I8 / _LIBM)    built from the pinned primitives above.  The reference's CUDA int8 path
+ *                                  it restates cannot run without an NVIDIA device: PARITY UNPINNED for the
+ *                                  last bits of its float sums (this file fixes its own summation orders).
+ *                                  The composition (quantization points, op order) is held by the measured
+ *                                  gap to LGO_REF staying inside the q8 noise band and by spec == decode
+ *                                  (tests/test_oracle_model.py).
  */
 #define _GNU_SOURCE
 #include <stdio.h>
