@@ -95,6 +95,25 @@ int  lg_hip_get_logits(lg_hip_model *m, int row, float *dst);
 /* Options: "store_logits" (0/1, default 0), "use_graph" (0/1, default 1). */
 int  lg_hip_set_option(lg_hip_model *m, const char *name, int value);
 
+/* ---- draft head: the gemma4-assistant network on the device (mtp_draft_device,
+ * mtp_draft_chain_device, mtp_free_device: src/mtp-internal.h:33-37, src/cuda/mtp-kernel.cuh:272-402).
+ * A head is a model object whose blocks own no cache: block L cross-attends the target's last
+ * sliding (n_kv_start-2) or last global (n_kv_start-1) cache layer (src/mtp.c:173-176,193-201).
+ * cfg: n_embd = the head's inner width, n_head_kv[L] / head_dim[L] / is_local[L] = those of the
+ * target layer the block reads, n_kv_start and n_embd_per_layer = 0, sliding_window ignored (the
+ * target's is used).  Tensors go through lg_hip_model_tensor under their GGUF names, the two
+ * next-token projections as "pre_projection.weight" (2*n_embd(target) -> inner) and
+ * "post_projection.weight" (inner -> n_embd(target), optional: without it drafts cannot chain);
+ * then lg_hip_model_commit(head, 1).  Destroy with lg_hip_model_destroy before the target. */
+int  lg_hip_draft_create(lg_hip_model *target, const struct lg_hip_config *cfg, lg_hip_model **out);
+/* One draft: the token the head expects after `token`, where `token` will sit at position pos
+ * and the target cache holds the positions before it.  chain = 0: h_prev is the target's hidden
+ * state of the last accepted row (lg_hip_get_hidden(target)); chain = 1: h_prev is the post-
+ * projection of this head's own hidden from its previous draft.  One captured graph per call
+ * and a 4-byte read-back, like the reference.  lg_hip_get_hidden(head) afterwards returns the
+ * head's post-norm hidden (inner width); lg_hip_get_logits(head, 0) its logits when stored. */
+int  lg_hip_draft_step(lg_hip_model *head, lg_hip_kv *target_kv, int token, int pos, int chain, int32_t *tok_out);
+
 /* ---- device-resident stepping: the same step with no host round trip between steps.
  * A schedule is n_steps blocks of n_rows tokens built by the caller (drafts come from a draft
  * head or, in the benchmark, are prepared in advance); each step verifies block `step`, writes

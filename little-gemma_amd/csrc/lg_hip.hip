@@ -133,6 +133,13 @@ struct lg_hip_model {
     int store_logits = 0, use_graph = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
+    // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
+    lg_hip_model *target = nullptr;
+    std::vector<lg_hip_model *> drafts;      // heads attached to this (target) model
+    uint8_t *w_pre = nullptr, *w_post = nullptr;         // next-token pre / post projections, tiled
+    int8_t *catq = nullptr;                  // q8 of [embedding(token) * sqrt(nb), h_prev], width 2*nb
+    float *hprev = nullptr;                  // post-projection of the previous draft's hidden (chained drafts)
+    bool draft_chain = false;
 };
 
 struct lg_hip_kv {
@@ -182,7 +189,8 @@ extern "C" int lg_hip_model_tensor(lg_hip_model *m, const char *name, uint32_t t
     if (!m || !name || !dims || !data || n_dims < 1 || n_dims > 4) return fail(-1, "model_tensor: bad argument");
     if (m->committed) return fail(-4, "model_tensor: model already committed");
     static const char *top[] = { "token_embd.weight", "output_norm.weight", "rope_freqs.weight",
-                                 "per_layer_token_embd.weight", "per_layer_model_proj.weight", "per_layer_proj_norm.weight" };
+                                 "per_layer_token_embd.weight", "per_layer_model_proj.weight", "per_layer_proj_norm.weight",
+                                 "pre_projection.weight", "post_projection.weight" };
     bool known = !strncmp(name, "blk.", 4);
     for (const char *t : top) known = known || !strcmp(name, t);
     if (!known) return 1;
@@ -302,9 +310,16 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (y.nkv <= 0 || H % y.nkv || H / y.nkv > 8) return fail(-2, "model_commit: layer %d: %d query heads per kv head (at most 8 are built)", L, H / y.nkv);
         if (y.nff % 32) return fail(-2, "model_commit: layer %d feed-forward width %d must be a multiple of 32", L, y.nff);
         y.qd = H * y.hd; y.kd = y.nkv * y.hd;
-        y.owns = L < m->n_kv_start;
-        y.src = y.owns ? L : m->n_kv_start - (y.is_local ? 2 : 1);          // src/cpu/model-cpu.c:175-179
+        y.owns = !m->target && L < m->n_kv_start;
+        const int kv_start = m->target ? m->target->n_kv_start : m->n_kv_start;
+        y.src = y.owns ? L : kv_start - (y.is_local ? 2 : 1);               // src/cpu/model-cpu.c:175-179, src/mtp.c:173-176
         if (y.src < 0) return fail(-2, "model_commit: layer %d has no layer to share KV with", L);
+        if (m->target) {
+            const Layer &t = m->target->L[y.src];
+            if (t.hd != y.hd || t.nkv != y.nkv || (t.is_local != 0) != (y.is_local != 0))
+                return fail(-2, "model_commit: draft block %d (head size %d, %d kv heads, %s) does not match the target layer %d it reads",
+                            L, y.hd, y.nkv, y.is_local ? "sliding" : "global", y.src);
+        }
         const HostTensor *q = find(m, lname(L, "attn_q.weight")), *k = find(m, lname(L, "attn_k.weight")),
                          *v = find(m, lname(L, "attn_v.weight"));
         if ((rc = check_mat(q, lname(L, "attn_q.weight"), E, y.qd))) return rc;
@@ -365,6 +380,22 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (y.nff > max_ff) max_ff = y.nff;
         if (y.qd > max_qd) max_qd = y.qd;
     }
+    if (m->target) {
+        const int nb = m->target->E;
+        const HostTensor *pre = find(m, "pre_projection.weight"), *post = find(m, "post_projection.weight");
+        if ((rc = check_mat(pre, "pre_projection.weight", 2 * (uint64_t)nb, E))) return rc;
+        std::vector<const uint8_t *> rows;
+        push_rows(rows, pre, 0, E);
+        if ((rc = upload_tiled(m, rows, 2 * nb, &m->w_pre, stage))) return rc;
+        if (post) {                                                 // optional: without it drafts cannot chain
+            if ((rc = check_mat(post, "post_projection.weight", E, nb))) return rc;
+            rows.clear();
+            push_rows(rows, post, 0, nb);
+            if ((rc = upload_tiled(m, rows, E, &m->w_post, stage))) return rc;
+        }
+        if (dev_alloc(m, &m->catq, (size_t)2 * nb * 5 / 4) || dev_alloc(m, &m->hprev, (size_t)nb)) return -7;
+        if (max_rows != 1) return fail(-2, "model_commit: a draft head runs one row at a time");
+    }
     m->host.clear();
     const size_t R = (size_t)max_rows;
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
@@ -395,7 +426,11 @@ extern "C" void lg_hip_model_destroy(lg_hip_model *m) {
     for (void *p : m->allocs) (void)hipFree(p);
     for (hipEvent_t e : m->prof.ev) (void)hipEventDestroy(e);
     if (m->pin) (void)hipHostFree(m->pin);
-    if (m->stream) (void)hipStreamDestroy(m->stream);
+    if (m->target) {
+        auto &v = m->target->drafts;
+        for (size_t i = 0; i < v.size(); ++i) if (v[i] == m) { v.erase(v.begin() + i); break; }
+    } else if (m->stream) (void)hipStreamDestroy(m->stream);
+    for (lg_hip_model *d : m->drafts) d->target = nullptr;        // orphaned heads refuse to run
     delete m;
 }
 
@@ -440,10 +475,13 @@ extern "C" void lg_hip_kv_destroy(lg_hip_kv *kv) {
     (void)hipDeviceSynchronize();
     // graphs captured for this cache hold its pointers
     const std::string tag = "kv" + std::to_string(kv->id) + ":";
-    for (auto it = kv->m->graphs.begin(); it != kv->m->graphs.end();) {
-        if (it->first.compare(0, tag.size(), tag) == 0) { (void)hipGraphExecDestroy(it->second); it = kv->m->graphs.erase(it); }
-        else ++it;
-    }
+    std::vector<lg_hip_model *> holders(kv->m->drafts);
+    holders.push_back(kv->m);
+    for (lg_hip_model *h : holders)
+        for (auto it = h->graphs.begin(); it != h->graphs.end();) {
+            if (it->first.compare(0, tag.size(), tag) == 0) { (void)hipGraphExecDestroy(it->second); it = h->graphs.erase(it); }
+            else ++it;
+        }
     for (size_t L = 0; L < kv->k.size(); ++L) {
         (void)hipFree(kv->k[L]); (void)hipFree(kv->v[L]); (void)hipFree(kv->px_k[L]); (void)hipFree(kv->px_v[L]);
     }
@@ -577,6 +615,25 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     int cur = 0;                                   // x[cur] holds the residual
     bool have_x = false;                           // false: rows are still token ids
     const float *pend_dout = nullptr, *pend_w = nullptr, *pend_os = nullptr;   // sub-layer output waiting to be added
+    const bool draft = m->target != nullptr;
+    const int pos_off = draft ? -1 : 0;            // a draft at pos sees the cache as a query at pos-1 (src/cuda/mtp-kernel.cuh:170-182)
+    if (draft) {
+        // x = pre . [embedding(token)*sqrt(nb), h_prev] (src/mtp.c:268-278); h_prev is the target's hidden of the
+        // accepted row, or for a chained draft post . (this head's previous hidden) (src/cuda/mtp-kernel.cuh:372-389)
+        const lg_hip_model *t = m->target;
+        const int nb = t->E;
+        if (m->draft_chain) {
+            MmArgs a{ m->w_post, E, nb, m->hprev, m->hq, nullptr };
+            launch_mm<M, false>(lx, KC_PMP, a);
+        }
+        DraftInArgs d{};
+        d.emb = t->emb; d.emb_seg = lg_segments(nb); d.emb_nit = nb / 32 / d.emb_seg; d.emb_scale = sqrtf((float)nb);
+        d.toks = m->sched; d.h_prev = m->draft_chain ? m->hprev : t->g_hidden; d.nb = nb; d.q = m->catq;
+        LAUNCH(KC_ROWS, lg_k_draft_input, dim3((2 * nb / 4 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, d, m->ctl);
+        MmArgs p{ m->w_pre, 2 * nb, E, m->x[0], m->catq, nullptr };
+        launch_mm<M, false>(lx, KC_PMP, p);
+        have_x = true;
+    }
 
     // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
     auto rows = [&](const float *w_pre, float *h_out) {
@@ -599,7 +656,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     }
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
-        const int window = (y.is_local && m->window > 0) ? m->window : 0;
+        const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
         rows(y.attn_norm, nullptr);
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
@@ -618,10 +675,10 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             AttnArgs a{};
             a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
-            a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max;
+            a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
             const size_t lds = (size_t)G * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
             LAUNCH(KC_ATTN, lg_k_attn, dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), lds, a, m->ctl);
-            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, m->aq, nullptr };
+            MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
             LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
         {   // attention output projection
@@ -684,7 +741,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -744,6 +801,47 @@ extern "C" int lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t
     memcpy(out, m->pin + 32, (size_t)rows * 4);
     *adv = m->pin[48];
     m->last_rows = rows; m->last_adv = *adv;
+    return 0;
+}
+
+// ---- draft head ---------------------------------------------------------------------------------
+extern "C" int lg_hip_draft_create(lg_hip_model *target, const struct lg_hip_config *c, lg_hip_model **out) {
+    if (!target || !c || !out || !target->committed) return fail(-1, "draft_create: the target model must be committed first");
+    if (target->target) return fail(-2, "draft_create: the target is itself a draft head");
+    if (target->n_kv_start < 2) return fail(-2, "draft_create: the target needs a sliding and a global cache layer to read");
+    if (c->n_embd_per_layer) return fail(-2, "draft_create: a draft head has no per-layer embedding");
+    lg_hip_model *m = nullptr;
+    int rc = lg_hip_model_create(c, target->device, &m);
+    if (rc) return rc;
+    (void)hipStreamDestroy(m->stream);
+    m->stream = target->stream;                    // same queue: a draft reads what the last verify step wrote
+    m->target = target;
+    m->window = target->window;
+    m->n_kv_start = 0;
+    target->drafts.push_back(m);
+    *out = m;
+    return 0;
+}
+
+extern "C" int lg_hip_draft_step(lg_hip_model *d, lg_hip_kv *kv, int token, int pos, int chain, int32_t *tok_out) {
+    if (!d || !kv || !tok_out || !d->target || !d->committed || kv->m != d->target) return fail(-1, "draft_step: bad draft / cache pointer");
+    const lg_hip_model *t = d->target;
+    if (token < 0 || token >= t->n_vocab) return fail(-2, "draft_step: token id %d outside the target vocabulary of %d", token, t->n_vocab);
+    if (pos < 1 || pos > kv->max_seq) return fail(-2, "draft_step: position %d (the cache must hold 1..%d positions before it)", pos, kv->max_seq);
+    if (chain && !d->w_post) return fail(-4, "draft_step: this head has no post-projection, drafts cannot chain");
+    if (d->H > t->max_rows * t->H) return fail(-2, "draft_step: %d draft heads do not fit the target's attention scratch", d->H);
+    HIP_TRY(hipSetDevice(d->device));
+    int rc;
+    int32_t tk = token;
+    if ((rc = load_block(d, &tk, 1, pos))) return rc;
+    d->draft_chain = chain != 0;
+    rc = launch_step(d, kv, 1, true);
+    d->draft_chain = false;
+    if (rc) return rc;
+    HIP_TRY(hipMemcpyAsync(d->pin + 32, d->out, 4, hipMemcpyDeviceToHost, d->stream));
+    HIP_TRY(hipStreamSynchronize(d->stream));
+    *tok_out = d->pin[32];
+    d->last_rows = 1; d->last_adv = 1;
     return 0;
 }
 
@@ -1028,7 +1126,7 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     a.q = dq; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
     a.kc = dk; a.vc = dv; a.seq = seq; a.kv_dim = kd; a.window = window;
     a.pm = dpm; a.pl = dpl; a.pacc = dpacc; a.tiles_max = tiles;
-    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, dxq, dxf };
+    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, 0, dxq, dxf };
     hipStream_t st;
     HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
     int rc = 0;

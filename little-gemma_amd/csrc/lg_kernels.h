@@ -181,6 +181,32 @@ __device__ __forceinline__ void lg_load_q8(const int8_t *q, int k, int8_t *lq) {
     lg_copy_batched<uint4>((const uint4 *)q, (uint4 *)lq, M * k * 5 / 64);
 }
 
+// Input of a draft head (src/mtp.c:268-276): cat = [dequant(token_embd[token]) * sqrt(nb), h_prev],
+// quantized to q8 as one row of width 2*nb in the activation order of lg_act_layout(2*nb).
+// One thread per 4 values, 8 lanes per group of 32.
+struct DraftInArgs {
+    const uint8_t *emb; int emb_nit, emb_seg; float emb_scale;   // the target's tiled token_embd
+    const int32_t *toks;        // token slot (index ctl->step)
+    const float   *h_prev;      // [nb]
+    int            nb;
+    int8_t        *q;           // q8 activation buffer, one row of 2*nb
+};
+__global__ __launch_bounds__(LG_WG) void lg_k_draft_input(DraftInArgs a, const StepCtl *ctl) {
+    const int quad = blockIdx.x * LG_WG + threadIdx.x, k = 2 * a.nb;
+    if (quad >= (k >> 2)) return;                            // k is a multiple of 256: whole wavefronts leave
+    const int e = quad << 2;
+    float4 v;
+    if (e < a.nb) {
+        const float4 w = lg_tiled_deq4(a.emb, a.emb_nit, a.emb_seg, a.toks[ctl->step], e);
+        v = make_float4(w.x * a.emb_scale, w.y * a.emb_scale, w.z * a.emb_scale, w.w * a.emb_scale);
+    } else v = *(const float4 *)(a.h_prev + (e - a.nb));
+    float d; int sum;
+    const uint32_t packed = lg_quant4_8lanes(v, &d, &sum);
+    const ActLayout lay = lg_act_layout(k);
+    ((uint32_t *)a.q)[lg_act_unit(lay, quad >> 2) * 4 + (quad & 3)] = packed;
+    if ((threadIdx.x & 7) == 0) lg_q8_ds<1>(a.q, k)[lg_act_block(lay, quad >> 3)] = make_float2(d, __int_as_float(sum));
+}
+
 // ---------------------------------------------------------------------------------------------
 // G row groups against M q8 activation rows held in LDS.  A row is cut into S contiguous K
 // segments (S = 8, or 32 for rows longer than 128 blocks); lane = r*S + c owns row r of the group
@@ -612,6 +638,7 @@ struct AttnArgs {
     int seq, kv_dim, window; // ring rows, row width, 0 = global
     float *pm, *pl, *pacc;   // partials: [M*H][tiles_max], [M*H][tiles_max][hd]
     int tiles_max;
+    int pos_off;             // added to the step position: -1 for a draft head, whose query at pos sees keys < pos
     __device__ __forceinline__ uint4 kc4(size_t off) const { return *(const uint4 *)(kc + off); }
     __device__ __forceinline__ uint4 vc4(size_t off) const { return *(const uint4 *)(vc + off); }
 };
@@ -633,7 +660,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
     uint32_t *vmask = (uint32_t *)(es + G * 32);              // [G]
     const int kvh = blockIdx.y, j = blockIdx.z;
-    const int pos0 = ctl->pos, pj = pos0 + j;
+    const int pos0 = ctl->pos + a.pos_off, pj = pos0 + j;
     const int startj = lg_win_start(pj, a.window);
     const int n = (lg_win_start(pos0, a.window) >> 5) + blockIdx.x;
     if (n < (startj >> 5) || n > (pj >> 5)) return;           // tile outside this row's keys
@@ -726,7 +753,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
 // Merge the tile partials of one (row, head) in ascending tile order, divide, quantize to q8.
 struct MergeArgs {
     const float *pm, *pl, *pacc; int tiles_max;
-    int H, hd, window;
+    int H, hd, window, pos_off;
     int8_t *xq;                // q8 activation buffer of the attention output, width H*hd (input of attn_output)
     float *xf;                 // optional f32 copy [M][H*hd]
 };
@@ -734,7 +761,7 @@ template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const StepCtl *ctl) {
     __shared__ float wts[512];                                // exp(m_tile - M) of up to 512 tiles at a time
     const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
-    const int pos = ctl->pos, pj = pos + j;
+    const int pos = ctl->pos + a.pos_off, pj = pos + j;
     const int first = lg_win_start(pos, a.window) >> 5;
     const int lo = (lg_win_start(pj, a.window) >> 5) - first, hi = (pj >> 5) - first;
     const size_t base = ((size_t)j * a.H + head) * a.tiles_max;

@@ -120,6 +120,14 @@ def load_backend():
     B.lg_model_device_kv.restype = C.c_void_p
     B.lg_model_last_hidden.argtypes = [C.c_void_p, f32p]
     B.lg_model_release.restype = None
+    B.lg_session_mtp_open.argtypes = [C.c_void_p, C.c_char_p]
+    B.lg_session_mtp_open.restype = C.c_void_p
+    B.lg_session_mtp_close.argtypes = [C.c_void_p]
+    B.lg_session_mtp_close.restype = None
+    B.lg_session_mtp_draft.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]
+    B.lg_session_mtp_hidden.argtypes = [C.c_void_p, C.c_void_p, f32p]
+    B.lg_session_mtp_logits.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
+    B.lg_session_generate_mtp.argtypes = [C.c_void_p, C.c_void_p, i32p, C.c_int, C.c_int, C.c_int, i32p] + [C.POINTER(C.c_int)] * 3
     _backend = B
     return B
 
@@ -189,6 +197,41 @@ class HipBackend:
         d = np.ascontiguousarray(drafts, np.int32) if drafts is not None else None
         n = self.B.lg_session_generate(self.s, p, len(p), n_gen, rows, _opt(d), emitted, C.byref(steps))
         return emitted[:n], steps.value
+
+    # --- draft head (mtp_open / mtp_draft / mtp_draft_chain of the reference interface)
+    def mtp_open(self, path):
+        t = self.B.lg_session_mtp_open(self.s, os.fsencode(path))
+        if not t:
+            raise HipError(f"cannot open draft head {path} for this model")
+        return t
+
+    def mtp_close(self, t):
+        self.B.lg_session_mtp_close(t)
+
+    def mtp_draft(self, t, token, pos, chain=False):
+        return self.B.lg_session_mtp_draft(self.s, t, int(token), int(pos), int(chain))
+
+    def mtp_hidden(self, t, n_inner):
+        h = np.zeros(n_inner, np.float32)
+        hip_check(self.B.lg_session_mtp_hidden(self.s, t, h), "draft hidden")
+        return h
+
+    def mtp_store_logits(self, t, on=True):
+        hip_check(self.B.lg_session_mtp_logits(self.s, t, int(on), None), "draft store_logits")
+
+    def mtp_logits(self, t, n_vocab):
+        out = np.zeros(n_vocab, np.float32)
+        hip_check(self.B.lg_session_mtp_logits(self.s, t, 1, out.ctypes.data), "draft logits")
+        return out
+
+    def generate_mtp(self, t, prompt, n_gen, rows):
+        p = np.ascontiguousarray(prompt, np.int32)
+        emitted = np.zeros(n_gen, np.int32)
+        steps, nd, na = C.c_int(0), C.c_int(0), C.c_int(0)
+        n = self.B.lg_session_generate_mtp(self.s, t, p, len(p), n_gen, rows, emitted, C.byref(steps), C.byref(nd), C.byref(na))
+        if n < 0:
+            raise HipError("generate_mtp rejected its arguments")
+        return emitted[:n], steps.value, nd.value, na.value
 
     def last_hidden(self, n_embd):
         h = np.zeros(n_embd, np.float32)

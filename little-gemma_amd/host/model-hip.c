@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include "model.h"
+#include "mtp-internal.h"
 #include "lg_hip.h"
 
 const int model_kv_host = 0;          /* cache rows live on the device */
@@ -171,15 +172,62 @@ lg_hip_model *lg_model_device(struct model *m) { return device_model(m); }
 lg_hip_kv    *lg_model_device_kv(struct kvcache *kv) { return device_kv(kv); }
 void lg_model_release(void) { if (g_dev) { lg_hip_model_destroy(g_dev); g_dev = NULL; g_owner = NULL; } }
 
-/* The draft head is not on the device yet: report "unavailable" so the caller pads the block
- * (src/run.c:58-63), as the CPU backend does (src/cpu/model-cpu.c:61-71). */
-struct mtp;
+/* ---- draft head on the device (src/cuda/mtp-kernel.cuh:272-402) --------------------------------
+ * First use uploads the head (mtp_cuda_init there); a failure disables drafting for the process
+ * ((void *)-1), and the caller pads the block (src/run.c:58-63). */
+static lg_hip_model *draft_model(struct mtp *t, const struct model *m) {
+    if (t->cuda == (void *)-1) return NULL;
+    if (t->cuda) return (lg_hip_model *)t->cuda;
+    lg_hip_model *target = device_model(m), *d = NULL;
+    int32_t *geo = malloc((size_t)t->n_layer * 4 * sizeof *geo);
+    if (!geo) { t->cuda = (void *)-1; return NULL; }
+    int32_t *is_local = geo, *ffn = geo + t->n_layer, *hd = geo + 2 * t->n_layer, *nkv = geo + 3 * t->n_layer;
+    for (int L = 0; L < t->n_layer; L++) {
+        is_local[L] = m->is_local[t->l[L].src]; ffn[L] = t->n_ff; hd[L] = t->l[L].hd; nkv[L] = m->n_head_kv[t->l[L].src];
+    }
+    struct lg_hip_config hc = {
+        .n_layer = t->n_layer, .n_embd = t->n_inner, .n_head = t->n_head, .n_vocab = t->n_vocab,
+        .sliding_window = m->cfg.sliding_window, .n_embd_per_layer = 0, .n_kv_start = 0,
+        .rms_eps = t->eps, .rope_freq_base = t->base_full, .rope_freq_base_swa = t->base_swa, .logit_softcap = t->softcap,
+        .is_local = is_local, .ffn_len = ffn, .head_dim = hd, .n_head_kv = nkv,
+    };
+    int ok = lg_hip_draft_create(target, &hc, &d) == 0;
+    free(geo);
+    const struct gguf_context *g = t->ctx;
+    for (uint64_t i = 0; ok && i < g->header.num_tensors; i++) {
+        const struct gguf_tensor *w = &g->tensors[i];
+        const char *name = w == t->pre ? "pre_projection.weight" : w == t->post ? "post_projection.weight" : w->name;
+        ok = lg_hip_model_tensor(d, name, w->type, w->n_dims, w->dims, w->data) >= 0;
+    }
+    ok = ok && lg_hip_model_commit(d, 1) == 0;
+    if (!ok) {
+        fprintf(stderr, "mtp: device upload failed, drafting disabled: %s\n", lg_hip_last_error());
+        if (d) lg_hip_model_destroy(d);
+        t->cuda = (void *)-1;
+        return NULL;
+    }
+    t->cuda = d;
+    return d;
+}
+static int draft_on_device(struct mtp *t, const struct model *m, const struct kvcache *kv, int token, int pos, int chain) {
+    lg_hip_model *d = draft_model(t, m);
+    int32_t tok = -1;
+    if (!d) return -1;
+    if (lg_hip_draft_step(d, device_kv(kv), token, pos, chain, &tok) != 0) {
+        if (chain) return -1;                      /* e.g. no post-projection: the caller pads */
+        die("draft_step");
+    }
+    return tok;
+}
 int  mtp_draft_device(struct mtp *t, const struct model *m, const struct kvcache *kv, int token, int pos) {
-    (void)t; (void)m; (void)kv; (void)token; (void)pos;
-    return -1;
+    return draft_on_device(t, m, kv, token, pos, 0);
 }
 int  mtp_draft_chain_device(struct mtp *t, const struct model *m, const struct kvcache *kv, int token, int pos) {
-    (void)t; (void)m; (void)kv; (void)token; (void)pos;
-    return -1;
+    return draft_on_device(t, m, kv, token, pos, 1);
 }
-void mtp_free_device(struct mtp *t) { (void)t; }
+void mtp_free_device(struct mtp *t) {
+    if (t->cuda && t->cuda != (void *)-1) lg_hip_model_destroy((lg_hip_model *)t->cuda);
+    t->cuda = NULL;
+}
+/* the head's device handle, for callers that read its hidden state or logits */
+lg_hip_model *lg_mtp_device(struct mtp *t, const struct model *m) { return draft_model(t, m); }

@@ -49,7 +49,7 @@ int main(int argc, char **argv) {
         else if (!strcmp(argv[i], "-n") && i + 1 < argc) n_gen = atoi(argv[++i]);
     }
     if (!model || !prompt) {
-        printf("Usage: %s -m <model.gguf> -p <id,id,...> [-n N] [-mtp <draft-ids.txt> | -mtp self]\n"
+        printf("Usage: %s -m <model.gguf> -p <id,id,...> [-n N] [-mtp <assistant.gguf> | -mtp <draft-ids.txt> | -mtp self]\n"
                "       (built with LG_MTP_N=%d: speculative blocks verify %d tokens per step)\n", argv[0], LG_MTP_N, LG_MTP_N);
         return 1;
     }
@@ -66,7 +66,32 @@ int main(int argc, char **argv) {
     if (mtp) {
         drafts = calloc((size_t)n_gen + 64, sizeof(int));
         if (!drafts) return 1;
-        if (!strcmp(mtp, "self")) {
+        const size_t ml = strlen(mtp);
+        if (ml > 5 && !strcmp(mtp + ml - 5, ".gguf")) {
+            /* a draft-head file, as the reference's -mtp takes (src/run.c:719): plain greedy run
+             * first, then the same generation with the head drafting; the outputs must be equal */
+            plain = calloc((size_t)n_gen, sizeof(int));
+            if (!plain || lg_session_kv(s, max_seq) != 0) return 1;
+            int st;
+            lg_session_generate(s, ids, n_prompt, n_gen, 1, NULL, plain, &st);
+            struct mtp *head = lg_session_mtp_open(s, mtp);
+            if (!head) return 1;
+            if (lg_session_kv(s, max_seq) != 0) return 1;
+            int steps = 0, nd = 0, na = 0;
+            double t0 = now_sec();
+            int g = lg_session_generate_mtp(s, head, ids, n_prompt, n_gen, LG_MTP_N, emitted, &steps, &nd, &na);
+            double dt = now_sec() - t0;
+            for (int i = 0; i < g; i++) printf("%s%d", i ? "," : "", emitted[i]);
+            printf("\n");
+            fprintf(stderr, "gen:    %d tokens in %.2fs (%.2f tok/s)\n", g, dt, g / (dt > 0 ? dt : 1e-9));
+            fprintf(stderr, "mtp:    %d steps, %d drafts, %d accepted (%.0f%%), block %d\n", steps, nd, na, nd ? 100.0 * na / nd : 0.0, LG_MTP_N);
+            int bad = g != n_gen || memcmp(plain, emitted, (size_t)g * sizeof(int)) != 0;
+            fprintf(stderr, "check:  -mtp output %s plain greedy output\n", bad ? "DIFFERS FROM" : "is byte-identical to");
+            lg_session_mtp_close(head);
+            free(emitted); free(drafts); free(plain);
+            lg_session_close(s);
+            return bad;
+        } else if (!strcmp(mtp, "self")) {
             plain = calloc((size_t)n_gen, sizeof(int));
             if (!plain || lg_session_kv(s, max_seq) != 0) return 1;
             int steps;

@@ -3,8 +3,10 @@
 #include <stdlib.h>
 #include <string.h>
 #include "session.h"
+#include "lg_hip.h"
 
 int lg_model_forward_spec_n(struct model *m, struct kvcache *kv, const int *toks, int rows, int pos, int *out);
+lg_hip_model *lg_mtp_device(struct mtp *t, const struct model *m);
 
 struct lg_session { struct gguf_context *ctx; struct model m; struct kvcache kv; int has_kv; };
 
@@ -75,5 +77,55 @@ int lg_session_generate(struct lg_session *s, const int *prompt, int n_prompt, i
         best = out[adv - 1];
     }
     if (steps) *steps = n_steps;
+    return g;
+}
+
+/* ---- with a draft head ------------------------------------------------------------------------ */
+struct mtp *lg_session_mtp_open(struct lg_session *s, const char *path) { return mtp_open(path, &s->m); }
+void lg_session_mtp_close(struct mtp *t) { mtp_free(t); }
+int  lg_session_mtp_draft(struct lg_session *s, struct mtp *t, int token, int pos, int chain) {
+    return chain ? mtp_draft_chain(t, &s->m, &s->kv, token, pos) : mtp_draft(t, &s->m, &s->kv, token, pos);
+}
+int  lg_session_mtp_hidden(struct lg_session *s, struct mtp *t, float *dst) {
+    lg_hip_model *d = lg_mtp_device(t, &s->m);
+    return d ? lg_hip_get_hidden(d, dst) : -1;
+}
+int  lg_session_mtp_logits(struct lg_session *s, struct mtp *t, int on, float *dst) {
+    lg_hip_model *d = lg_mtp_device(t, &s->m);
+    if (!d) return -1;
+    if (!dst) return lg_hip_set_option(d, "store_logits", on);
+    return lg_hip_get_logits(d, 0, dst);
+}
+
+/* The reference's speculative loop (src/run.c:54-71 mtp_step inside :737-768): the head drafts
+ * toks[1] from the target's hidden, chains toks[2..] on its own, the target verifies the block.
+ * A draft that is unavailable (-1) is padded with the previous token. */
+int lg_session_generate_mtp(struct lg_session *s, struct mtp *t, const int *prompt, int n_prompt, int n_gen, int rows,
+                            int *emitted, int *steps, int *n_draft, int *n_accept) {
+    if (n_prompt < 1 || !s->has_kv || rows < 2 || rows > 16) return -1;
+    model_prefill(&s->m, &s->kv, prompt, n_prompt - 1, 0);
+    int pos = n_prompt - 1, g = 0, n_steps = 0, nd = 0, na = 0;
+    int best = model_forward_next(&s->m, &s->kv, prompt[n_prompt - 1], pos++);
+    while (g < n_gen) {
+        emitted[g++] = best;
+        if (g >= n_gen) break;
+        if (pos + rows - 1 >= s->kv.max_seq) { best = model_forward_next(&s->m, &s->kv, best, pos++); n_steps++; continue; }
+        int toks[16], out[16];
+        toks[0] = best;
+        int d = mtp_draft(t, &s->m, &s->kv, best, pos);
+        toks[1] = d >= 0 ? d : best;
+        for (int j = 2; j < rows; j++) {
+            int dj = mtp_draft_chain(t, &s->m, &s->kv, toks[j - 1], pos + j - 1);
+            toks[j] = dj >= 0 ? dj : toks[j - 1];
+        }
+        int adv = lg_model_forward_spec_n(&s->m, &s->kv, toks, rows, pos, out);
+        n_steps++; nd += rows - 1; na += adv - 1;
+        pos += adv;
+        for (int e = 1; e < adv && g < n_gen; e++) emitted[g++] = toks[e];
+        best = out[adv - 1];
+    }
+    if (steps) *steps = n_steps;
+    if (n_draft) *n_draft = nd;
+    if (n_accept) *n_accept = na;
     return g;
 }

@@ -28,4 +28,15 @@ int  lg_session_forward_spec(struct lg_session *s, const int *toks, int rows, in
  * Returns tokens emitted; *steps = target forwards/verify steps run. */
 int  lg_session_generate(struct lg_session *s, const int *prompt, int n_prompt, int n_gen, int rows,
                          const int *drafts, int *emitted, int *steps);
+/* Draft head (include/model.h:156-178): open a gemma4-assistant file for this session's model,
+ * one draft (chain = 0: from the target's hidden; 1: chained on the head's own), the head's
+ * post-norm hidden, its logits (dst NULL: switch storing on/off), and the reference's
+ * speculative loop with the head proposing every block. */
+struct mtp *lg_session_mtp_open(struct lg_session *s, const char *path);
+void lg_session_mtp_close(struct mtp *t);
+int  lg_session_mtp_draft(struct lg_session *s, struct mtp *t, int token, int pos, int chain);
+int  lg_session_mtp_hidden(struct lg_session *s, struct mtp *t, float *dst);
+int  lg_session_mtp_logits(struct lg_session *s, struct mtp *t, int on, float *dst);
+int  lg_session_generate_mtp(struct lg_session *s, struct mtp *t, const int *prompt, int n_prompt, int n_gen, int rows,
+                             int *emitted, int *steps, int *n_draft, int *n_accept);
 #endif

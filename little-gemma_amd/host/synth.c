@@ -55,11 +55,11 @@ static int add_layer(struct plan *p, int L, const char *leaf, uint32_t type, uin
     return plan_add(p, name, type, cols, rows, centre);
 }
 
-static void fill(const struct planned *t, void *dst, const struct lg_synth_spec *s) {
+static void fill(const struct planned *t, void *dst, float norm_jitter, float w_std) {
     if (t->type == GGML_TYPE_F32) {
         float *o = dst;
         for (uint64_t i = 0; i < t->cols * t->rows; i++)
-            o[i] = t->centre * (1.0f + s->norm_jitter * uniform_pm1(t->key, i));
+            o[i] = t->centre * (1.0f + norm_jitter * uniform_pm1(t->key, i));
         return;
     }
     const uint64_t row_bytes = t->cols / 32 * LG_Q4_0_BYTES;
@@ -71,7 +71,7 @@ static void fill(const struct planned *t, void *dst, const struct lg_synth_spec 
             uint64_t ctr = ((uint64_t)r * (t->cols / 32) + b) * 16;
             for (int j = 0; j < 16; j++) {
                 normal_pair(t->key, ctr + (uint64_t)j, &buf[2 * j], &buf[2 * j + 1]);
-                buf[2 * j] *= s->w_std; buf[2 * j + 1] *= s->w_std;
+                buf[2 * j] *= w_std; buf[2 * j + 1] *= w_std;
             }
             lg_quantize_q4_0(buf, o + b * LG_Q4_0_BYTES, 32);
         }
@@ -159,7 +159,68 @@ int lg_synth_write(const char *path, const struct lg_synth_spec *s) {
     for (int i = 0; i < p.n; i++) {
         size_t bytes;
         void *dst = lg_gw_tensor_data(w, p.t[i].index, &bytes);
-        fill(&p.t[i], dst, s);
+        fill(&p.t[i], dst, s->norm_jitter, s->w_std);
+    }
+    free(p.t);
+    return lg_gw_close(w) == 0 ? 0 : -6;
+}
+
+/* The draft head file the reference's mtp_open reads (src/mtp.c:124-215): architecture
+ * "gemma4-assistant", its keys under that prefix, the two next-token projections, its own
+ * token_embd (the head's LM head, inner width) and per block q / output / FFN matrices and norms;
+ * no k/v projections (the blocks read the target's cache). */
+int lg_synth_write_assistant(const char *path, const struct lg_synth_assistant_spec *s) {
+    if (s->n_layer <= 0 || s->n_inner % 32 || s->n_backbone % 32 || s->n_ff % 32 || s->head_dim_swa % 32 ||
+        s->head_dim_full % 32 || s->n_full < 0 || s->n_full > s->n_layer || s->n_head <= 0) {
+        fprintf(stderr, "lg_synth_write_assistant: invalid spec\n");
+        return -1;
+    }
+    struct lg_gguf_writer *w = lg_gw_open(path, 3, 32);
+    if (!w) { perror(path); return -2; }
+    const char *A = "gemma4-assistant";
+    char key[128];
+    int rc = lg_gw_meta_str(w, "general.architecture", A);
+#define KU(leaf, v) (snprintf(key, sizeof key, "%s.%s", A, leaf), rc |= lg_gw_meta_u32(w, key, (uint32_t)(v)))
+#define KF(leaf, v) (snprintf(key, sizeof key, "%s.%s", A, leaf), rc |= lg_gw_meta_f32(w, key, (v)))
+    KU("block_count", s->n_layer);
+    KU("embedding_length", s->n_inner);
+    KU("embedding_length_out", s->n_backbone);
+    KU("attention.head_count", s->n_head);
+    KU("feed_forward_length", s->n_ff);
+    KF("attention.layer_norm_rms_epsilon", s->rms_eps);
+    KF("rope.freq_base", s->rope_base);
+    KF("rope.freq_base_swa", s->rope_base_swa);
+    KF("final_logit_softcapping", s->softcap);
+#undef KU
+#undef KF
+    if (rc) { lg_gw_close(w); return -4; }
+    struct plan p = { w, NULL, 0, 0, s->seed };
+    const uint64_t I = (uint64_t)s->n_inner, B = (uint64_t)s->n_backbone, F = (uint64_t)s->n_ff;
+    rc |= plan_add(&p, "token_embd.weight", GGML_TYPE_Q4_0, I, (uint64_t)s->n_vocab, 0);
+    rc |= plan_add(&p, "output_norm.weight", GGML_TYPE_F32, I, 1, 1.0f);
+    rc |= plan_add(&p, "nextn.pre_projection.weight", GGML_TYPE_Q4_0, 2 * B, I, 0);
+    if (s->has_post) rc |= plan_add(&p, "nextn.post_projection.weight", GGML_TYPE_Q4_0, I, B, 0);
+    for (int L = 0; L < s->n_layer && !rc; L++) {
+        const int full = L >= s->n_layer - s->n_full;
+        const uint64_t hd = (uint64_t)(full ? s->head_dim_full : s->head_dim_swa), qd = hd * (uint64_t)s->n_head;
+        const float qk = s->qk_norm > 0 ? s->qk_norm : sqrtf(1.28f / sqrtf((float)hd));
+        rc |= add_layer(&p, L, "attn_norm.weight", GGML_TYPE_F32, I, 1, 1.0f);
+        rc |= add_layer(&p, L, "attn_q.weight", GGML_TYPE_Q4_0, I, qd, 0);
+        rc |= add_layer(&p, L, "attn_q_norm.weight", GGML_TYPE_F32, hd, 1, qk);
+        rc |= add_layer(&p, L, "attn_output.weight", GGML_TYPE_Q4_0, qd, I, 0);
+        rc |= add_layer(&p, L, "post_attention_norm.weight", GGML_TYPE_F32, I, 1, 1.0f);
+        rc |= add_layer(&p, L, "ffn_norm.weight", GGML_TYPE_F32, I, 1, 1.0f);
+        rc |= add_layer(&p, L, "ffn_gate.weight", GGML_TYPE_Q4_0, I, F, 0);
+        rc |= add_layer(&p, L, "ffn_up.weight", GGML_TYPE_Q4_0, I, F, 0);
+        rc |= add_layer(&p, L, "ffn_down.weight", GGML_TYPE_Q4_0, F, I, 0);
+        rc |= add_layer(&p, L, "post_ffw_norm.weight", GGML_TYPE_F32, I, 1, 1.0f);
+        if (s->out_scale > 0) rc |= add_layer(&p, L, "layer_output_scale.weight", GGML_TYPE_F32, 1, 1, s->out_scale);
+    }
+    if (rc || lg_gw_commit(w) != 0) { fprintf(stderr, "lg_synth_write_assistant: cannot lay out %s\n", path); free(p.t); lg_gw_close(w); return -5; }
+    for (int i = 0; i < p.n; i++) {
+        size_t bytes;
+        void *dst = lg_gw_tensor_data(w, p.t[i].index, &bytes);
+        fill(&p.t[i], dst, s->norm_jitter, s->w_std);
     }
     free(p.t);
     return lg_gw_close(w) == 0 ? 0 : -6;

@@ -32,4 +32,17 @@ struct lg_synth_spec {
 /* 0 on success; a negative code and a message on stderr otherwise. */
 int lg_synth_write(const char *path, const struct lg_synth_spec *spec);
 
+/* A draft head ("gemma4-assistant", src/mtp.c:124-215) for a target of width n_backbone whose
+ * sliding / global layers have heads of head_dim_swa / head_dim_full: the last n_full blocks
+ * read the global cache, the others the sliding one. */
+struct lg_synth_assistant_spec {
+    int32_t n_layer, n_inner, n_backbone, n_head, n_ff, n_vocab;
+    int32_t head_dim_swa, head_dim_full, n_full;
+    int32_t has_post;          /* 0: no post-projection (drafts cannot chain) */
+    float   w_std, qk_norm, norm_jitter, out_scale;
+    float   rms_eps, rope_base, rope_base_swa, softcap;
+    uint64_t seed;
+};
+int lg_synth_write_assistant(const char *path, const struct lg_synth_assistant_spec *spec);
+
 #endif

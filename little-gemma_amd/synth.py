@@ -40,3 +40,37 @@ def write_model(path, **spec):
     if rc != 0:
         raise RuntimeError(f"lg_synth_write({path}) failed with {rc}")
     return full
+
+
+class AssistantSpec(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "n_layer", "n_inner", "n_backbone", "n_head", "n_ff", "n_vocab", "head_dim_swa", "head_dim_full", "n_full",
+        "has_post")] + [(n, C.c_float) for n in ("w_std", "qk_norm", "norm_jitter", "out_scale", "rms_eps", "rope_base",
+                                                 "rope_base_swa", "softcap")] + [("seed", C.c_uint64)]
+
+
+ASSISTANT_DEFAULTS = dict(n_layer=4, n_inner=256, n_head=4, n_full=1, has_post=1, w_std=0.02, qk_norm=0.0,
+                          norm_jitter=0.1, out_scale=0.0, rms_eps=1e-6, rope_base=1e6, rope_base_swa=1e4,
+                          softcap=30.0, seed=4321)
+
+
+def assistant_for(target, **over):
+    """Spec of a draft head ("gemma4-assistant") that fits the target spec: 4 blocks, 256 wide, the last one
+    reading the global cache (when the target's head sizes differ; otherwise all read the sliding one)."""
+    hd_l = target["head_dim"]
+    hd_g = target.get("head_dim_full") or hd_l
+    spec = dict(ASSISTANT_DEFAULTS, n_backbone=target["n_embd"], n_vocab=target["n_vocab"], head_dim_swa=hd_l,
+                head_dim_full=hd_g, n_ff=1024, qk_norm=target.get("qk_norm", 0.0),
+                rope_base=target.get("rope_base", 1e6), rope_base_swa=target.get("rope_base_swa", 1e4))
+    spec.update(over)
+    return spec
+
+
+def write_assistant(path, **spec):
+    s = AssistantSpec(**spec)
+    lib = hostlib.lib()
+    lib.lg_synth_write_assistant.restype = C.c_int
+    rc = lib.lg_synth_write_assistant(os.fsencode(path), C.byref(s))
+    if rc != 0:
+        raise RuntimeError(f"lg_synth_write_assistant({path}) failed with {rc}")
+    return spec

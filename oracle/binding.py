@@ -72,6 +72,13 @@ def lib():
     L.lgo_prefill.argtypes = [C.c_void_p, C.c_void_p, c_i32p, C.c_int, C.c_int, C.c_int]
     L.lgo_forward_spec.argtypes = [C.c_void_p, C.c_void_p, c_i32p, C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]
     L.lgo_set_threads.argtypes = [C.c_int]
+    L.lgo_forward_spec_all.argtypes = [C.c_void_p, C.c_void_p, c_i32p, C.c_int, C.c_int, C.c_int, c_i32p, C.c_void_p]
+    L.lgo_mtp_open.argtypes = [C.c_char_p, C.c_void_p]
+    L.lgo_mtp_open.restype = C.c_void_p
+    L.lgo_mtp_close.argtypes = [C.c_void_p]
+    L.lgo_mtp_info.argtypes = [C.c_void_p, c_i32p, C.c_int]
+    L.lgo_mtp_draft.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, c_f32p, C.c_int, C.c_void_p, C.c_void_p]
+    L.lgo_mtp_post.argtypes = [C.c_void_p, c_f32p, C.c_int, c_f32p]
     _lib = L
     return L
 
@@ -156,6 +163,54 @@ class Oracle:
                                       hidden.ctypes.data if want_hidden else None)
         return adv, out, hidden
 
+    def forward_spec_all(self, kv, toks, pos, mode, want_hidden=False):
+        """The verify step as the device runs it: every row forwarded (rejected rows reach the cache too)."""
+        t = np.ascontiguousarray(toks, np.int32)
+        out = np.full(len(t), -1, np.int32)
+        hidden = np.zeros(self.info["n_embd"], np.float32) if want_hidden else None
+        adv = self.L.lgo_forward_spec_all(self.h, kv, t, len(t), pos, mode, out,
+                                          hidden.ctypes.data if want_hidden else None)
+        return adv, out, hidden
+
+    def mtp_open(self, path):
+        return OracleDraft(self, path)
+
+
+MTP_KEYS = ("n_layer", "n_inner", "n_bb", "n_vocab", "n_head", "n_ff", "has_post")
+
+
+class OracleDraft:
+    """A draft-head file under the CPU oracle, attached to its target."""
+
+    def __init__(self, target, path):
+        self.L, self.target = target.L, target
+        self.h = self.L.lgo_mtp_open(os.fsencode(path), target.h)
+        if not self.h:
+            raise RuntimeError(f"oracle: cannot open draft head {path} for this target")
+        v = np.zeros(8, np.int32)
+        n = self.L.lgo_mtp_info(self.h, v, 8)
+        self.info = dict(zip(MTP_KEYS, (int(x) for x in v[:n])))
+
+    def close(self):
+        if self.h:
+            self.L.lgo_mtp_close(self.h)
+            self.h = None
+
+    def draft(self, kv, token, pos, h_prev, mode, want_logits=False):
+        hidden = np.zeros(self.info["n_inner"], np.float32)
+        logits = np.zeros(self.info["n_vocab"], np.float32) if want_logits else None
+        tok = self.L.lgo_mtp_draft(self.h, self.target.h, kv, token, pos, np.ascontiguousarray(h_prev, np.float32), mode,
+                                   hidden.ctypes.data, logits.ctypes.data if want_logits else None)
+        if tok < 0:
+            raise ValueError("oracle draft rejected its arguments")
+        return tok, hidden, logits
+
+    def post(self, hidden, mode):
+        out = np.zeros(self.info["n_bb"], np.float32)
+        if self.L.lgo_mtp_post(self.h, np.ascontiguousarray(hidden, np.float32), mode, out) != 0:
+            return None
+        return out
+
 
 def ref_available(n=4):
     return os.path.exists(os.path.join(HERE, "_ref", f"libref_n{n}.so"))
@@ -189,6 +244,14 @@ def ref_lib(n=4):
         R.ref_dequantize.argtypes = [C.c_uint, c_u8p, c_f32p, C.c_longlong]
         for f in ("ref_n_vocab", "ref_n_embd", "ref_n_layer"):
             getattr(R, f).argtypes = [C.c_void_p]
+        R.ref_mtp_open.argtypes = [C.c_void_p, C.c_char_p]
+        R.ref_mtp_open.restype = C.c_void_p
+        R.ref_mtp_free.argtypes = [C.c_void_p]
+        R.ref_mtp_draft.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+        R.ref_mtp_n_vocab.argtypes = [C.c_void_p]
+        R.ref_mtp_n_inner.argtypes = [C.c_void_p]
+        R.ref_mtp_logits.argtypes = [C.c_void_p, c_f32p]
+        R.ref_mtp_hidden.argtypes = [C.c_void_p, c_f32p]
         _ref[n] = R
     return _ref[n]
 
@@ -248,3 +311,21 @@ class Reference:
         h = np.zeros(self.n_embd, np.float32)
         self.R.ref_last_hidden(self.h, h)
         return h
+
+    # the reference's host draft head (src/mtp.c), h_prev = this model's last_hidden
+    def mtp_open(self, path):
+        t = self.R.ref_mtp_open(self.h, os.fsencode(path))
+        if not t:
+            raise RuntimeError(f"reference: cannot open draft head {path}")
+        return t
+
+    def mtp_free(self, t):
+        self.R.ref_mtp_free(t)
+
+    def mtp_draft(self, t, kv, token, pos):
+        tok = self.R.ref_mtp_draft(self.h, t, kv, token, pos)
+        logits = np.zeros(self.R.ref_mtp_n_vocab(t), np.float32)
+        hidden = np.zeros(self.R.ref_mtp_n_inner(t), np.float32)
+        self.R.ref_mtp_logits(t, logits)
+        self.R.ref_mtp_hidden(t, hidden)
+        return tok, hidden, logits

@@ -717,3 +717,232 @@ int lgo_forward_spec(struct lgo_model *o, struct lgo_kv *kv, const int *toks, in
     } while (j < rows && out[j - 1] == toks[j]);
     return j;
 }
+
+/* ======================  draft head  ====================================== */
+/* The gemma4-assistant network (src/mtp.c).  LGO_REF restates the reference's host draft
+ * (src/mtp.c:258-356) in its own order of operations and is pinned by running that file from the
+ * reference build (oracle/_ref) on the same GGUFs.  The int8 class is what the device computes:
+ * q8 activations at every matmul input, this build's float orders, the cache seen through the
+ * tiled attention as a query at pos-1 (src/cuda/mtp-kernel.cuh:170-182).  The reference's device
+ * draft (f16 weights, f32 activations, CUDA summation order) cannot run here: PARITY UNPINNED for
+ * its last bits, and for the chained draft's post-projection, which has no CPU counterpart. */
+struct lgo_mtp_layer {
+    const float *attn_norm, *q_norm, *post_attn, *ffn_norm, *post_ffw, *out_scale;
+    const struct gguf_tensor *q, *o, *gate, *up, *down;
+    int hd, local, src;
+};
+struct lgo_mtp {
+    struct gguf_context *ctx;
+    int n_layer, n_inner, n_bb, n_vocab, n_head, n_ff;
+    float eps, base_full, base_swa, softcap;
+    const struct gguf_tensor *pre, *post, *head;
+    const float *out_norm;
+    struct lgo_mtp_layer *l;
+};
+
+void lgo_mtp_close(struct lgo_mtp *t) {
+    if (!t) return;
+    free(t->l);
+    free_gguf(t->ctx);
+    free(t);
+}
+
+struct lgo_mtp *lgo_mtp_open(const char *path, const struct lgo_model *target) {
+    struct lgo_mtp *t = calloc(1, sizeof *t);
+    if (!t) return NULL;
+    t->ctx = load_gguf(path);
+    if (!t->ctx) { free(t); return NULL; }
+    const struct gguf_context *g = t->ctx;
+    const char *arch = gguf_get_str(g, "general.architecture", "");
+    char key[96];
+#define AK(leaf) (snprintf(key, sizeof key, "%s.%s", arch, leaf), key)
+    t->n_layer = (int)gguf_get_u32(g, AK("block_count"), 0);
+    t->n_inner = (int)gguf_get_u32(g, AK("embedding_length"), 0);
+    t->n_bb = (int)gguf_get_u32(g, AK("embedding_length_out"), 0);
+    t->n_head = (int)gguf_get_u32(g, AK("attention.head_count"), 0);
+    t->n_ff = (int)gguf_get_u32(g, AK("feed_forward_length"), 0);
+    t->eps = gguf_get_f32(g, AK("attention.layer_norm_rms_epsilon"), 1e-6f);
+    t->base_full = gguf_get_f32(g, AK("rope.freq_base"), 1e6f);
+    t->base_swa = gguf_get_f32(g, AK("rope.freq_base_swa"), 1e4f);
+    t->softcap = gguf_get_f32(g, AK("final_logit_softcapping"), 0.0f);
+#undef AK
+    t->pre = gguf_find_tensor(g, "nextn.pre_projection.weight");
+    t->post = gguf_find_tensor(g, "nextn.post_projection.weight");
+    t->head = gguf_find_tensor(g, "token_embd.weight");
+    t->out_norm = f32_tensor(g, "output_norm.weight");
+    const struct model *m = &target->m;
+    if (!t->n_layer || !t->pre || !t->head || !t->out_norm || t->n_bb != m->cfg.n_embd || m->cfg.n_kv_start < 2) { lgo_mtp_close(t); return NULL; }
+    t->n_vocab = (int)t->head->dims[1];
+    const int src_full = m->cfg.n_kv_start - 1, src_swa = m->cfg.n_kv_start - 2;      /* src/mtp.c:173-176 */
+    t->l = calloc((size_t)t->n_layer, sizeof *t->l);
+    for (int L = 0; L < t->n_layer; L++) {
+        struct lgo_mtp_layer *b = &t->l[L];
+        b->attn_norm = layer_f(g, L, "attn_norm.weight");   b->q_norm = layer_f(g, L, "attn_q_norm.weight");
+        b->post_attn = layer_f(g, L, "post_attention_norm.weight"); b->ffn_norm = layer_f(g, L, "ffn_norm.weight");
+        b->post_ffw = layer_f(g, L, "post_ffw_norm.weight"); b->out_scale = layer_f(g, L, "layer_output_scale.weight");
+        b->q = layer_t(g, L, "attn_q.weight"); b->o = layer_t(g, L, "attn_output.weight");
+        b->gate = layer_t(g, L, "ffn_gate.weight"); b->up = layer_t(g, L, "ffn_up.weight"); b->down = layer_t(g, L, "ffn_down.weight");
+        if (!b->attn_norm || !b->q_norm || !b->post_attn || !b->ffn_norm || !b->post_ffw || !b->q || !b->o || !b->gate || !b->up || !b->down) { lgo_mtp_close(t); return NULL; }
+        b->hd = (int)b->q->dims[1] / t->n_head;
+        b->local = b->hd == m->head_dim[src_swa];                                    /* src/mtp.c:196-198 */
+        b->src = b->local ? src_swa : src_full;
+        if (b->hd != m->head_dim[b->src]) { lgo_mtp_close(t); return NULL; }
+    }
+    return t;
+}
+
+int lgo_mtp_info(const struct lgo_mtp *t, int32_t *out, int cap) {
+    int32_t v[] = { t->n_layer, t->n_inner, t->n_bb, t->n_vocab, t->n_head, t->n_ff, t->post != NULL };
+    int n = (int)(sizeof v / sizeof v[0]);
+    for (int i = 0; i < n && i < cap; i++) out[i] = v[i];
+    return n;
+}
+
+/* A cache element as the reference's HOST draft reads it (src/mtp.c:96-113): its private f16
+ * reader gives f16 subnormals half their value (exponent 127-15+e+1 with e starting at -1 and one
+ * further decrement per shift; model-cpu.c:201-210 starts one higher and is exact).  LGO_REF keeps
+ * that so that it stays bit-identical with the reference build; the int8 class, like the
+ * reference's device draft (__half loads), converts exactly. */
+static float kv_elem(const void *base, size_t i, int f16) {
+    if (!f16) return ((const float *)base)[i];
+    const uint16_t h = ((const uint16_t *)base)[i];
+    const float v = lg_f16_to_f32(h);
+    return ((h & 0x7C00u) == 0 && (h & 0x03FFu) != 0) ? 0.5f * v : v;
+}
+
+/* One draft.  h_prev: n_bb floats (the target's post-norm hidden of the accepted row, or a chained
+ * head hidden lifted by lgo_mtp_post).  hidden_out (n_inner, post output norm) and logits
+ * (n_vocab) may be NULL.  Returns the first maximum of the soft-capped logits. */
+int lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv, int token, int pos,
+                  const float *h_prev, int mode, float *hidden_out, float *logits_out) {
+    const struct model *m = &target->m;
+    const struct config *c = &m->cfg;
+    const int ni = t->n_inner, nb = t->n_bb, ref = mode == LGO_REF, exact = mode == LGO_I8;
+    const float eps = t->eps;
+    if (pos < 1 || token < 0 || token >= c->n_vocab) return -1;
+    if (ref != (kv->mode == LGO_REF)) { fprintf(stderr, "oracle: kv cache was created for another mode\n"); return -1; }
+    int qmax = 0, widest = 2 * nb;
+    for (int L = 0; L < t->n_layer; L++) if (t->n_head * t->l[L].hd > qmax) qmax = t->n_head * t->l[L].hd;
+    if (qmax > widest) widest = qmax;
+    if (t->n_ff > widest) widest = t->n_ff;
+    struct qact a = { malloc((size_t)widest), malloc((size_t)widest / 32 * 4) };
+    float *cat = malloc((size_t)2 * nb * 4), *x = malloc((size_t)ni * 4), *h = malloc((size_t)ni * 4);
+    float *q = malloc((size_t)qmax * 4), *xb = malloc((size_t)qmax * 4), *o = malloc((size_t)ni * 4);
+    float *g1 = malloc((size_t)t->n_ff * 4), *g2 = malloc((size_t)t->n_ff * 4), *att = malloc((size_t)(pos + 1) * 4);
+    float *tab = malloc((size_t)qmax * 4), *logits = logits_out ? logits_out : malloc((size_t)t->n_vocab * 4);
+
+    float *erow = dequantize_row(target->token_embd, token, nb);                     /* src/mtp.c:268-276 */
+    const float es = sqrtf((float)nb);
+    for (int i = 0; i < nb; i++) cat[i] = erow[i] * es;
+    free(erow);
+    memcpy(cat + nb, h_prev, (size_t)nb * 4);
+    if (ref) lgo_matmul_f32(t->pre->data, t->pre->type, 2 * nb, ni, cat, x);
+    else { quant_into(&a, cat, 2 * nb); mm(t->pre, 2 * nb, ni, &a, x); }
+
+    for (int L = 0; L < t->n_layer; L++) {
+        const struct lgo_mtp_layer *b = &t->l[L];
+        const int hd = b->hd, src = b->src, qd = t->n_head * hd;
+        const int kd = kv->kv_dim[src], nkv = m->n_head_kv[src], gqa = t->n_head / nkv, seq = kv->seq[src];
+        fill_tab(tab, b->local ? t->base_swa : t->base_full, hd);
+        lgo_rmsnorm(h, x, b->attn_norm, ni, eps, !ref);
+        if (ref) lgo_matmul_f32(b->q->data, b->q->type, ni, qd, h, q);
+        else { quant_into(&a, h, ni); mm(b->q, ni, qd, &a, q); }
+        for (int hh = 0; hh < t->n_head; hh++) {
+            lgo_rmsnorm(q + hh * hd, q + hh * hd, b->q_norm, hd, eps, !ref);
+            lgo_rope(q + hh * hd, hd, pos, tab, NULL, exact);
+        }
+        /* the cache holds positions < pos; sliding blocks see the window back from pos (src/mtp.c:298-302) */
+        const int start = (b->local && c->sliding_window > 0 && pos - c->sliding_window + 1 > 0) ? pos - c->sliding_window + 1 : 0;
+        if (ref) {
+            const void *Kc = kv->k[src], *Vc = kv->v[src];
+            const int f16 = kv->f16[src];
+            for (int hh = 0; hh < t->n_head; hh++) {
+                const float *qh = q + hh * hd;
+                const int kvh = hh / gqa;
+                for (int p = start; p < pos; p++) {
+                    const size_t off = (size_t)(p % seq) * kd + (size_t)kvh * hd;
+                    float s = 0.0f;
+                    for (int i = 0; i < hd; i++) s += qh[i] * kv_elem(Kc, off + i, f16);
+                    att[p] = s;
+                }
+                {   /* softmax (src/mtp.c:62-68) */
+                    float *v = att + start; const int n = pos - start;
+                    float mx = v[0];
+                    for (int i = 1; i < n; i++) if (v[i] > mx) mx = v[i];
+                    float sum = 0.0f;
+                    for (int i = 0; i < n; i++) { v[i] = expf(v[i] - mx); sum += v[i]; }
+                    for (int i = 0; i < n; i++) v[i] /= sum;
+                }
+                float *outh = xb + hh * hd;
+                for (int i = 0; i < hd; i++) outh[i] = 0.0f;
+                for (int p = start; p < pos; p++) {
+                    const size_t off = (size_t)(p % seq) * kd + (size_t)kvh * hd;
+                    const float w = att[p];
+                    for (int i = 0; i < hd; i++) outh[i] += w * kv_elem(Vc, off + i, f16);
+                }
+            }
+        } else {
+            /* a query at pos-1 with the window one shorter: keys max(0, pos-window+1) .. pos-1 */
+            #pragma omp parallel for schedule(static)
+            for (int hh = 0; hh < t->n_head; hh++)
+                lgo_attention_f16(xb + hh * hd, q + hh * hd, kv->k[src], kv->v[src], hd, kd, hh / gqa, seq, start, pos - 1, 1, exact);
+        }
+        if (ref) lgo_matmul_f32(b->o->data, b->o->type, qd, ni, xb, o);
+        else { quant_into(&a, xb, qd); mm(b->o, qd, ni, &a, o); }
+        lgo_rmsnorm(o, o, b->post_attn, ni, eps, !ref);
+        for (int i = 0; i < ni; i++) h[i] = x[i] + o[i];
+
+        lgo_rmsnorm(x, h, b->ffn_norm, ni, eps, !ref);
+        if (ref) {
+            lgo_matmul_f32(b->gate->data, b->gate->type, ni, t->n_ff, x, g1);
+            lgo_matmul_f32(b->up->data, b->up->type, ni, t->n_ff, x, g2);
+        } else { quant_into(&a, x, ni); mm(b->gate, ni, t->n_ff, &a, g1); mm(b->up, ni, t->n_ff, &a, g2); }
+        for (int i = 0; i < t->n_ff; i++) g1[i] = lgo_gelu(g1[i], exact) * g2[i];
+        if (ref) lgo_matmul_f32(b->down->data, b->down->type, t->n_ff, ni, g1, o);
+        else { quant_into(&a, g1, t->n_ff); mm(b->down, t->n_ff, ni, &a, o); }
+        lgo_rmsnorm(o, o, b->post_ffw, ni, eps, !ref);
+        if (ref) {
+            for (int i = 0; i < ni; i++) x[i] = h[i] + o[i];
+            if (b->out_scale) for (int i = 0; i < ni; i++) x[i] *= b->out_scale[0];
+        } else {
+            for (int i = 0; i < ni; i++) { const float v = h[i] + o[i]; x[i] = b->out_scale ? v * b->out_scale[0] : v; }
+        }
+    }
+    lgo_rmsnorm(x, x, t->out_norm, ni, eps, !ref);
+    if (hidden_out) memcpy(hidden_out, x, (size_t)ni * 4);
+    if (ref) lgo_matmul_f32(t->head->data, t->head->type, ni, t->n_vocab, x, logits);
+    else { quant_into(&a, x, ni); mm(t->head, ni, t->n_vocab, &a, logits); }
+    if (t->softcap > 0.0f)
+        for (int v = 0; v < t->n_vocab; v++) logits[v] = t->softcap * (exact ? lg_tanhf(logits[v] / t->softcap) : tanhf(logits[v] / t->softcap));
+    int best = 0;
+    for (int v = 1; v < t->n_vocab; v++) if (logits[v] > logits[best]) best = v;
+    if (!logits_out) free(logits);
+    free(a.q); free(a.d); free(cat); free(x); free(h); free(q); free(xb); free(o); free(g1); free(g2); free(att); free(tab);
+    return best;
+}
+
+/* h_prev of a chained draft: post-projection of the head's own post-norm hidden
+ * (src/cuda/mtp-kernel.cuh:372-389).  Returns -1 when the file has no post-projection. */
+int lgo_mtp_post(struct lgo_mtp *t, const float *hidden, int mode, float *h_out) {
+    if (!t->post) return -1;
+    if (mode == LGO_REF) { lgo_matmul_f32(t->post->data, t->post->type, t->n_inner, t->n_bb, hidden, h_out); return 0; }
+    struct qact a = { malloc((size_t)t->n_inner), malloc((size_t)t->n_inner / 32 * 4) };
+    quant_into(&a, hidden, t->n_inner);
+    mm(t->post, t->n_inner, t->n_bb, &a, h_out);
+    free(a.q); free(a.d);
+    return 0;
+}
+
+/* The verify step as the DEVICE runs it: every row goes through the decoder (so the cache rows of
+ * rejected drafts are written too), then the accept rule.  Same result as lgo_forward_spec for
+ * out[0..adv-1] and adv; differs in what the cache holds at pos+adv .. pos+rows-1 afterwards, which
+ * only a chained draft ever reads. */
+int lgo_forward_spec_all(struct lgo_model *o, struct lgo_kv *kv, const int *toks, int rows, int pos,
+                         int mode, int *out, float *hidden) {
+    float *hrow = malloc((size_t)o->m.cfg.n_embd * 4 * (size_t)rows);
+    for (int j = 0; j < rows; j++) out[j] = lgo_forward(o, kv, toks[j], pos + j, mode, NULL, hrow + (size_t)j * o->m.cfg.n_embd);
+    const int adv = lgo_accept(toks, out, rows);
+    if (hidden) memcpy(hidden, hrow + (size_t)(adv - 1) * o->m.cfg.n_embd, (size_t)o->m.cfg.n_embd * 4);
+    free(hrow);
+    return adv;
+}

@@ -67,5 +67,18 @@ void  lgo_prefill(struct lgo_model *m, struct lgo_kv *kv, const int *tokens, int
 int   lgo_forward_spec(struct lgo_model *m, struct lgo_kv *kv, const int *toks, int rows, int pos,
                        int mode, int *out, float *hidden);
 void  lgo_set_threads(int n);
+/* the verify step as the device runs it: all rows forwarded (cache rows of rejected drafts
+ * written), then the accept rule */
+int   lgo_forward_spec_all(struct lgo_model *m, struct lgo_kv *kv, const int *toks, int rows, int pos,
+                           int mode, int *out, float *hidden);
+
+/* ---- draft head (src/mtp.c; device form src/cuda/mtp-kernel.cuh:272-402) -------------- */
+struct lgo_mtp;
+struct lgo_mtp *lgo_mtp_open(const char *gguf_path, const struct lgo_model *target);
+void  lgo_mtp_close(struct lgo_mtp *t);
+int   lgo_mtp_info(const struct lgo_mtp *t, int32_t *out, int cap);   /* n_layer,n_inner,n_bb,n_vocab,n_head,n_ff,has_post */
+int   lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv, int token, int pos,
+                    const float *h_prev, int mode, float *hidden_out, float *logits_out);
+int   lgo_mtp_post(struct lgo_mtp *t, const float *hidden, int mode, float *h_out);
 
 #endif

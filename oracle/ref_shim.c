@@ -1,7 +1,7 @@
 /* ref_shim.c — thin ctypes-friendly entry points around the REFERENCE's own CPU backend.
  *
  * TEST INFRASTRUCTURE ONLY.  This file is compiled together with the reference's
- * src/gguf.c, src/quant.c, src/model.c and src/cpu/model-cpu.c, taken from where they lie
+ * src/gguf.c, src/quant.c, src/model.c, src/cpu/model-cpu.c and src/mtp.c, taken from where they lie
  * (see Makefile target _ref), into oracle/_ref/libref_n<N>.so; no reference source is copied
  * into this repository.  It supplies the one symbol those files expect from the CLI
  * (model_pick, src/run.c:83) and flattens the structs for Python.
@@ -10,6 +10,7 @@
 #include <string.h>
 #include "model.h"
 #include "quant.h"
+#include "mtp-internal.h"
 
 int (*model_pick)(const float *logits, int n) = NULL;
 
@@ -57,3 +58,12 @@ int ref_forward_spec(struct ref_handle *h, struct kvcache *kv, const int *toks, 
 }
 void ref_last_hidden(struct ref_handle *h, float *out) { memcpy(out, h->m.last_hidden, (size_t)h->m.cfg.n_embd * 4); }
 int ref_dequantize(unsigned type, const void *src, float *out, long long n) { return dequantize_into(type, src, out, n) ? 0 : -1; }
+
+/* the reference's host draft (src/mtp.c:258-356): it reads m.last_hidden, which the forwards above keep */
+struct mtp *ref_mtp_open(struct ref_handle *h, const char *path) { return mtp_open(path, &h->m); }
+void ref_mtp_free(struct mtp *t) { mtp_free(t); }
+int  ref_mtp_draft(struct ref_handle *h, struct mtp *t, struct kvcache *kv, int token, int pos) { return mtp_draft(t, &h->m, kv, token, pos); }
+int  ref_mtp_n_vocab(struct mtp *t) { return t->n_vocab; }
+int  ref_mtp_n_inner(struct mtp *t) { return t->n_inner; }
+void ref_mtp_logits(struct mtp *t, float *out) { memcpy(out, t->logits, (size_t)t->n_vocab * 4); }
+void ref_mtp_hidden(struct mtp *t, float *out) { memcpy(out, t->x, (size_t)t->n_inner * 4); }
