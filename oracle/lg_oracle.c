@@ -20,6 +20,15 @@
  *                                  The composition (quantization points, op order) is held by the measured
  *                                  gap to LGO_REF staying inside the q8 noise band and by spec == decode
  *                                  (tests/test_oracle_model.py).
+ *   lgo_mtp_draft(LGO_REF)         bit-identical tokens, hidden state and logits against the reference's host
+ *                                  draft head (src/mtp.c, in oracle/_ref) and its committed fixtures
+ *                                  (tests/test_oracle_draft.py), including that file's f16 subnormal reading
+ *   lgo_mtp_draft(LGO_I8), lgo_mtp_post   same code path with q8 activations and this build's orders; the
+ *                                  reference's device draft (f16 weights, CUDA sums) cannot run here: PARITY
+ *                                  UNPINNED for its last bits and for the chained draft's post-projection,
+ *                                  which has no CPU counterpart in the reference.  Held by the gap to LGO_REF
+ *                                  and by the key-range test (a draft at pos reads positions < pos only).
+ *   lgo_forward_spec_all           equal to lgo_forward_spec in adv, out[0..adv-1] and hidden
  */
 #define _GNU_SOURCE
 #include <stdio.h>

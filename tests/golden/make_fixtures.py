@@ -8,6 +8,11 @@ Outputs (data only):
   ref_<model>.npz       model spec hash, prompt, per-step greedy tokens of the reference `run` path
                         (model_prefill + model_forward_next), full logits of a few steps,
                         last_hidden of the final step, and a model_forward_spec transcript
+  ref_draft_<model>.npz the reference's host draft head (src/mtp.c mtp_draft) on a generated
+                        gemma4-assistant file: 16 decode steps, after each one the drafted token,
+                        the head's post-norm hidden and, for three steps, its full logits
+
+Usage: make_fixtures.py [all | model | draft]
 """
 import hashlib
 import importlib
@@ -88,5 +93,44 @@ def main():
         ref.kv_free(kv); ref.kv_free(kv2); ref.close()
 
 
+def draft_fixtures():
+    assert ob.ref_available(4), "build the reference first: make -C oracle ref"
+    for name, spec in MODELS.items():
+        path, head = f"/tmp/lg_golden_{name}.gguf", f"/tmp/lg_golden_{name}_assistant.gguf"
+        lg.synth.write_model(path, **spec)
+        aspec = lg.synth.assistant_for(spec)
+        lg.synth.write_assistant(head, **aspec)
+        ref = ob.Reference(path, 4)
+        t = ref.mtp_open(head)
+        kv = ref.kv_new(N_PROMPT + 32)
+        prng = np.random.default_rng(spec["seed"] + 2)
+        prompt = prng.integers(0, spec["n_vocab"], N_PROMPT).astype(np.int32)
+        ref.prefill(kv, prompt[:-1], 0)
+        tok, pos = int(prompt[-1]), N_PROMPT - 1
+        chosen, drafts, hiddens, logits = [], [], [], {}
+        for step in range(16):
+            tok = ref.forward_next(kv, tok, pos)          # chosen token, will sit at pos + 1
+            pos += 1
+            d, h, row = ref.mtp_draft(t, kv, tok, pos)
+            chosen.append(tok); drafts.append(d); hiddens.append(h)
+            if step in (0, 7, 15):
+                logits[step] = row
+        np.savez_compressed(
+            os.path.join(HERE, f"ref_draft_{name}.npz"),
+            spec_json=np.frombuffer(json.dumps(spec, sort_keys=True).encode(), np.uint8),
+            assistant_json=np.frombuffer(json.dumps(aspec, sort_keys=True).encode(), np.uint8),
+            gguf_sha256=np.frombuffer(sha256(path).encode(), np.uint8),
+            assistant_sha256=np.frombuffer(sha256(head).encode(), np.uint8),
+            prompt=prompt, chosen=np.array(chosen, np.int32), drafts=np.array(drafts, np.int32),
+            hidden=np.stack(hiddens), logit_steps=np.array(sorted(logits), np.int32),
+            logits=np.stack([logits[s] for s in sorted(logits)]))
+        print(name, "chosen", chosen[:8], "drafts", drafts[:8], "accepted", sum(int(drafts[i] == chosen[i + 1]) for i in range(15)))
+        ref.mtp_free(t); ref.kv_free(kv); ref.close()
+
+
 if __name__ == "__main__":
-    main()
+    what = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if what in ("all", "model"):
+        main()
+    if what in ("all", "draft"):
+        draft_fixtures()
