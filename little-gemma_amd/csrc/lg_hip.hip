@@ -15,6 +15,7 @@
 
 #include "../../include/lg_hip.h"
 #include "lg_kernels.h"
+#include "lg_mfma.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
 
@@ -130,7 +131,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -397,9 +398,9 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (max_rows != 1) return fail(-2, "model_commit: a draft head runs one row at a time");
     }
     m->host.clear();
-    const size_t R = (size_t)max_rows;
+    const size_t R = (size_t)(max_rows > LG_WIDE ? max_rows : LG_WIDE);      // prefill runs blocks of LG_WIDE rows
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
-        dev_alloc(m, &m->dout, R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
+        dev_alloc(m, &m->dout, 4 * R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
         dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4) ||
         dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
         dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
@@ -409,7 +410,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
     HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
     m->sched_cap = 4096;
-    if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
+    if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS + LG_WIDE) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
         dev_alloc(m, &m->adv, (size_t)m->sched_cap))
         return -7;
     HIP_TRY(hipHostMalloc((void **)&m->pin, 256 * sizeof(int32_t), hipHostMallocDefault));
@@ -450,7 +451,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         kv->kv_dim[L] = y.kd;
         if (y.hd > max_hd) max_hd = y.hd;
         const bool ring = y.is_local && m->window > 0;
-        const int span = ring ? m->window + LG_HIP_MAX_ROWS : max_seq;       // keys any block can touch
+        const int span = ring ? m->window + LG_WIDE : max_seq;                 // keys any block can touch
         int t = (span < max_seq ? span : max_seq) / 32 + 2;
         if (t > tiles) tiles = t;
         if (!y.owns) continue;
@@ -461,7 +462,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         (void)hipMemset(kv->k[L], 0, bytes); (void)hipMemset(kv->v[L], 0, bytes);
     }
     kv->tiles_max = tiles;
-    const size_t slots = (size_t)m->max_rows * m->H * tiles;
+    const size_t slots = (size_t)(m->max_rows > LG_WIDE ? m->max_rows : LG_WIDE) * m->H * tiles;
     if (hipMalloc((void **)&kv->pm, slots * 4) != hipSuccess || hipMalloc((void **)&kv->pl, slots * 4) != hipSuccess ||
         hipMalloc((void **)&kv->pacc, slots * max_hd * 4) != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory for attention partials"); }
     HIP_TRY(hipDeviceSynchronize());
@@ -594,6 +595,13 @@ struct Launcher {
 template <int M, bool DUMP>
 static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
     const int S = lg_segments(a.k), rw = 64 / S, ngroups = a.m / rw;
+    if constexpr (M > LG_HIP_MAX_ROWS) {                 // wide (prefill) block: matrix-core kernels, 32 weight rows per workgroup
+        if (a.m % 32) { lx.rc = fail(-2, "wide matmul: %d rows is not a multiple of 32", a.m); return; }
+        // S = 32: four workgroups per row block, each a quarter of the K segments, writing its own slab of a.out
+        const dim3 grid(a.m / 32, (M + LG_WIDE - 1) / LG_WIDE, S == 32 ? 4 : 1);
+        if (S == 32) LAUNCH(cls, (lg_k_mm_wide<M, 32, DUMP>), grid, dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+        else         LAUNCH(cls, (lg_k_mm_wide<M, 8, DUMP>), grid, dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+    } else {
     const size_t lds = lds_mm(M, a.k);
     if (S == 32) {
         const int W = 4;
@@ -605,6 +613,8 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
         const int W = ngroups >= 1024 ? 2 : 1;
         LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
     }
+    }
+    (void)rw; (void)ngroups;
 }
 
 // one block of M rows through the decoder (and the head when with_head)
@@ -615,6 +625,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     int cur = 0;                                   // x[cur] holds the residual
     bool have_x = false;                           // false: rows are still token ids
     const float *pend_dout = nullptr, *pend_w = nullptr, *pend_os = nullptr;   // sub-layer output waiting to be added
+    int pend_parts = 1;                            // 4 when that output is four slabs of partial sums (wide ffn_down)
     const bool draft = m->target != nullptr;
     const int pos_off = draft ? -1 : 0;            // a draft at pos sees the cache as a query at pos-1 (src/cuda/mtp-kernel.cuh:170-182)
     if (draft) {
@@ -641,12 +652,12 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq;
         if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
-        s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os;
+        s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os; s.dparts = pend_parts;
         s.w_pre = w_pre; s.h_out = h_out;
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
         LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M), dim3(LG_WG), 0, s, m->ctl);
         if (s.x_out) cur ^= 1;
-        have_x = true; pend_dout = pend_w = pend_os = nullptr;
+        have_x = true; pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
     };
 
     if (m->ple) {
@@ -689,10 +700,14 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         {   // feed-forward: gate/up + GeGLU, then down
             rows(y.ffn_norm, nullptr);
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
-            LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M, 4>), dim3(y.nff / 32), dim3(256), lds_mm(M, E), a);
+            if constexpr (M > LG_HIP_MAX_ROWS)
+                LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+            else
+                LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M, 4>), dim3(y.nff / 32), dim3(256), lds_mm(M, E), a);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
             launch_mm<M, false>(lx, KC_DOWN, d);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
+            pend_parts = (M > LG_HIP_MAX_ROWS && lg_segments(y.nff) == 32) ? 4 : 1;
         }
         if (m->ple) {   // per-layer embedding block
             rows(nullptr, nullptr);
@@ -702,12 +717,20 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
             a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
             a.pq = m->pq;
-            LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E), a, m->ctl);
+            if constexpr (M > LG_HIP_MAX_ROWS)
+                LAUNCH(KC_PLEGATE, (lg_k_mm_plegate_wide<M>), dim3(m->ple / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, m->ctl, M);
+            else
+                LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E), a, m->ctl);
             MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, nullptr };
             launch_mm<M, false>(lx, KC_PLEPROJ, p);
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
         }
     }
+    if constexpr (M > LG_HIP_MAX_ROWS) {
+        if (with_head) return fail(-2, "a wide block has no head: verify blocks hold at most %d rows", LG_HIP_MAX_ROWS);
+        if (!lx.rc && !dry) hipLaunchKernelGGL(lg_k_advance, dim3(1), dim3(1), 0, m->stream, m->ctl, M);
+        return lx.rc;
+    } else
     if (with_head && !lx.rc) {
         rows(m->output_norm, m->hidden_rows);
         int grid = 512;                                  // two workgroups per CU, each walks `passes` blocks of 64 rows
@@ -734,6 +757,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
         case 6: return enqueue_step<6>(m, kv, with_head, dry);
         case 7: return enqueue_step<7>(m, kv, with_head, dry);
         case 8: return enqueue_step<8>(m, kv, with_head, dry);
+        case LG_WIDE: return enqueue_step<LG_WIDE>(m, kv, with_head, dry);
     }
     return fail(-2, "rows %d outside 1..%d", rows, LG_HIP_MAX_ROWS);
 }
@@ -762,9 +786,9 @@ static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head)
     return 0;
 }
 
-static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int rows, int pos) {
+static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int rows, int pos, bool wide = false) {
     if (!m || !kv || !toks || kv->m != m) return fail(-1, "bad model / cache / token pointer");
-    if (rows < 1 || rows > m->max_rows) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
+    if (rows < 1 || (rows > m->max_rows && !(wide && rows == LG_WIDE))) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
     if (pos < 0 || pos + rows > kv->max_seq) return fail(-2, "positions %d..%d do not fit a cache of %d", pos, pos + rows - 1, kv->max_seq);
     for (int i = 0; i < n; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "token id %d outside the vocabulary of %d", toks[i], m->n_vocab);
     return 0;
@@ -774,6 +798,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     if (!m || !name) return fail(-1, "set_option: null argument");
     if (!strcmp(name, "store_logits")) m->store_logits = value != 0;
     else if (!strcmp(name, "use_graph")) m->use_graph = value != 0;
+    else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
 }
@@ -849,9 +874,15 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
     if (n <= 0) return 0;
     if (!m) return fail(-1, "prefill: null model");
     HIP_TRY(hipSetDevice(m->device));
+    bool wide_ok = !m->target && m->wide_prefill;
+    for (int L = 0; L < m->n_layer && wide_ok; ++L) {
+        const Layer &y = m->L[L];
+        wide_ok = y.qkv_m % 32 == 0 && y.nff % 32 == 0;
+    }
     for (int done = 0; done < n;) {
-        const int rows = n - done < m->max_rows ? n - done : m->max_rows;
-        int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done);
+        int rows = n - done < m->max_rows ? n - done : m->max_rows;
+        if (wide_ok && n - done >= LG_WIDE) rows = LG_WIDE;      // matrix-core blocks while the prompt lasts, verify-width blocks for the tail
+        int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done, true);
         if (rc) return rc;
         if ((rc = load_block(m, toks + done, rows, pos0 + done))) return rc;
         if ((rc = launch_step(m, kv, rows, false))) return rc;
@@ -1030,8 +1061,9 @@ static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, cons
 extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *x, int rows, float *out, int32_t *dots,
                                   int8_t *xq, float *xd, int32_t *xsum, int repeats, float *kernel_ms) {
     if (!w || !x) return fail(-1, "matmul: null input");
-    if (rows < 1 || rows > LG_HIP_MAX_ROWS || !lg_hip_repacked_bytes(k, mrows) || lds_mm(rows, k) > 160 * 1024)
-        return fail(-2, "matmul: rows %d (1..%d), k %d (multiple of 256, rows*k*1.25 <= 160 KiB), m %d (multiple of 8)", rows, LG_HIP_MAX_ROWS, k, mrows);
+    const bool wide = rows == LG_WIDE;                   // one full row tile through the matrix-core kernel
+    if (rows < 1 || (rows > LG_HIP_MAX_ROWS && !wide) || !lg_hip_repacked_bytes(k, mrows) || (!wide && lds_mm(rows, k) > 160 * 1024) || (wide && mrows % 32))
+        return fail(-2, "matmul: rows %d (1..%d, or %d with m %% 32 == 0), k %d (multiple of 256, rows*k*1.25 <= 160 KiB), m %d (multiple of 8)", rows, LG_HIP_MAX_ROWS, LG_WIDE, k, mrows);
     if (lg_hip_device_count() < 1) return fail(-3, "matmul: no HIP device");
     const int nb = k / 32;
     std::vector<uint8_t> tiled(lg_hip_repacked_bytes(k, mrows));
@@ -1039,7 +1071,7 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     if (rc) return rc;
     Scratch sc;
     uint8_t *dw; float *dx, *dout; int32_t *ddots = nullptr; int8_t *dq;
-    if (sc.get(&dw, tiled.size()) || sc.get(&dx, (size_t)rows * k) || sc.get(&dout, (size_t)rows * mrows) ||
+    if (sc.get(&dw, tiled.size()) || sc.get(&dx, (size_t)rows * k) || sc.get(&dout, (size_t)rows * mrows * 4) ||
         sc.get(&dq, (size_t)rows * k * 5 / 4)) return -7;
     if (dots && sc.get(&ddots, (size_t)rows * mrows * nb)) return -7;
     HIP_TRY(hipMemcpy(dw, tiled.data(), tiled.size(), hipMemcpyHostToDevice));
@@ -1048,12 +1080,17 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
     switch (rows) {
 #define CASE(M) case M: rc = matmul_rows<M>(st, dw, k, mrows, dx, dout, ddots, dq, repeats, kernel_ms); break;
-        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(LG_WIDE)
 #undef CASE
     }
     (void)hipStreamDestroy(st);
     if (rc) return rc;
-    if (out) HIP_TRY(hipMemcpy(out, dout, (size_t)rows * mrows * 4, hipMemcpyDeviceToHost));
+    if (out && wide && lg_segments(k) == 32) {             // four slabs of partial sums: the top of the segment tree is added here
+        std::vector<float> parts((size_t)4 * rows * mrows);
+        HIP_TRY(hipMemcpy(parts.data(), dout, parts.size() * 4, hipMemcpyDeviceToHost));
+        const size_t n = (size_t)rows * mrows;
+        for (size_t i = 0; i < n; ++i) out[i] = (parts[i] + parts[n + i]) + (parts[2 * n + i] + parts[3 * n + i]);
+    } else if (out) HIP_TRY(hipMemcpy(out, dout, (size_t)rows * mrows * 4, hipMemcpyDeviceToHost));
     if (dots) HIP_TRY(hipMemcpy(dots, ddots, (size_t)rows * mrows * nb * 4, hipMemcpyDeviceToHost));
     // the device keeps activation rows in the matmul's own order (lg_act_layout); hand them back in natural order
     const ActLayout lay = lg_act_layout(k);
@@ -1061,14 +1098,19 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
         std::vector<int8_t> dev((size_t)rows * k);
         HIP_TRY(hipMemcpy(dev.data(), dq, dev.size(), hipMemcpyDeviceToHost));
         for (int j = 0; j < rows; ++j)
-            for (int w = 0; w < k / 16; ++w) memcpy(xq + (size_t)j * k + (size_t)w * 16, dev.data() + (size_t)j * k + (size_t)lg_act_unit(lay, w) * 16, 16);
+            for (int w = 0; w < k / 16; ++w) {
+                const int u = lg_act_unit(lay, w);
+                if (!wide) { memcpy(xq + (size_t)j * k + (size_t)w * 16, dev.data() + (size_t)j * k + (size_t)u * 16, 16); continue; }
+                for (int hh = 0; hh < 2; ++hh)           // wide layout: halves of a unit of all 32 rows side by side
+                    memcpy(xq + (size_t)j * k + (size_t)w * 16 + hh * 8, dev.data() + ((size_t)(u * 2 + hh) * 32 + j) * 8, 8);
+            }
     }
     if (xd || xsum) {
         std::vector<float2> ds((size_t)rows * nb);
         HIP_TRY(hipMemcpy(ds.data(), dq + (size_t)rows * k, ds.size() * 8, hipMemcpyDeviceToHost));
         for (int j = 0; j < rows; ++j)
             for (int b = 0; b < nb; ++b) {
-                const float2 v = ds[(size_t)j * nb + lg_act_block(lay, b)];
+                const float2 v = wide ? ds[(size_t)lg_act_block(lay, b) * 32 + j] : ds[(size_t)j * nb + lg_act_block(lay, b)];
                 if (xd) xd[(size_t)j * nb + b] = v.x;
                 if (xsum) memcpy(&xsum[(size_t)j * nb + b], &v.y, 4);
             }
@@ -1132,7 +1174,7 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     int rc = 0;
     switch (rows) {
 #define CASE(M) case M: rc = attention_rows<M>(st, a, g, ctl, tiles, repeats, kernel_ms); break;
-        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(LG_WIDE)
 #undef CASE
     }
     (void)hipStreamDestroy(st);

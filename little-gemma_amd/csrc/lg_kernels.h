@@ -28,6 +28,7 @@ struct StepCtl {            // device-resident step state
 struct RowArgs {
     const float   *x;        // [M][E] residual stream; nullptr when the rows are embeddings
     const float   *dout;     // [M][E] previous sub-layer output to be rmsnormed and added, or nullptr
+    int            dparts;   // 4: dout is four [M][E] slabs of partial sums, added here as (p0+p1)+(p2+p3); else 1
     const float   *w_post;   // [E] norm weight for dout
     const float   *os;       // scalar layer_output_scale applied after the add, or nullptr
     float         *x_out;    // [M][E] updated residual, or nullptr
@@ -58,6 +59,23 @@ template <int M>
 __device__ __forceinline__ const float2 *lg_q8_ds(const int8_t *q, int k) { return (const float2 *)(q + (size_t)M * k); }
 template <int M>
 __device__ __forceinline__ float2 *lg_q8_ds(int8_t *q, int k) { return (float2 *)(q + (size_t)M * k); }
+// Where row j keeps byte `byte` of its natural 16-byte unit w, and the {scale, sum} pair of block b.
+// Blocks of up to LG_HIP_MAX_ROWS_DEV rows: row-major rows in the order of lg_act_layout (what the
+// wavefront-dot kernels stage in LDS).  Wider blocks (the matrix-core kernels): tiles of 32 rows, and
+// inside a tile the 8-byte halves of a unit of all 32 rows side by side, so that the 64 lanes of an
+// operand load (row n = lane % 32, half = lane / 32) read 512 consecutive bytes.
+template <int M>
+__device__ __forceinline__ size_t lg_q8_off(int k, int j, int w, int byte) {
+    const int u = lg_act_unit(lg_act_layout(k), w);
+    if (M <= LG_HIP_MAX_ROWS_DEV) return (size_t)j * k + (size_t)u * 16 + byte;
+    return (size_t)(j >> 5) * 32 * k + ((size_t)(u * 2 + (byte >> 3)) * 32 + (j & 31)) * 8 + (byte & 7);
+}
+template <int M>
+__device__ __forceinline__ size_t lg_q8_ds_idx(int k, int j, int b) {
+    const int u = lg_act_block(lg_act_layout(k), b);
+    if (M <= LG_HIP_MAX_ROWS_DEV) return (size_t)j * (k >> 5) + u;
+    return (size_t)(j >> 5) * 32 * (k >> 5) + (size_t)u * 32 + (j & 31);
+}
 #define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
@@ -82,6 +100,15 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         const float4 *dr = (const float4 *)(s.dout + (size_t)j * E), *wr = (const float4 *)s.w_post;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { dv[v] = dr[t + 256 * v]; wpost[v] = wr[t + 256 * v]; }
+        if (s.dparts == 4) {                                 // top of the K-segment tree of a matmul that was split over four workgroups
+            const size_t slab = (size_t)M * nq;
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 p1 = dr[slab + t + 256 * v], p2 = dr[2 * slab + t + 256 * v], p3 = dr[3 * slab + t + 256 * v], p0 = dv[v];
+                dv[v] = make_float4((p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y),
+                                    (p0.z + p1.z) + (p2.z + p3.z), (p0.w + p1.w) + (p2.w + p3.w));
+            }
+        }
     }
     if (s.w_pre) {
         const float4 *wr = (const float4 *)s.w_pre;
@@ -128,9 +155,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ho[t + 256 * v] = xv[v];
     }
-    uint32_t *qrow = (uint32_t *)(s.q + (size_t)j * E);
-    float2 *drow = lg_q8_ds<M>(s.q, E) + (size_t)j * (E >> 5);
-    const ActLayout lay = lg_act_layout(E);
+    float2 *dsb = lg_q8_ds<M>(s.q, E);
     #pragma unroll
     for (int v = 0; v < LG_ROWV; ++v) {
         // nq is a multiple of 64, so a whole wavefront is either inside the row or outside it
@@ -138,8 +163,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
         const int quad = t + 256 * v;                        // 4 values = a quarter of a 16-byte unit
-        qrow[lg_act_unit(lay, quad >> 2) * 4 + (quad & 3)] = packed;
-        if ((t & 7) == 0) drow[lg_act_block(lay, quad >> 3)] = make_float2(d, __int_as_float(sum));
+        *(uint32_t *)(s.q + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
+        if ((t & 7) == 0) dsb[lg_q8_ds_idx<M>(E, j, quad >> 3)] = make_float2(d, __int_as_float(sum));
     }
 }
 
@@ -154,6 +179,11 @@ __global__ __launch_bounds__(LG_WG) void lg_k_quant_flat(const float *x, int row
     const uint32_t packed = lg_quant4_8lanes(h, &d, &sum);
     if (!live) return;
     const int j = g / nb, b = g - j * nb;
+    if (rows > LG_HIP_MAX_ROWS_DEV) {                        // a wide block: the matrix-core kernels' layout
+        *(uint32_t *)(q + lg_q8_off<LG_HIP_MAX_ROWS_DEV + 1>(k, j, b * 2 + (l >> 2), (l & 3) * 4)) = packed;
+        if (l == 0) ds[lg_q8_ds_idx<LG_HIP_MAX_ROWS_DEV + 1>(k, j, b)] = make_float2(d, __int_as_float(sum));
+        return;
+    }
     const ActLayout lay = lg_act_layout(k);
     ((uint32_t *)(q + (size_t)j * k))[lg_act_unit(lay, b * 2 + (l >> 2)) * 4 + (l & 3)] = packed;
     if (l == 0) ds[(size_t)j * nb + lg_act_block(lay, b)] = make_float2(d, __int_as_float(sum));
@@ -809,9 +839,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
         const int q = lg_quant1_32lanes(r, &dq, &sum);
         if (d < hd) {
             const int e = head * hd + d;                       // element of the row, natural order
-            const ActLayout lay = lg_act_layout(qd);          // order the attn_output matmul reads
-            a.xq[(size_t)j * qd + lg_act_unit(lay, e >> 4) * 16 + (e & 15)] = (int8_t)q;
-            if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[(size_t)j * (qd >> 5) + lg_act_block(lay, e >> 5)] = make_float2(dq, __int_as_float(sum));
+            a.xq[lg_q8_off<M>(qd, j, e >> 4, e & 15)] = (int8_t)q;      // order the attn_output matmul reads
+            if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));
             if (a.xf) a.xf[(size_t)j * qd + e] = r;
         }
     }

@@ -1,0 +1,233 @@
+// lg_mfma.h — the q4_0 x q8 matmul for wide row blocks (prefill), on the matrix cores.
+//
+// Same arithmetic and the same float order as the wavefront-dot kernels of lg_kernels.h (so a
+// prompt processed 32 positions at a time leaves bit-identical cache rows): per 32-weight block an
+// exact int32 dot, then p = fma(xd*dw, (float)dot, p) along each of the S contiguous K segments,
+// then the adjacent-pair tree over the segments.  What changes is who computes the dots:
+// one v_mfma_i32_32x32x32_i8 gives the 32 x 32 block dots of 32 weight rows against 32 activation
+// rows for one q4_0 block (K = 32).
+//
+// Operand roles: A = weights (row m = lane % 32 of the 32-row block, k-half h = lane / 32),
+// B = activations (row n = lane % 32 of the row tile, same k-half).  The result register i of lane
+// (n, h) is the dot of activation row n with weight row 8*(i/4) + 4*h + i%4.  A lane's 16 k-values
+// are, for the weights, the two nibbles of the 8 bytes h*8..h*8+7 of the block (elements
+// 8h..8h+7 and 16+8h..16+8h+7), and the same elements of the activation block: any common order
+// of the contraction index gives the same integer.
+//
+// Weights keep the tile layout of lg_device.h.  A workgroup (8 wavefronts, two per SIMD so that the
+// float epilogue of one overlaps the loads of the other) owns one 32-row block and 8 K segments:
+// per step `it` four of its wavefronts load the block's 256 (row, segment) slots (one 16-byte load
+// per lane), park them in LDS in operand order (double buffered, one barrier per step), and every
+// wavefront then runs the one segment it owns.  Activations and their {scale, sum} pairs are read
+// straight from the q8 activation buffer, which producers of wide blocks write in operand order
+// (lg_q8_off: a wavefront's operand load is 512 consecutive bytes).
+#pragma once
+#include "lg_kernels.h"
+
+typedef int lg_v4i __attribute__((ext_vector_type(4)));
+typedef int lg_v16i __attribute__((ext_vector_type(16)));
+
+#define LG_WIDE 32                         // activation rows per row tile
+
+#define LG_WIDE_WG 512                     // 8 wavefronts: two per SIMD, one K segment each
+
+struct MfmaGeo {
+    static constexpr int AW_STRIDE = 33;   // uint2 per (segment, half) row of the operand store (32 + 1 pad)
+    static constexpr size_t aw_bytes = (size_t)8 * 2 * AW_STRIDE * 8;
+    static constexpr size_t dw_bytes = (size_t)8 * 32 * 4;
+    static constexpr int U = 5;            // steps per chunk: tiles and activation operands are requested a chunk ahead
+    static constexpr size_t step_bytes = aw_bytes + dw_bytes;
+    static constexpr size_t lds_bytes = 2 * U * step_bytes;       // double-buffered chunks; the final exchange (32 KiB) reuses it
+};
+static_assert(8 * 16 * 64 * 4 <= MfmaGeo::lds_bytes, "the final exchange must fit");
+
+// One 32-row weight block `rb` against row tile `tile` of the R-row q8 activation buffer, for the 8
+// K segments 8*part .. 8*part+7 (S = 8: part = 0 and that is the whole row; S = 32: one quarter, the
+// caller adds the four partial results in tree order).  Wavefront w owns segment 8*part + w.
+// On return wavefront w, lane (n, h) holds in res[0..1] the finished sums of activation row
+// tile*32 + n and weight rows 32*rb + lg_wide_col(w, h) + {0, 1}.  All 512 threads must call it;
+// `smem` needs MfmaGeo::lds_bytes and is free again on return.
+__device__ __forceinline__ int lg_wide_col(int wave, int h) { return 8 * (wave >> 1) + 4 * h + 2 * (wave & 1); }
+
+template <int R, int S, bool DUMP>
+__device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, int part, const int8_t *q_in, int tile, int rows,
+                                              unsigned char *smem, float (&res)[2], int32_t *dots, int m_total) {
+    using G = MfmaGeo;
+    constexpr int RW = 64 / S, TPB = 32 / RW;                 // weight rows per tile group; tiles per 32-row block and step
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = k >> 5, nit = nb / S;
+    const int n = lane & 31, h = lane >> 5, c = 8 * part + wave;
+    // operands of row tile `tile` in the wide q8 layout (lg_q8_off): per 16-byte unit the two halves of the
+    // 32 rows side by side, so lane (n, h) reads 8 of 512 consecutive bytes; rows past `rows` hold
+    // whatever the buffer holds and their results are dropped by the caller
+    const int8_t *atile = q_in + (size_t)tile * 32 * k + (size_t)(h * 32 + n) * 8;
+    const float2 *dstile = lg_q8_ds<R>(q_in, k) + (size_t)tile * 32 * nb + n;
+
+    // wavefronts 0..3 fetch the step's 256 (row, segment) slots: slot -> tile, lane inside the tile, row of the block
+    const int slot = (wave & 3) * 64 + lane;
+    int st_tile, st_lane, st_m, st_c;
+    if (S == 8) { st_tile = slot >> 6; st_lane = slot & 63; st_m = st_tile * 8 + (st_lane >> 3); st_c = st_lane & 7; }
+    else        { st_tile = slot >> 4; st_c = slot & 7; const int r = (slot >> 3) & 1; st_lane = r * 32 + 8 * part + st_c; st_m = st_tile * 2 + r; }
+    const uint8_t *tbase = w + (size_t)(rb * TPB + st_tile) * nit * LG_TILE;
+    // A chunk of U steps is requested while the previous one is consumed (enough bytes in flight to
+    // cover the memory latency), parked in LDS in one go, and followed by a single barrier.
+    uint4 tq[G::U]; uint32_t ts[G::U];
+    uint2 b0[G::U], b1[G::U], nb0[G::U], nb1[G::U]; float2 xs[G::U], nxs[G::U];
+    auto fetch = [&](int it0) {
+        #pragma unroll
+        for (int u = 0; u < G::U; ++u) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;    // clamp: never read past the row block
+            if (wave < 4) {
+                const uint8_t *t = tbase + (size_t)it * LG_TILE;
+                tq[u] = *(const uint4 *)(t + st_lane * 16);
+                ts[u] = *(const uint16_t *)(t + 1024 + st_lane * 2);
+            }
+            nb0[u] = *(const uint2 *)(atile + (size_t)(it * 2 * S + c) * 512);
+            nb1[u] = *(const uint2 *)(atile + (size_t)(it * 2 * S + S + c) * 512);
+            nxs[u] = dstile[(size_t)(it * S + c) * 32];
+        }
+    };
+    float p[16];
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = 0.0f;
+    fetch(0);
+    for (int it0 = 0; it0 < nit; it0 += G::U) {
+        unsigned char *cbase = smem + (size_t)((it0 / G::U) & 1) * G::U * G::step_bytes;
+        if (wave < 4) {                                       // park in operand order
+            #pragma unroll
+            for (int u = 0; u < G::U; ++u) {
+                uint2 *aw = (uint2 *)(cbase + (size_t)u * G::step_bytes);
+                float *dwf = (float *)((unsigned char *)aw + G::aw_bytes);
+                aw[(st_c * 2 + 0) * G::AW_STRIDE + st_m] = make_uint2(tq[u].x, tq[u].y);
+                aw[(st_c * 2 + 1) * G::AW_STRIDE + st_m] = make_uint2(tq[u].z, tq[u].w);
+                dwf[st_c * 32 + st_m] = lg_h2f((uint16_t)ts[u]);
+            }
+        }
+        #pragma unroll
+        for (int u = 0; u < G::U; ++u) { b0[u] = nb0[u]; b1[u] = nb1[u]; xs[u] = nxs[u]; }
+        if (it0 + G::U < nit) fetch(it0 + G::U);
+        __syncthreads();
+        #pragma unroll
+        for (int u = 0; u < G::U; ++u) {
+            if (it0 + u >= nit) break;
+            const int it = it0 + u;
+            const uint2 *aw = (const uint2 *)(cbase + (size_t)u * G::step_bytes);
+            const float *dwf = (const float *)((const unsigned char *)aw + G::aw_bytes);
+            const uint2 a = aw[(wave * 2 + h) * G::AW_STRIDE + n];
+            lg_v4i av, bv;
+            av[0] = (int)(a.x & 0x0F0F0F0Fu); av[1] = (int)(a.y & 0x0F0F0F0Fu);
+            av[2] = (int)((a.x >> 4) & 0x0F0F0F0Fu); av[3] = (int)((a.y >> 4) & 0x0F0F0F0Fu);
+            bv[0] = (int)b0[u].x; bv[1] = (int)b0[u].y; bv[2] = (int)b1[u].x; bv[3] = (int)b1[u].y;
+            lg_v16i acc = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc, 0, 0, 0);
+            const int corr = 8 * __float_as_int(xs[u].y);
+            #pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 d4 = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
+                const float dv[4] = { d4.x, d4.y, d4.z, d4.w };
+                #pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int dot = acc[4 * g + j] - corr;
+                    if (DUMP) {
+                        const int row = 32 * rb + 8 * g + 4 * h + j;
+                        if (tile * LG_WIDE + n < rows) dots[((size_t)(tile * LG_WIDE + n) * m_total + row) * nb + (c * nit + it)] = dot;
+                    }
+                    p[4 * g + j] = lg_fmaf(xs[u].x * dv[j], (float)dot, p[4 * g + j]);
+                }
+            }
+        }
+    }
+    // adjacent-pair tree over the eight segments (one per wavefront)
+    __syncthreads();
+    float *red = (float *)smem;                              // [8 wavefronts][16][64]
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) red[(wave * 16 + i) * 64 + lane] = p[i];
+    __syncthreads();
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int i = 2 * wave + j;
+        float v[8];
+        #pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = red[(u * 16 + i) * 64 + lane];
+        res[j] = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    }
+    __syncthreads();
+}
+
+// Plain matmul for wide blocks: out[row][i] f32.  grid = (m / 32, row tiles, parts): S = 8 has one
+// part; S = 32 has four, each writing its own [R][m] slab of `out` (the consumer adds them as
+// (p0 + p1) + (p2 + p3), the top of the segment tree).
+template <int R, int S, bool DUMP>
+__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_wide(MmArgs a, int rows) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float res[2];
+    lg_mfma_block<R, S, DUMP>(a.w, a.k, blockIdx.x, blockIdx.z, a.q_in, blockIdx.y, rows, smem, res, a.dots, a.m);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, an = blockIdx.y * LG_WIDE + (lane & 31);
+    if (an < rows)
+        *(float2 *)(a.out + (size_t)blockIdx.z * R * a.m + (size_t)an * a.m + 32 * blockIdx.x + lg_wide_col(wave, lane >> 5)) = make_float2(res[0], res[1]);
+}
+
+// 32 x 32 finished values (activation row, column of this workgroup's block) -> one q8 block per
+// row, written in the activation order of a consumer of width kq.  vbuf: [32][33] floats in LDS.
+template <int R>
+__device__ __forceinline__ void lg_wide_quant32(float *vbuf, int8_t *q, int kq, int block, int tile, int rows) {
+    const int t = threadIdx.x, n = t >> 3, qd = t & 7, an = tile * LG_WIDE + n;
+    if (t >= 256) return;                                    // whole wavefronts leave; the other four stay whole
+    const float4 v = make_float4(vbuf[n * 33 + 4 * qd], vbuf[n * 33 + 4 * qd + 1], vbuf[n * 33 + 4 * qd + 2], vbuf[n * 33 + 4 * qd + 3]);
+    float d; int sum;
+    const uint32_t packed = lg_quant4_8lanes(v, &d, &sum);
+    if (an >= rows) return;
+    const int quad = block * 8 + qd;
+    *(uint32_t *)(q + lg_q8_off<R>(kq, an, quad >> 2, (quad & 3) * 4)) = packed;
+    if (qd == 0) lg_q8_ds<R>(q, kq)[lg_q8_ds_idx<R>(kq, an, block)] = make_float2(d, __int_as_float(sum));
+}
+
+// Gate/up with the GeGLU and the q8 of its result (see lg_k_mm_geglu): the tiled matrix holds, per
+// 32 FFN columns, a block of 32 gate rows followed by the block of the 32 up rows.  grid = (n_ff/32, row tiles).
+template <int R>
+__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_geglu_wide(GegluArgs a, int rows) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float vbuf[32 * 33];
+    float g[2], u[2];
+    lg_mfma_block<R, 8, false>(a.w, a.k, 2 * blockIdx.x, 0, a.q_in, blockIdx.y, rows, smem, g, nullptr, 0);
+    lg_mfma_block<R, 8, false>(a.w, a.k, 2 * blockIdx.x + 1, 0, a.q_in, blockIdx.y, rows, smem, u, nullptr, 0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, col = lg_wide_col(wave, lane >> 5);
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) vbuf[n * 33 + col + j] = lg_gelu(g[j]) * u[j];
+    __syncthreads();
+    lg_wide_quant32<R>(vbuf, a.gq, a.n_ff, blockIdx.x, blockIdx.y, rows);
+}
+
+// PLE gate for wide blocks (see lg_k_mm_plegate): gelu(inp_gate . x) * ipl[layer], q8 of the result.
+// grid = (ple/32, row tiles).
+template <int R>
+__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_plegate_wide(PleGateArgs a, const StepCtl *ctl, int rows) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float vbuf[32 * 33];
+    __shared__ float ipl[32][32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, ple = a.ple;
+    #pragma unroll
+    for (int jj = 0; jj < LG_WIDE / (LG_WIDE_WG / 64); ++jj) {     // fixed trip count: the loads of all rows go out together
+        const int j = wave + jj * (LG_WIDE_WG / 64);
+        int an = blockIdx.y * LG_WIDE + j;
+        if (an >= rows) an = rows - 1;
+        const float *pr = a.pmp_raw + (size_t)an * a.n_layer * ple + (size_t)a.layer * ple;
+        const int tok = a.toks[ctl->step * R + an];
+        const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
+        const int e = blockIdx.x * 32 + (lane & 31);
+        const float4 p4 = 4 * lane < ple ? *(const float4 *)(pr + 4 * lane) : make_float4(0, 0, 0, 0);
+        const float pe = pr[e], wn = a.proj_norm[e];
+        const float tk = lg_q4_0_elem(trow, a.layer * ple + e) * a.tscale;
+        const float4 p = make_float4(p4.x * a.pscale, p4.y * a.pscale, p4.z * a.pscale, p4.w * a.pscale);
+        const float ss = lg_wave_sum64(lg_sumsq4(p, 0.0f));
+        const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
+        if (lane < 32) ipl[j][lane] = (pe * a.pscale * sc * wn + tk) * a.rsqrt2;
+    }
+    float r[2];
+    lg_mfma_block<R, 8, false>(a.w, a.k, blockIdx.x, 0, a.q_in, blockIdx.y, rows, smem, r, nullptr, 0);
+    const int n = lane & 31, col = lg_wide_col(wave, lane >> 5);
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) vbuf[n * 33 + col + j] = lg_gelu(r[j]) * ipl[n][col + j];
+    __syncthreads();
+    lg_wide_quant32<R>(vbuf, a.pq, ple, blockIdx.x, blockIdx.y, rows);
+}
