@@ -136,6 +136,7 @@ def main():
     ap.add_argument("--model-dir", default=os.environ.get("LG_BENCH_DIR", "/tmp"))
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--seed", type=int, default=7)
+    ap.add_argument("--prefill", type=int, default=1024, help="positions of the prompt-processing measurement; 0 skips it")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU; the verify step is not sharded (run with --gpus 1)", file=sys.stderr)
@@ -152,7 +153,7 @@ def main():
         os.replace(path + ".tmp", path)
         log(f"wrote {path} in {time.time() - t0:.1f}s")
     total = a.steps + a.warmup
-    max_seq = ctx + (total + 2) * a.rows + 64
+    max_seq = max(ctx + (total + 2) * a.rows + 64, a.prefill + 64)
     t0 = time.time()
     gpu = lg.hiplib.HipBackend(path, max_seq, max_rows=max(a.rows, 1))
     log(f"weights on the device in {time.time() - t0:.1f}s")
@@ -219,6 +220,21 @@ def main():
         "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
                    "wall_ms_per_step": 1e3 * wall / a.steps, "plain_decode_ms_per_token_host_sync": decode_ms},
     }
+    # prompt processing on the matrix cores: 32-row blocks through the int8 MFMA kernels (a fresh cache, host clock
+    # around a synchronised call; the first call captures the graph and is not timed)
+    if a.prefill > 0:
+        prng = np.random.default_rng(a.seed + 1)
+        ptoks = prng.integers(1, info["n_vocab"], a.prefill).astype(np.int32)
+        gpu.new_cache(max_seq)
+        gpu.prefill(ptoks[:64], 0)
+        gpu.new_cache(max_seq)
+        t0 = time.time()
+        gpu.prefill(ptoks, 0)
+        dt = time.time() - t0
+        macs = sum(c["bytes"] for c in prof if c["name"] != "lm_head" and c["name"] != "attn_tiles") / (18.0 / 32.0)   # weights touched per position
+        line["prefill"] = {"positions": int(a.prefill), "ms": 1e3 * dt, "tok_per_s": a.prefill / dt,
+                           "kernel": "v_mfma_i32_32x32x32_i8, 32-row blocks", "int8_TOPs": 2.0 * macs * a.prefill / dt / 1e12,
+                           "mfma_peak_TOPs": 5000.0, "mfma_utilisation": 2.0 * macs * a.prefill / dt / 5.0e15}
     gpu.close()
     if a.cpu_seconds > 0:
         try:

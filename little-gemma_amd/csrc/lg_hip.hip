@@ -38,7 +38,7 @@ extern "C" int lg_hip_device_count(void) {
     return n;
 }
 extern "C" int lg_hip_ring_rows(int window, int max_seq) {
-    int r = (window + 32 + 31) / 32 * 32;          // window + spare for a block of draft rows, tile multiple
+    int r = (window + LG_WIDE_ROWS + 31) / 32 * 32;   // window + spare for the widest block written before its queries run, tile multiple
     return r < max_seq ? r : max_seq;
 }
 
@@ -398,7 +398,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (max_rows != 1) return fail(-2, "model_commit: a draft head runs one row at a time");
     }
     m->host.clear();
-    const size_t R = (size_t)(max_rows > LG_WIDE ? max_rows : LG_WIDE);      // prefill runs blocks of LG_WIDE rows
+    const size_t R = (size_t)(max_rows > LG_WIDE_ROWS ? max_rows : LG_WIDE_ROWS);      // prefill runs blocks of LG_WIDE_ROWS rows
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
         dev_alloc(m, &m->dout, 4 * R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
         dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4) ||
@@ -410,7 +410,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
     HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
     m->sched_cap = 4096;
-    if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS + LG_WIDE) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
+    if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS + LG_WIDE_ROWS) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
         dev_alloc(m, &m->adv, (size_t)m->sched_cap))
         return -7;
     HIP_TRY(hipHostMalloc((void **)&m->pin, 256 * sizeof(int32_t), hipHostMallocDefault));
@@ -451,7 +451,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         kv->kv_dim[L] = y.kd;
         if (y.hd > max_hd) max_hd = y.hd;
         const bool ring = y.is_local && m->window > 0;
-        const int span = ring ? m->window + LG_WIDE : max_seq;                 // keys any block can touch
+        const int span = ring ? m->window + LG_WIDE_ROWS : max_seq;                 // keys any block can touch
         int t = (span < max_seq ? span : max_seq) / 32 + 2;
         if (t > tiles) tiles = t;
         if (!y.owns) continue;
@@ -462,7 +462,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         (void)hipMemset(kv->k[L], 0, bytes); (void)hipMemset(kv->v[L], 0, bytes);
     }
     kv->tiles_max = tiles;
-    const size_t slots = (size_t)(m->max_rows > LG_WIDE ? m->max_rows : LG_WIDE) * m->H * tiles;
+    const size_t slots = (size_t)(m->max_rows > LG_WIDE_ROWS ? m->max_rows : LG_WIDE_ROWS) * m->H * tiles;
     if (hipMalloc((void **)&kv->pm, slots * 4) != hipSuccess || hipMalloc((void **)&kv->pl, slots * 4) != hipSuccess ||
         hipMalloc((void **)&kv->pacc, slots * max_hd * 4) != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory for attention partials"); }
     HIP_TRY(hipDeviceSynchronize());
@@ -758,6 +758,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
         case 7: return enqueue_step<7>(m, kv, with_head, dry);
         case 8: return enqueue_step<8>(m, kv, with_head, dry);
         case LG_WIDE: return enqueue_step<LG_WIDE>(m, kv, with_head, dry);
+        case LG_WIDE_ROWS: return enqueue_step<LG_WIDE_ROWS>(m, kv, with_head, dry);
     }
     return fail(-2, "rows %d outside 1..%d", rows, LG_HIP_MAX_ROWS);
 }
@@ -788,7 +789,7 @@ static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head)
 
 static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int rows, int pos, bool wide = false) {
     if (!m || !kv || !toks || kv->m != m) return fail(-1, "bad model / cache / token pointer");
-    if (rows < 1 || (rows > m->max_rows && !(wide && rows == LG_WIDE))) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
+    if (rows < 1 || (rows > m->max_rows && !(wide && (rows == LG_WIDE || rows == LG_WIDE_ROWS)))) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
     if (pos < 0 || pos + rows > kv->max_seq) return fail(-2, "positions %d..%d do not fit a cache of %d", pos, pos + rows - 1, kv->max_seq);
     for (int i = 0; i < n; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "token id %d outside the vocabulary of %d", toks[i], m->n_vocab);
     return 0;
@@ -881,7 +882,8 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
     }
     for (int done = 0; done < n;) {
         int rows = n - done < m->max_rows ? n - done : m->max_rows;
-        if (wide_ok && n - done >= LG_WIDE) rows = LG_WIDE;      // matrix-core blocks while the prompt lasts, verify-width blocks for the tail
+        if (wide_ok && n - done >= LG_WIDE_ROWS) rows = LG_WIDE_ROWS;     // matrix-core blocks while the prompt lasts,
+        else if (wide_ok && n - done >= LG_WIDE) rows = LG_WIDE;        // a single row tile, then verify-width blocks for the tail
         int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done, true);
         if (rc) return rc;
         if ((rc = load_block(m, toks + done, rows, pos0 + done))) return rc;

@@ -268,11 +268,11 @@ int lgo_accept(const int *toks, const int *out, int rows) {
     return adv;
 }
 
-/* sliding-window ring length of the int8 class: the window plus spare rows for a block of
- * draft rows written before any query runs (src/cuda/model-cuda.cuh:1016-1035 uses
+/* sliding-window ring length of the int8 class: the window plus spare rows for the widest block
+ * (128 prompt rows, or a few draft rows) written before any of its queries runs (src/cuda/model-cuda.cuh:1016-1035 uses
  * window + widest chunk), rounded to the 32-key attention tile */
 int lgo_ring_rows(int window, int max_seq) {
-    int r = (window + 32 + 31) / 32 * 32;
+    int r = (window + 128 + 31) / 32 * 32;
     return r < max_seq ? r : max_seq;
 }
 
