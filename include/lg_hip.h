@@ -80,7 +80,9 @@ int  lg_hip_kv_restore_prefix(lg_hip_kv *kv, int n);
 int  lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n_rows, int pos,
                          int32_t *out, int32_t *adv);
 /* model_prefill (include/model.h:121): positions pos0..pos0+n-1, cache writes only, no head.
- * Runs as blocks of up to max_rows rows through the same kernels as the verify step. */
+ * Runs as blocks of 128 rows whose matmuls use the int8 matrix cores (the reference's chunked
+ * prefill, src/cuda/prefill-kernel.cuh:631-675), then one 32-row block, then verify-width blocks
+ * for the tail; every block leaves the cache rows that position-by-position decode would. */
 int  lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int pos0);
 /* Post-output-norm hidden state of the last valid row of the latest verify step (n_embd
  * floats): what the reference keeps in g_hidden / model.last_hidden for the draft head
@@ -92,7 +94,8 @@ int  lg_hip_set_hidden_row(lg_hip_model *m, int row);
 /* Soft-capped logits of row `row` of the latest step (n_vocab floats).  Only stored while the
  * "store_logits" option is on (model_forward, include/model.h:98, needs them; the verify does not). */
 int  lg_hip_get_logits(lg_hip_model *m, int row, float *dst);
-/* Options: "store_logits" (0/1, default 0), "use_graph" (0/1, default 1). */
+/* Options: "store_logits" (0/1, default 0), "use_graph" (0/1, default 1), "wide_prefill" (0/1,
+ * default 1: 0 sends the whole prompt through verify-width blocks). */
 int  lg_hip_set_option(lg_hip_model *m, const char *name, int value);
 
 /* ---- draft head: the gemma4-assistant network on the device (mtp_draft_device,
