@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 lg = importlib.import_module("little-gemma_amd")
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel (gate/up + GeGLU at the E4B shape), from the FETCH_SIZE and
+# WRITE_SIZE counter runs summarised under profiles/ (scaled by the copy-kernel calibration given there):
+# reads 29.41 MB for M = 5 (29.26 MB for M = 1), writes 0.15 MB.  Other shapes have no counter run.
+MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.41e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.26e6 + 0.03e6}
 CTX = 2048
 WORKLOADS = {
     "e4b": ("E4B-shape q4_0 verify step (42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144, "
@@ -202,7 +206,8 @@ def main():
     dom = max((c for c in prof if c["bytes"] > 0), key=lambda c: c["ms"])
     dom_gbs = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom["name"], "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": dom_gbs / HBM_PEAK_GBS, "traffic": None,
+                "frac": dom_gbs / HBM_PEAK_GBS,
+                "traffic": MEASURED_TRAFFIC.get((a.workload, dom["name"], a.rows)),
                 "bytes_per_launch": dom["bytes"] / max(dom["launches"], 1), "ms_per_launch": dom["ms"] / max(dom["launches"], 1),
                 "launches_per_step": dom["launches"]}
     step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9
