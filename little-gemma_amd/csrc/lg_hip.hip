@@ -75,6 +75,29 @@ static void repack_rows(const uint8_t *const *rows, int k, int m, uint8_t *dst) 
     for (auto &th : pool) th.join();
 }
 
+// Row-block tiles (lg_k_geglu_t): tile (64-row block, kb) holds for lane r the 16 nibble bytes of block kb
+// of row 64*block + r, then the 64 f16 scales; tiles ordered [block][kb].  Same size as the segment tiles.
+static void repack_rowblocks(const uint8_t *const *rows, int k, int m, uint8_t *dst) {
+    const int nb = k / 32, blocks = m / 64;
+    auto work = [&](int b0, int b1) {
+        for (int b = b0; b < b1; ++b)
+            for (int kb = 0; kb < nb; ++kb) {
+                uint8_t *tile = dst + ((size_t)b * nb + kb) * LG_TILE;
+                for (int r = 0; r < 64; ++r) {
+                    const uint8_t *blk = rows[b * 64 + r] + (size_t)kb * 18;
+                    memcpy(tile + r * 16, blk + 2, 16);
+                    memcpy(tile + 1024 + r * 2, blk, 2);
+                }
+            }
+    };
+    unsigned hw = std::thread::hardware_concurrency();
+    int nt = (int)(hw ? (hw > 16 ? 16 : hw) : 4);
+    if ((size_t)blocks * nb < 4096 || nt < 2) { work(0, blocks); return; }
+    std::vector<std::thread> pool;
+    for (int t = 0; t < nt; ++t) pool.emplace_back(work, (int)((long long)blocks * t / nt), (int)((long long)blocks * (t + 1) / nt));
+    for (auto &th : pool) th.join();
+}
+
 extern "C" int lg_hip_repack_q4_0(const void *src, int k, int m, void *dst) {
     if (!lg_hip_repacked_bytes(k, m)) return fail(-2, "repack: k=%d must be a multiple of 256 (1024 above 4096) and m=%d of 8", k, m);
     std::vector<const uint8_t *> rows((size_t)m);
@@ -232,11 +255,12 @@ static int check_mat(const HostTensor *t, const std::string &name, uint64_t k, u
 }
 // upload a tiled matrix whose virtual rows are given by `rows`
 static int upload_tiled(lg_hip_model *m, const std::vector<const uint8_t *> &rows, int k, uint8_t **out,
-                        std::vector<uint8_t> &stage) {
+                        std::vector<uint8_t> &stage, bool rowblocks = false) {
     const size_t bytes = lg_hip_repacked_bytes(k, (int)rows.size());
-    if (!bytes) return fail(-6, "model_commit: cannot tile a %zu x %d matrix", rows.size(), k);
+    if (!bytes || (rowblocks && (rows.size() % 64 || lg_segments(k) != 8))) return fail(-6, "model_commit: cannot tile a %zu x %d matrix", rows.size(), k);
     stage.resize(bytes);
-    repack_rows(rows.data(), k, (int)rows.size(), stage.data());
+    if (rowblocks) repack_rowblocks(rows.data(), k, (int)rows.size(), stage.data());
+    else repack_rows(rows.data(), k, (int)rows.size(), stage.data());
     if (dev_alloc(m, out, bytes)) return -7;
     HIP_TRY(hipMemcpy(*out, stage.data(), bytes, hipMemcpyHostToDevice));
     m->weight_bytes += bytes;
@@ -350,7 +374,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if ((rc = check_mat(u, lname(L, "ffn_up.weight"), E, y.nff))) return rc;
         if ((rc = check_mat(d, lname(L, "ffn_down.weight"), y.nff, E))) return rc;
         for (int t = 0; t < y.nff / 32; ++t) { push_rows(rows, g, (uint64_t)t * 32, 32); push_rows(rows, u, (uint64_t)t * 32, 32); }
-        if ((rc = upload_tiled(m, rows, E, &y.wgu, stage))) return rc;
+        if ((rc = upload_tiled(m, rows, E, &y.wgu, stage, true))) return rc;    // row-block tiles (lg_k_geglu_t)
         rows.clear();
         push_rows(rows, d, 0, E);
         if ((rc = upload_tiled(m, rows, y.nff, &y.wdown, stage))) return rc;
@@ -401,7 +425,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     const size_t R = (size_t)(max_rows > LG_WIDE_ROWS ? max_rows : LG_WIDE_ROWS);      // prefill runs blocks of LG_WIDE_ROWS rows
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
         dev_alloc(m, &m->dout, 4 * R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
-        dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4) ||
+        dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4 + (size_t)12 * E) ||
         dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
         dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
@@ -647,8 +671,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     }
 
     // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
-    auto rows = [&](const float *w_pre, float *h_out) {
+    auto rows = [&](const float *w_pre, float *h_out, bool units = false) {
         RowArgs s{};
+        s.q_units = units && M <= LG_HIP_MAX_ROWS;
         s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq;
         if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
@@ -698,12 +723,12 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
         }
         {   // feed-forward: gate/up + GeGLU, then down
-            rows(y.ffn_norm, nullptr);
+            rows(y.ffn_norm, nullptr, true);                     // consumed by lg_k_geglu_t: unit order
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
             else
-                LAUNCH(KC_GATEUP, (lg_k_mm_geglu<M, 4>), dim3(y.nff / 32), dim3(256), lds_mm(M, E), a);
+                LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, a);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
             launch_mm<M, false>(lx, KC_DOWN, d);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;

@@ -37,6 +37,7 @@ struct RowArgs {
     const uint8_t *emb;      // tiled token_embd: rows are token lookups scaled by emb_scale
     const int32_t *toks;     // token schedule base ([n_steps][M])
     int8_t        *q;        // q8 activation buffer: [M][E] values, then [M][E/32] {scale, sum}
+    int            q_units;  // 1: write q in the block-major unit order of lg_k_geglu_t instead (M <= 8 only)
     int            emb_nit, emb_seg;
     float          emb_scale;
     int            E;
@@ -163,6 +164,12 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
         const int quad = t + 256 * v;                        // 4 values = a quarter of a 16-byte unit
+        if (M <= LG_HIP_MAX_ROWS_DEV && s.q_units) {          // units of 32 dwords per (block, 3 rows): see lg_k_geglu_t
+            uint32_t *unit = (uint32_t *)s.q + ((size_t)(quad >> 3) * ((M + 2) / 3) + j / 3) * 32;
+            unit[(j % 3) * 8 + (quad & 7)] = packed;
+            if ((t & 7) == 0) *(float2 *)(unit + 24 + 2 * (j % 3)) = make_float2(d, __int_as_float(sum));
+            continue;
+        }
         *(uint32_t *)(s.q + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
         if ((t & 7) == 0) dsb[lg_q8_ds_idx<M>(E, j, quad >> 3)] = make_float2(d, __int_as_float(sum));
     }
@@ -352,56 +359,103 @@ __global__ __launch_bounds__(LG_WG, 2) void lg_k_mm(MmArgs a) {
     }
 }
 
-// Gate/up matmul with the GeGLU and the q8 quantization of its result as epilogue.  The tiled
-// matrix interleaves 32 gate rows with the 32 up rows of the same indices, so a workgroup of 4
-// wavefronts owns one 32-wide quantization group: wavefront w computes gate and up rows 8w..8w+7
-// of it, sharing each activation load between the two.
+// Gate/up matmul with the GeGLU and the q8 quantization of its result as epilogue.
 struct GegluArgs {
-    const uint8_t *w;        // tiled [2*n_ff][k], virtual row order: 32 gate, 32 up, 32 gate, ...
+    const uint8_t *w;        // row-block tiles of [2*n_ff][k], virtual row order: 32 gate, 32 up, 32 gate, ...
     int            k, n_ff;
-    const int8_t  *q_in;
+    const int8_t  *q_in;     // verify blocks: unit order (below); wide blocks: lg_q8_off
     int8_t        *gq;       // q8 activation buffer of the result, width n_ff
 };
-// WV = 4: wavefront w computes gate AND up rows 8w..8w+7 (shared activation loads);
-// WV = 8: wavefronts 0-3 compute the gate rows, 4-7 the up rows (twice the wavefronts per CU to
-// hide latency, at the price of reading the activations twice from LDS).
-template <int M, int WV>
-__global__ __launch_bounds__(64 * WV, 2) void lg_k_mm_geglu(GegluArgs a) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    int8_t *lq = (int8_t *)smem;
-    float2 *lds = (float2 *)(smem + (size_t)M * a.k);
-    __shared__ float gbuf[2][LG_HIP_MAX_ROWS_DEV][32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
-    const int t = blockIdx.x;                               // 32-wide slice of n_ff
-    const size_t gstride = (size_t)nit * LG_TILE;
-    const int c = lane & 7, r = lane >> 3;
-    if (WV == 4) {
-        const uint8_t *wg[2] = { a.w + ((size_t)t * 8 + wave) * gstride, a.w + ((size_t)t * 8 + 4 + wave) * gstride };
-        const int row[2] = { 0, 0 };
-        WChunk<2> first;
-        lg_mm_fetch<2>(first, wg, 0, nit, lane);
-        lg_load_q8<M>(a.q_in, a.k, lq);
-        __syncthreads();
-        float acc[2][M];
-        lg_mm_groups<M, 8, 2, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
-        if (c < M) gbuf[0][c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * lg_pick<M>(acc[1], c);
-    } else {
-        const uint8_t *wg[1] = { a.w + ((size_t)t * 8 + wave) * gstride };      // groups 0-3 gate, 4-7 up
-        const int row[1] = { 0 };
-        WChunk<1> first;
-        lg_mm_fetch<1>(first, wg, 0, nit, lane);
-        lg_load_q8<M>(a.q_in, a.k, lq);
-        __syncthreads();
-        float acc[1][M];
-        lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
-        if (c < M) gbuf[wave >> 2][c][(wave & 3) * 8 + r] = lg_pick<M>(acc[0], c);
+// Gate/up + GeGLU for verify blocks (M <= 8): a wavefront is 64 weight rows x one of
+// the 8 K segments, so every lane of it multiplies its own weight block with the SAME activation
+// block.  The activations then travel through the scalar cache into SGPRs (loads from the constant
+// address space with a wavefront-uniform address) and feed v_dot4 as scalar operands: no LDS fill,
+// no barrier before the first dot, no per-lane activation traffic.  Weights: tile (row block of 64 =
+// the 32 gate rows and 32 up rows of 32 FFN columns, block kb) = lane r's 16 nibble bytes at r*16 and
+// scale at 1024 + r*2, tiles ordered [row block][kb] ("row-block tiles", lg_hip_repack_q4_0_rowblocks).
+// Activations: per block kb and group of 3 rows one unit of 32 dwords: 3 x 8 dwords of int8, then
+// 3 x {scale, sum}, 2 unused; a unit is requested while the previous one is consumed.
+typedef const __attribute__((address_space(4))) int *lg_cint;
+template <int M>
+__global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
+    __shared__ float red[8][M][64];
+    constexpr int NU = (M + 2) / 3, CH = 5;
+    const int lane = threadIdx.x & 63;
+    const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));      // K segment of this wavefront
+    const int t = blockIdx.x, nb = a.k >> 5, nit = nb >> 3, nunits = nit * NU;
+    const uint8_t *wt = a.w + ((size_t)t * nb + (size_t)s * nit) * LG_TILE;
+    lg_cint au = (lg_cint)(uintptr_t)a.q_in + (size_t)s * nunits * 32;
+    float p[M];
+    #pragma unroll
+    for (int j = 0; j < M; ++j) p[j] = 0.0f;
+    uint4 wq[CH], nwq[CH]; uint32_t wd[CH], nwd[CH];
+    auto fetch = [&](int it0) {
+        #pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;
+            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
+            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+        }
+    };
+    fetch(0);
+    int cur[32], nxt[32];
+    #pragma unroll
+    for (int i = 0; i < 32; ++i) cur[i] = au[i];
+    for (int it0 = 0; it0 < nit; it0 += CH) {
+        #pragma unroll
+        for (int u = 0; u < CH; ++u) { wq[u] = nwq[u]; wd[u] = nwd[u]; }
+        if (it0 + CH < nit) fetch(it0 + CH);
+        #pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if (it0 + c >= nit) break;
+            const uint4 q = wq[c];
+            const int lo0 = q.x & 0x0F0F0F0F, lo1 = q.y & 0x0F0F0F0F, lo2 = q.z & 0x0F0F0F0F, lo3 = q.w & 0x0F0F0F0F;
+            const int hi0 = (q.x >> 4) & 0x0F0F0F0F, hi1 = (q.y >> 4) & 0x0F0F0F0F, hi2 = (q.z >> 4) & 0x0F0F0F0F, hi3 = (q.w >> 4) & 0x0F0F0F0F;
+            const float dw = lg_h2f((uint16_t)wd[c]);
+            #pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                const int tu = (it0 + c) * NU + u, tn = tu + 1 < nunits ? tu + 1 : tu;
+                // the unit in `cur` must have arrived before the next one is requested: scalar loads
+                // return out of order, so the only wait there is waits for everything in flight
+                asm volatile("" :: "s"(cur[0]), "s"(cur[8]), "s"(cur[16]), "s"(cur[24]), "s"(cur[31]));
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for (int i = 0; i < 32; ++i) nxt[i] = au[(size_t)tn * 32 + i];
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for (int r = 0; r < 3; ++r) {
+                    const int j = u * 3 + r;
+                    if (j < M) {
+                        int dot = 0;
+                        dot = __builtin_amdgcn_sdot4(lo0, cur[r * 8 + 0], dot, false);
+                        dot = __builtin_amdgcn_sdot4(lo1, cur[r * 8 + 1], dot, false);
+                        dot = __builtin_amdgcn_sdot4(lo2, cur[r * 8 + 2], dot, false);
+                        dot = __builtin_amdgcn_sdot4(lo3, cur[r * 8 + 3], dot, false);
+                        dot = __builtin_amdgcn_sdot4(hi0, cur[r * 8 + 4], dot, false);
+                        dot = __builtin_amdgcn_sdot4(hi1, cur[r * 8 + 5], dot, false);
+                        dot = __builtin_amdgcn_sdot4(hi2, cur[r * 8 + 6], dot, false);
+                        dot = __builtin_amdgcn_sdot4(hi3, cur[r * 8 + 7], dot, false);
+                        p[j] = lg_fmaf(__int_as_float(cur[24 + 2 * r]) * dw, (float)(dot - 8 * cur[25 + 2 * r]), p[j]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                #pragma unroll
+                for (int i = 0; i < 32; ++i) cur[i] = nxt[i];
+            }
+        }
     }
+    #pragma unroll
+    for (int j = 0; j < M; ++j) red[s][j][lane] = p[j];
     __syncthreads();
-    for (int j = threadIdx.x >> 5; j < M; j += 2 * WV) {         // half-wavefront per row, one value per lane
+    for (int j = threadIdx.x >> 5; j < M; j += 16) {         // half-wavefront per row, one FFN column per lane
         const int i = threadIdx.x & 31;
-        const float g = WV == 4 ? gbuf[0][j][i] : lg_gelu(gbuf[0][j][i]) * gbuf[1][j][i];
+        float g[8], u[8];
+        #pragma unroll
+        for (int c = 0; c < 8; ++c) { g[c] = red[c][j][i]; u[c] = red[c][j][32 + i]; }
+        const float gate = ((g[0] + g[1]) + (g[2] + g[3])) + ((g[4] + g[5]) + (g[6] + g[7]));
+        const float up = ((u[0] + u[1]) + (u[2] + u[3])) + ((u[4] + u[5]) + (u[6] + u[7]));
         float d; int sum;
-        const int q = lg_quant1_32lanes(g, &d, &sum);
+        const int q = lg_quant1_32lanes(lg_gelu(gate) * up, &d, &sum);
         const ActLayout lay = lg_act_layout(a.n_ff);          // order the ffn_down matmul reads
         a.gq[(size_t)j * a.n_ff + lg_act_unit(lay, t * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
         if (i == 0) lg_q8_ds<M>(a.gq, a.n_ff)[(size_t)j * (a.n_ff >> 5) + lg_act_block(lay, t)] = make_float2(d, __int_as_float(sum));

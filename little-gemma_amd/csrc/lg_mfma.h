@@ -50,7 +50,9 @@ static_assert(8 * 16 * 64 * 4 <= MfmaGeo::lds_bytes, "the final exchange must fi
 // `smem` needs MfmaGeo::lds_bytes and is free again on return.
 __device__ __forceinline__ int lg_wide_col(int wave, int h) { return 8 * (wave >> 1) + 4 * h + 2 * (wave & 1); }
 
-template <int R, int S, bool DUMP>
+// RB: the weights are in row-block tiles (lg_k_geglu_t: tile (64-row block, kb), lane = row) instead of
+// the segment tiles of lg_device.h; S must then be 8.
+template <int R, int S, bool DUMP, bool RB = false>
 __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, int part, const int8_t *q_in, int tile, int rows,
                                               unsigned char *smem, float (&res)[2], int32_t *dots, int m_total) {
     using G = MfmaGeo;
@@ -67,9 +69,15 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
     // wavefronts 0..3 fetch the step's 256 (row, segment) slots: slot -> tile, lane inside the tile, row of the block
     const int slot = (wave & 3) * 64 + lane;
     int st_tile, st_lane, st_m, st_c;
-    if (S == 8) { st_tile = slot >> 6; st_lane = slot & 63; st_m = st_tile * 8 + (st_lane >> 3); st_c = st_lane & 7; }
-    else        { st_tile = slot >> 4; st_c = slot & 7; const int r = (slot >> 3) & 1; st_lane = r * 32 + 8 * part + st_c; st_m = st_tile * 2 + r; }
-    const uint8_t *tbase = w + (size_t)(rb * TPB + st_tile) * nit * LG_TILE;
+    const uint8_t *tbase;
+    if (RB) {       // slot = (segment, row): the 32 rows of block rb are lanes 32*(rb&1) .. +31 of tile (rb/2, segment*nit + it)
+        st_c = slot >> 5; st_m = slot & 31; st_lane = 32 * (rb & 1) + st_m; st_tile = 0;
+        tbase = w + ((size_t)(rb >> 1) * nb + (size_t)st_c * nit) * LG_TILE;
+    } else {
+        if (S == 8) { st_tile = slot >> 6; st_lane = slot & 63; st_m = st_tile * 8 + (st_lane >> 3); st_c = st_lane & 7; }
+        else        { st_tile = slot >> 4; st_c = slot & 7; const int r = (slot >> 3) & 1; st_lane = r * 32 + 8 * part + st_c; st_m = st_tile * 2 + r; }
+        tbase = w + (size_t)(rb * TPB + st_tile) * nit * LG_TILE;
+    }
     // A chunk of U steps is requested while the previous one is consumed (enough bytes in flight to
     // cover the memory latency), parked in LDS in one go, and followed by a single barrier.
     uint4 tq[G::U]; uint32_t ts[G::U];
@@ -183,15 +191,15 @@ __device__ __forceinline__ void lg_wide_quant32(float *vbuf, int8_t *q, int kq, 
     if (qd == 0) lg_q8_ds<R>(q, kq)[lg_q8_ds_idx<R>(kq, an, block)] = make_float2(d, __int_as_float(sum));
 }
 
-// Gate/up with the GeGLU and the q8 of its result (see lg_k_mm_geglu): the tiled matrix holds, per
-// 32 FFN columns, a block of 32 gate rows followed by the block of the 32 up rows.  grid = (n_ff/32, row tiles).
+// Gate/up with the GeGLU and the q8 of its result (see lg_k_geglu_t): row-block tiles, per 32 FFN
+// columns a block of 32 gate rows followed by the block of the 32 up rows.  grid = (n_ff/32, row tiles).
 template <int R>
 __global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_geglu_wide(GegluArgs a, int rows) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float vbuf[32 * 33];
     float g[2], u[2];
-    lg_mfma_block<R, 8, false>(a.w, a.k, 2 * blockIdx.x, 0, a.q_in, blockIdx.y, rows, smem, g, nullptr, 0);
-    lg_mfma_block<R, 8, false>(a.w, a.k, 2 * blockIdx.x + 1, 0, a.q_in, blockIdx.y, rows, smem, u, nullptr, 0);
+    lg_mfma_block<R, 8, false, true>(a.w, a.k, 2 * blockIdx.x, 0, a.q_in, blockIdx.y, rows, smem, g, nullptr, 0);
+    lg_mfma_block<R, 8, false, true>(a.w, a.k, 2 * blockIdx.x + 1, 0, a.q_in, blockIdx.y, rows, smem, u, nullptr, 0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, col = lg_wide_col(wave, lane >> 5);
     #pragma unroll
     for (int j = 0; j < 2; ++j) vbuf[n * 33 + col + j] = lg_gelu(g[j]) * u[j];
