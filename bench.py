@@ -28,8 +28,8 @@ lg = importlib.import_module("little-gemma_amd")
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel (gate/up + GeGLU at the E4B shape), from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised under profiles/ (scaled by the copy-kernel calibration given there):
-# reads 29.41 MB for M = 5 (29.26 MB for M = 1), writes 0.15 MB.  Other shapes have no counter run.
-MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.41e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.26e6 + 0.03e6}
+# reads 29.55 MB for M = 5 (29.36 MB for M = 1), writes 0.15 MB (0.03 MB).  Other shapes have no counter run.
+MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.55e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.36e6 + 0.03e6}
 CTX = 2048
 WORKLOADS = {
     "e4b": ("E4B-shape q4_0 verify step (42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144, "
@@ -238,7 +238,7 @@ def main():
         dt = time.time() - t0
         macs = sum(c["bytes"] for c in prof if c["name"] != "lm_head" and c["name"] != "attn_tiles") / (18.0 / 32.0)   # weights touched per position
         line["prefill"] = {"positions": int(a.prefill), "ms": 1e3 * dt, "tok_per_s": a.prefill / dt,
-                           "kernel": "v_mfma_i32_32x32x32_i8, 32-row blocks", "int8_TOPs": 2.0 * macs * a.prefill / dt / 1e12,
+                           "kernel": "v_mfma_i32_32x32x32_i8, 128-row blocks", "int8_TOPs": 2.0 * macs * a.prefill / dt / 1e12,
                            "mfma_peak_TOPs": 5000.0, "mfma_utilisation": 2.0 * macs * a.prefill / dt / 5.0e15}
     gpu.close()
     if a.cpu_seconds > 0:
