@@ -689,6 +689,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         rows(nullptr, nullptr);
         MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, nullptr };
         launch_mm<M, false>(lx, KC_PMP, a);
+        IplArgs i{ m->pmp_raw, m->ple, nl, M, m->proj_norm, m->pte, m->sched,
+                   1.0f / sqrtf((float)E), sqrtf((float)m->ple), 1.0f / sqrtf(2.0f), m->eps };
+        LAUNCH(KC_PMP, lg_k_ipl, dim3(nl, M), dim3(64), 0, i, m->ctl);
     }
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
@@ -735,17 +738,17 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_parts = (M > LG_HIP_MAX_ROWS && lg_segments(y.nff) == 32) ? 4 : 1;
         }
         if (m->ple) {   // per-layer embedding block
-            rows(nullptr, nullptr);
-            PleGateArgs a{};
-            a.w = y.winp; a.k = E; a.ple = m->ple; a.q_in = m->hq;
-            a.pmp_raw = m->pmp_raw; a.layer = L; a.n_layer = nl;
-            a.proj_norm = m->proj_norm; a.pte = m->pte; a.toks = m->sched;
-            a.pscale = 1.0f / sqrtf((float)E); a.tscale = sqrtf((float)m->ple); a.rsqrt2 = 1.0f / sqrtf(2.0f); a.eps = m->eps;
-            a.pq = m->pq;
-            if constexpr (M > LG_HIP_MAX_ROWS)
-                LAUNCH(KC_PLEGATE, (lg_k_mm_plegate_wide<M>), dim3(m->ple / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, m->ctl, M);
-            else
-                LAUNCH(KC_PLEGATE, (lg_k_mm_plegate<M>), dim3(m->ple / 32), dim3(LG_WG), lds_mm(M, E), a, m->ctl);
+            PleGateArgs a{ y.winp, E, m->ple, m->hq, m->pmp_raw, L, nl, m->pq };
+            if constexpr (M > LG_HIP_MAX_ROWS) {
+                rows(nullptr, nullptr);
+                LAUNCH(KC_PLEGATE, (lg_k_mm_plegate_wide<M>), dim3(m->ple / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+            } else {
+                // the residual update after ffn_down and its q8 happen inside the gate kernel (no rows kernel here)
+                RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps };
+                LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32), dim3(LG_RPG_WG), lds_mm(M, E), r);
+                cur ^= 1;
+                pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+            }
             MmArgs p{ y.wproj, m->ple, E, m->dout, m->pq, nullptr };
             launch_mm<M, false>(lx, KC_PLEPROJ, p);
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;

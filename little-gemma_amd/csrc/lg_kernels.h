@@ -398,6 +398,12 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
         }
     };
     fetch(0);
+    // The units were written by the previous kernel on other XCDs, so the first read of each 128-byte
+    // unit from this XCD misses its L2; walked one unit ahead, those misses would queue up behind each
+    // other.  One vector load per unit, issued now, brings the segment's lines in side by side.
+    int touch = 0;
+    for (int i = lane; i < nunits; i += 64)
+        touch |= *(const volatile int *)((const int *)a.q_in + ((size_t)s * nunits + i) * 32);
     int cur[32], nxt[32];
     #pragma unroll
     for (int i = 0; i < 32; ++i) cur[i] = au[i];
@@ -444,6 +450,7 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
             }
         }
     }
+    asm volatile("" :: "v"(touch));
     #pragma unroll
     for (int j = 0; j < M; ++j) red[s][j][lane] = p[j];
     __syncthreads();
@@ -462,63 +469,136 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
     }
 }
 
-// PLE gate: inp_gate matmul on the q8 of the updated residual, then gelu(.) * ipl and q8.
-// ipl for this layer is finished here from the raw per_layer_model_proj output and the token's
-// per-layer embedding row (the reference builds it once per step in build_per_layer_n,
-// src/cuda/model-cuda.cuh:1121-1147): ipl = (rmsnorm(proj/sqrt(E)) * w + tok*sqrt(ple)) / sqrt(2).
-struct PleGateArgs {
-    const uint8_t *w;        // tiled inp_gate [ple][E]
-    int            k, ple;
-    const int8_t  *q_in;
-    const float   *pmp_raw;  // [M][n_layer*ple] raw projection
-    int            layer, n_layer;
+// Per-layer inputs of a block, finished once per step from the raw per_layer_model_proj output and the
+// tokens' per-layer embedding rows (the reference builds them once per step in build_per_layer_n,
+// src/cuda/model-cuda.cuh:1121-1147): ipl = (rmsnorm(proj/sqrt(E)) * w + tok*sqrt(ple)) / sqrt(2),
+// in place over the raw projection.  One wavefront per (layer, row); ple <= 256.
+struct IplArgs {
+    float         *pmp;      // [rows][n_layer*ple]: raw projection in, ipl out
+    int            ple, n_layer, rows_per_step;
     const float   *proj_norm;     // [ple]
     const uint8_t *pte;      // per_layer_token_embd, plain q4_0 rows of n_layer*ple
     const int32_t *toks;
     float          pscale, tscale, rsqrt2, eps;
+};
+__global__ __launch_bounds__(64) void lg_k_ipl(IplArgs a, const StepCtl *ctl) {
+    const int lane = threadIdx.x, L = blockIdx.x, j = blockIdx.y, ple = a.ple, e0 = 4 * lane;
+    float *pr = a.pmp + (size_t)j * a.n_layer * ple + (size_t)L * ple;
+    const bool on = e0 < ple;
+    const float4 p4 = on ? *(const float4 *)(pr + e0) : make_float4(0, 0, 0, 0);
+    const float4 wn = on ? *(const float4 *)(a.proj_norm + e0) : make_float4(0, 0, 0, 0);
+    const int tok = a.toks[ctl->step * a.rows_per_step + j];
+    const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
+    float tk[4];
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) tk[i] = on ? lg_q4_0_elem(trow, L * ple + e0 + i) * a.tscale : 0.0f;
+    const float4 p = make_float4(p4.x * a.pscale, p4.y * a.pscale, p4.z * a.pscale, p4.w * a.pscale);
+    const float ss = lg_wave_sum64(lg_sumsq4(p, 0.0f));                 // one quad per lane
+    const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
+    if (on) *(float4 *)(pr + e0) = make_float4((p.x * sc * wn.x + tk[0]) * a.rsqrt2, (p.y * sc * wn.y + tk[1]) * a.rsqrt2,
+                                               (p.z * sc * wn.z + tk[2]) * a.rsqrt2, (p.w * sc * wn.w + tk[3]) * a.rsqrt2);
+}
+
+// PLE gate: inp_gate matmul on the q8 of the updated residual, then gelu(.) * ipl and q8.
+struct PleGateArgs {
+    const uint8_t *w;        // tiled inp_gate [ple][E]
+    int            k, ple;
+    const int8_t  *q_in;
+    const float   *ipl;      // [M][n_layer*ple] per-layer inputs (lg_k_ipl)
+    int            layer, n_layer;
     int8_t        *pq;       // q8 activation buffer of the result, width ple
 };
+// Verify blocks (wide blocks: lg_k_mm_plegate_wide): the row work that precedes the matmul is folded in,
+// i.e. the residual update x += rmsnorm(dout) * w_post and the q8 of the new x (what lg_k_rows does
+// between two other matmuls).  Each of the ple/32 workgroups repeats the update of all M rows: the matmul needs every row
+// whole, and a kernel boundary costs more than the repeated work.  1024 threads: four groups of 256, a
+// group takes rows g, g+4 with the lane assignment and summation order of lg_k_rows; the quantized rows
+// go straight to LDS, workgroup 0 also writes the new residual; wavefronts 0..3 then run the matmul.
+struct RowsPleGateArgs {
+    PleGateArgs    g;
+    const float   *x, *dout, *w_post;   // [M][E] residual, [M][E] ffn_down output, [E]
+    float         *x_out;               // [M][E]
+    float          eps;
+};
+#define LG_RPG_WG 1024
 template <int M>
-__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_plegate(PleGateArgs a, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_RPG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
-    float2 *lds = (float2 *)(smem + (size_t)M * a.k);
+    float2 *lds = (float2 *)(smem + (size_t)M * a.g.k);
     __shared__ float gbuf[LG_HIP_MAX_ROWS_DEV][32];
-    __shared__ float ipl[LG_HIP_MAX_ROWS_DEV][32];           // this workgroup's 32 elements of ipl, per row
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nit = a.k >> 8;
-    const int ple = a.ple;
-    const uint8_t *wg[1] = { a.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
+    __shared__ float ipl[LG_HIP_MAX_ROWS_DEV][32];
+    __shared__ float red[LG_HIP_MAX_ROWS_DEV][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
+    const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + (wave & 3)) * nit * LG_TILE };
     const int row[1] = { 0 };
     WChunk<1> first;
-    lg_mm_fetch<1>(first, wg, 0, nit, lane);
-    // ipl slice: all loads of a row issued together (projection slice, token row bytes, norm weight)
-    for (int j = wave; j < M; j += LG_WG / 64) {
-        const float *pr = a.pmp_raw + (size_t)j * a.n_layer * ple + (size_t)a.layer * ple;
-        const int tok = a.toks[ctl->step * M + j];
-        const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
-        const int e = blockIdx.x * 32 + (lane & 31);
-        const float4 p4 = 4 * lane < ple ? *(const float4 *)(pr + 4 * lane) : make_float4(0, 0, 0, 0);
-        const float pe = pr[e], wn = a.proj_norm[e];
-        const float tk = lg_q4_0_elem(trow, a.layer * ple + e) * a.tscale;
-        const float4 p = make_float4(p4.x * a.pscale, p4.y * a.pscale, p4.z * a.pscale, p4.w * a.pscale);
-        const float ss = lg_wave_sum64(lg_sumsq4(p, 0.0f));                 // ple <= 256: one quad per lane
-        const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
-        if (lane < 32) ipl[j][lane] = (pe * a.pscale * sc * wn + tk) * a.rsqrt2;
+    if (wave < 4) lg_mm_fetch<1>(first, wg, 0, nit, lane);
+    for (int j = wave; j < M; j += LG_RPG_WG / 64)
+        if (lane < 32) ipl[j][lane] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + lane];
+    {
+        constexpr int RJ = (M + 3) / 4;                       // rows per group
+        const int t = threadIdx.x & 255, grp = threadIdx.x >> 8, gw = wave & 3, nq = E >> 2;
+        float4 xv[RJ][LG_ROWV], dv[RJ][LG_ROWV], wp[LG_ROWV];
+        const float4 *wr = (const float4 *)a.w_post;
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) wp[v] = wr[t + 256 * v];
+        #pragma unroll
+        for (int r = 0; r < RJ; ++r) {
+            const int j = grp + 4 * r;
+            if (j >= M) break;                                // uniform per wavefront
+            const float4 *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[r][v] = xr[t + 256 * v]; dv[r][v] = dr[t + 256 * v]; }
+        }
+        #pragma unroll
+        for (int r = 0; r < RJ; ++r) {
+            const int j = grp + 4 * r;
+            if (j >= M) break;
+            float ss = 0.0f;
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[r][v], ss);
+            ss = lg_wave_sum64(ss);
+            if (lane == 0) red[j][gw] = ss;
+        }
+        __syncthreads();
+        #pragma unroll
+        for (int r = 0; r < RJ; ++r) {
+            const int j = grp + 4 * r;
+            if (j >= M) break;
+            const float ss = (red[j][0] + red[j][1]) + (red[j][2] + red[j][3]);
+            const float sc = 1.0f / sqrtf(ss / (float)E + a.eps);
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) {
+                if (t + 256 * v >= nq) break;                 // nq is a multiple of 64: whole wavefronts
+                const float4 w = wp[v], d = dv[r][v];
+                float4 x = xv[r][v];
+                x.x = x.x + d.x * sc * w.x;  x.y = x.y + d.y * sc * w.y;
+                x.z = x.z + d.z * sc * w.z;  x.w = x.w + d.w * sc * w.w;
+                if (blockIdx.x == 0) ((float4 *)(a.x_out + (size_t)j * E))[t + 256 * v] = x;
+                float dq; int sum;
+                const uint32_t packed = lg_quant4_8lanes(x, &dq, &sum);
+                const int quad = t + 256 * v;
+                *(uint32_t *)(lq + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
+                if ((t & 7) == 0) lds[lg_q8_ds_idx<M>(E, j, quad >> 3)] = make_float2(dq, __int_as_float(sum));
+            }
+        }
     }
-    lg_load_q8<M>(a.q_in, a.k, lq);
     __syncthreads();
-    float acc[1][M];
-    lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, a.k, acc, lane, nullptr, 0, row);
-    const int c = lane & 7, r = lane >> 3;
-    if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * ipl[c][wave * 8 + r];
+    if (wave < 4) {
+        float acc[1][M];
+        lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
+        const int c = lane & 7, r = lane >> 3;
+        if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * ipl[c][wave * 8 + r];
+    }
     __syncthreads();
-    for (int j = threadIdx.x >> 5; j < M; j += LG_WG / 32) {
+    for (int j = threadIdx.x >> 5; j < M; j += LG_RPG_WG / 32) {
         const int i = threadIdx.x & 31;
         float d; int sum;
         const int q = lg_quant1_32lanes(gbuf[j][i], &d, &sum);
         const ActLayout lay = lg_act_layout(ple);
-        a.pq[(size_t)j * ple + lg_act_unit(lay, blockIdx.x * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
-        if (i == 0) lg_q8_ds<M>(a.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, blockIdx.x)] = make_float2(d, __int_as_float(sum));
+        a.g.pq[(size_t)j * ple + lg_act_unit(lay, blockIdx.x * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
+        if (i == 0) lg_q8_ds<M>(a.g.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, blockIdx.x)] = make_float2(d, __int_as_float(sum));
     }
 }
 

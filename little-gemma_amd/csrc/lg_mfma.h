@@ -210,27 +210,17 @@ __global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_geglu_wide(GegluArgs a, in
 // PLE gate for wide blocks (see lg_k_mm_plegate): gelu(inp_gate . x) * ipl[layer], q8 of the result.
 // grid = (ple/32, row tiles).
 template <int R>
-__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_plegate_wide(PleGateArgs a, const StepCtl *ctl, int rows) {
+__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_plegate_wide(PleGateArgs a, int rows) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float vbuf[32 * 33];
     __shared__ float ipl[32][32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, ple = a.ple;
     #pragma unroll
-    for (int jj = 0; jj < LG_WIDE / (LG_WIDE_WG / 64); ++jj) {     // fixed trip count: the loads of all rows go out together
+    for (int jj = 0; jj < LG_WIDE / (LG_WIDE_WG / 64); ++jj) {
         const int j = wave + jj * (LG_WIDE_WG / 64);
         int an = blockIdx.y * LG_WIDE + j;
         if (an >= rows) an = rows - 1;
-        const float *pr = a.pmp_raw + (size_t)an * a.n_layer * ple + (size_t)a.layer * ple;
-        const int tok = a.toks[ctl->step * R + an];
-        const uint8_t *trow = a.pte + (size_t)tok * ((size_t)a.n_layer * ple / 32 * 18);
-        const int e = blockIdx.x * 32 + (lane & 31);
-        const float4 p4 = 4 * lane < ple ? *(const float4 *)(pr + 4 * lane) : make_float4(0, 0, 0, 0);
-        const float pe = pr[e], wn = a.proj_norm[e];
-        const float tk = lg_q4_0_elem(trow, a.layer * ple + e) * a.tscale;
-        const float4 p = make_float4(p4.x * a.pscale, p4.y * a.pscale, p4.z * a.pscale, p4.w * a.pscale);
-        const float ss = lg_wave_sum64(lg_sumsq4(p, 0.0f));
-        const float sc = 1.0f / sqrtf(ss / (float)ple + a.eps);
-        if (lane < 32) ipl[j][lane] = (pe * a.pscale * sc * wn + tk) * a.rsqrt2;
+        if (lane < 32) ipl[j][lane] = a.ipl[(size_t)an * a.n_layer * ple + (size_t)a.layer * ple + blockIdx.x * 32 + lane];
     }
     float r[2];
     lg_mfma_block<R, 8, false>(a.w, a.k, blockIdx.x, 0, a.q_in, blockIdx.y, rows, smem, r, nullptr, 0);
