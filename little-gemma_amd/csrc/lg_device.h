@@ -183,7 +183,7 @@ __device__ __forceinline__ float lg_q4_0_elem(const uint8_t *row, int e) {
 // Inner product of one weight tile lane (16 nibble bytes = one q4_0 block) with the 32 int8 of
 // an activation block: sum(c*q) - 8*sum(q) == sum((c-8)*q), exact in int32.
 __device__ __forceinline__ int lg_block_dot(uint4 wq, int4 a0, int4 a1, int act_sum) {
-    int dot = 0;
+    int dot = -8 * act_sum;                                   // starts the accumulator: one multiply instead of a move and a subtract
     dot = __builtin_amdgcn_sdot4((int)(wq.x & 0x0F0F0F0Fu), a0.x, dot, false);
     dot = __builtin_amdgcn_sdot4((int)(wq.y & 0x0F0F0F0Fu), a0.y, dot, false);
     dot = __builtin_amdgcn_sdot4((int)(wq.z & 0x0F0F0F0Fu), a0.z, dot, false);
@@ -192,5 +192,5 @@ __device__ __forceinline__ int lg_block_dot(uint4 wq, int4 a0, int4 a1, int act_
     dot = __builtin_amdgcn_sdot4((int)((wq.y >> 4) & 0x0F0F0F0Fu), a1.y, dot, false);
     dot = __builtin_amdgcn_sdot4((int)((wq.z >> 4) & 0x0F0F0F0Fu), a1.z, dot, false);
     dot = __builtin_amdgcn_sdot4((int)((wq.w >> 4) & 0x0F0F0F0Fu), a1.w, dot, false);
-    return dot - 8 * act_sum;
+    return dot;
 }

@@ -671,9 +671,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     }
 
     // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
-    auto rows = [&](const float *w_pre, float *h_out, bool units = false) {
+    auto rows = [&](const float *w_pre, float *h_out, int units = 0) {
         RowArgs s{};
-        s.q_units = units && M <= LG_HIP_MAX_ROWS;
+        s.q_units = M <= LG_HIP_MAX_ROWS ? units : 0;
         s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq;
         if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
@@ -726,10 +726,15 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
         }
         {   // feed-forward: gate/up + GeGLU, then down
-            rows(y.ffn_norm, nullptr, true);                     // consumed by lg_k_geglu_t: unit order
+            // verify blocks: 1..3 rows through v_dot4 with scalar operands, 4..8 rows through the matrix cores
+            // (its float work per tile does not grow with the row count); each has its own activation order
+            constexpr bool mfma = M >= 4 && M <= LG_HIP_MAX_ROWS;
+            rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+            else if constexpr (mfma)
+                LAUNCH(KC_GATEUP, (lg_k_geglu_m<M>), dim3(y.nff / 32), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, a);
             else
                 LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, a);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };

@@ -37,7 +37,7 @@ struct RowArgs {
     const uint8_t *emb;      // tiled token_embd: rows are token lookups scaled by emb_scale
     const int32_t *toks;     // token schedule base ([n_steps][M])
     int8_t        *q;        // q8 activation buffer: [M][E] values, then [M][E/32] {scale, sum}
-    int            q_units;  // 1: write q in the block-major unit order of lg_k_geglu_t instead (M <= 8 only)
+    int            q_units;  // write q in a block-major order instead (M <= 8 only): 1 = units of lg_k_geglu_t, 2 = blocks of lg_k_geglu_m
     int            emb_nit, emb_seg;
     float          emb_scale;
     int            E;
@@ -77,6 +77,7 @@ __device__ __forceinline__ size_t lg_q8_ds_idx(int k, int j, int b) {
     if (M <= LG_HIP_MAX_ROWS_DEV) return (size_t)j * (k >> 5) + u;
     return (size_t)(j >> 5) * 32 * (k >> 5) + (size_t)u * 32 + (j & 31);
 }
+#define LG_MU_DWORDS 80                     // dwords per block of the lg_k_geglu_m activation order
 #define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
@@ -164,10 +165,17 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
         const int quad = t + 256 * v;                        // 4 values = a quarter of a 16-byte unit
-        if (M <= LG_HIP_MAX_ROWS_DEV && s.q_units) {          // units of 32 dwords per (block, 3 rows): see lg_k_geglu_t
+        if (M <= LG_HIP_MAX_ROWS_DEV && s.q_units == 1) {     // units of 32 dwords per (block, 3 rows): see lg_k_geglu_t
             uint32_t *unit = (uint32_t *)s.q + ((size_t)(quad >> 3) * ((M + 2) / 3) + j / 3) * 32;
             unit[(j % 3) * 8 + (quad & 7)] = packed;
             if ((t & 7) == 0) *(float2 *)(unit + 24 + 2 * (j % 3)) = make_float2(d, __int_as_float(sum));
+            continue;
+        }
+        if (M <= LG_HIP_MAX_ROWS_DEV && s.q_units == 2) {     // 80 dwords per block, 8 row slots: see lg_k_geglu_m
+            uint32_t *blk = (uint32_t *)s.q + (size_t)(quad >> 3) * LG_MU_DWORDS;
+            const int dw = quad & 7;
+            blk[j * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))] = packed;
+            if ((t & 7) == 0) *(int2 *)(blk + 64 + 2 * j) = make_int2(__float_as_int(d), -8 * sum);
             continue;
         }
         *(uint32_t *)(s.q + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_draft_input(DraftInArgs a, const S
 // Weights are fetched in chunks of LG_U tiles per group; the first chunk is requested before the
 // activations are staged (weights depend on nothing), each later chunk while the previous one is
 // being consumed.
-#define LG_U 5
+#define LG_U 2
 template <int G>
 struct WChunk { uint4 q[G][LG_U]; uint32_t s[G][LG_U]; };
 
@@ -379,7 +387,7 @@ typedef const __attribute__((address_space(4))) int *lg_cint;
 template <int M>
 __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
     __shared__ float red[8][M][64];
-    constexpr int NU = (M + 2) / 3, CH = 5;
+    constexpr int NU = (M + 2) / 3, CH = 2;
     const int lane = threadIdx.x & 63;
     const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));      // K segment of this wavefront
     const int t = blockIdx.x, nb = a.k >> 5, nit = nb >> 3, nunits = nit * NU;
@@ -432,7 +440,7 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
                 for (int r = 0; r < 3; ++r) {
                     const int j = u * 3 + r;
                     if (j < M) {
-                        int dot = 0;
+                        int dot = -8 * cur[25 + 2 * r];       // the -8*sum term of the block dot, formed on the scalar unit
                         dot = __builtin_amdgcn_sdot4(lo0, cur[r * 8 + 0], dot, false);
                         dot = __builtin_amdgcn_sdot4(lo1, cur[r * 8 + 1], dot, false);
                         dot = __builtin_amdgcn_sdot4(lo2, cur[r * 8 + 2], dot, false);
@@ -441,7 +449,7 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
                         dot = __builtin_amdgcn_sdot4(hi1, cur[r * 8 + 5], dot, false);
                         dot = __builtin_amdgcn_sdot4(hi2, cur[r * 8 + 6], dot, false);
                         dot = __builtin_amdgcn_sdot4(hi3, cur[r * 8 + 7], dot, false);
-                        p[j] = lg_fmaf(__int_as_float(cur[24 + 2 * r]) * dw, (float)(dot - 8 * cur[25 + 2 * r]), p[j]);
+                        p[j] = lg_fmaf(__int_as_float(cur[24 + 2 * r]) * dw, (float)dot, p[j]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -453,6 +461,100 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
     asm volatile("" :: "v"(touch));
     #pragma unroll
     for (int j = 0; j < M; ++j) red[s][j][lane] = p[j];
+    __syncthreads();
+    for (int j = threadIdx.x >> 5; j < M; j += 16) {         // half-wavefront per row, one FFN column per lane
+        const int i = threadIdx.x & 31;
+        float g[8], u[8];
+        #pragma unroll
+        for (int c = 0; c < 8; ++c) { g[c] = red[c][j][i]; u[c] = red[c][j][32 + i]; }
+        const float gate = ((g[0] + g[1]) + (g[2] + g[3])) + ((g[4] + g[5]) + (g[6] + g[7]));
+        const float up = ((u[0] + u[1]) + (u[2] + u[3])) + ((u[4] + u[5]) + (u[6] + u[7]));
+        float d; int sum;
+        const int q = lg_quant1_32lanes(lg_gelu(gate) * up, &d, &sum);
+        const ActLayout lay = lg_act_layout(a.n_ff);          // order the ffn_down matmul reads
+        a.gq[(size_t)j * a.n_ff + lg_act_unit(lay, t * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
+        if (i == 0) lg_q8_ds<M>(a.gq, a.n_ff)[(size_t)j * (a.n_ff >> 5) + lg_act_block(lay, t)] = make_float2(d, __int_as_float(sum));
+    }
+}
+
+// Gate/up + GeGLU for verify blocks of 4..8 rows on the matrix cores.  Same weight tiles and the same
+// wavefront = 64 weight rows x one K segment split as lg_k_geglu_t, but the 8 v_dot4 per (tile, row) become
+// two v_mfma_i32_32x32x32_i8 per tile whatever M is: A = the block's activations (row m = draft row, 8 row
+// slots, the other 24 rows of the operand are don't-cares whose results are never read), B = the tile's 32
+// gate rows, then its 32 up rows, as columns.  A lane's operand is the K half l/32 of column l%32, while a
+// tile keeps weight row l whole in lane l, so the two halves of the wavefront first trade 8 bytes each
+// (v_permlane32_swap): lane (n, h) then holds nibble bytes 8h..8h+7 of gate row n and of up row n, i.e.
+// K = 8h..8h+7 and 16+8h..16+8h+7.  The activation bytes are stored in that order (dwords 0 1 4 5 | 2 3 6 7
+// of a row's 32), 80 dwords per block: 8 row slots x 8 dwords, then 8 x {scale, -8*sum}.  Result register
+// i of lane (n, h) is draft row 4h+i of column n, so a lane applies 4 scale pairs per column, and the
+// per-block float work is 8 x (add, cvt, mul, fma) however many draft rows there are.
+// Each wavefront copies its own K segment of the activations into LDS once (wave-private, no barrier).
+typedef int lg_v4i __attribute__((ext_vector_type(4)));
+typedef int lg_v16i __attribute__((ext_vector_type(16)));
+typedef unsigned lg_v2u __attribute__((ext_vector_type(2)));
+template <int M>
+__global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];     // [8 segments][nit][80 dwords]
+    __shared__ float red[8][LG_HIP_MAX_ROWS_DEV][64];
+    constexpr int CH = 2;
+    const int lane = threadIdx.x & 63, n = lane & 31, h = lane >> 5;
+    const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));      // K segment of this wavefront
+    const int t = blockIdx.x, nb = a.k >> 5, nit = nb >> 3;
+    const uint8_t *wt = a.w + ((size_t)t * nb + (size_t)s * nit) * LG_TILE;
+    uint4 wq[CH], nwq[CH]; uint32_t wd[CH], nwd[CH];
+    auto fetch = [&](int it0) {
+        #pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;
+            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
+            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+        }
+    };
+    fetch(0);
+    unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
+    {
+        const uint4 *src = (const uint4 *)(a.q_in + (size_t)s * nit * (LG_MU_DWORDS * 4));
+        for (int i = lane; i < nit * (LG_MU_DWORDS / 4); i += 64) ((uint4 *)la)[i] = src[i];
+        // read back below by other lanes of this wavefront only: LDS serves a wavefront's accesses in order,
+        // the fences keep the compiler from moving the reads above the writes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    float pg[4] = { 0.0f, 0.0f, 0.0f, 0.0f }, pu[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+    const int arow = n < 8 ? n : 7;                           // operand rows past the 8 slots: any readable bytes
+    for (int it0 = 0; it0 < nit; it0 += CH) {
+        #pragma unroll
+        for (int u = 0; u < CH; ++u) { wq[u] = nwq[u]; wd[u] = nwd[u]; }
+        if (it0 + CH < nit) fetch(it0 + CH);
+        #pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if (it0 + c >= nit) break;
+            const unsigned char *lb = la + (size_t)(it0 + c) * (LG_MU_DWORDS * 4);
+            const lg_v4i av = *(const lg_v4i *)(lb + arow * 32 + h * 16);
+            const int4 sc0 = *(const int4 *)(lb + 256 + h * 32), sc1 = *(const int4 *)(lb + 256 + h * 32 + 16);
+            const uint4 q = wq[c];
+            const lg_v2u s0 = __builtin_amdgcn_permlane32_swap(q.x, q.z, false, false);
+            const lg_v2u s1 = __builtin_amdgcn_permlane32_swap(q.y, q.w, false, false);
+            const lg_v2u sd = __builtin_amdgcn_permlane32_swap(wd[c], wd[c], false, false);
+            lg_v4i bg, bu;
+            bg.x = s0.x & 0x0F0F0F0F; bg.y = s1.x & 0x0F0F0F0F; bg.z = (s0.x >> 4) & 0x0F0F0F0F; bg.w = (s1.x >> 4) & 0x0F0F0F0F;
+            bu.x = s0.y & 0x0F0F0F0F; bu.y = s1.y & 0x0F0F0F0F; bu.z = (s0.y >> 4) & 0x0F0F0F0F; bu.w = (s1.y >> 4) & 0x0F0F0F0F;
+            const float dg = lg_h2f((uint16_t)sd.x), du = lg_h2f((uint16_t)sd.y);
+            const lg_v16i z = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+            const lg_v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bg, z, 0, 0, 0);
+            const lg_v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bu, z, 0, 0, 0);
+            const float xd[4] = { __int_as_float(sc0.x), __int_as_float(sc0.z), __int_as_float(sc1.x), __int_as_float(sc1.z) };
+            const int s8[4] = { sc0.y, sc0.w, sc1.y, sc1.w };
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pg[i] = lg_fmaf(xd[i] * dg, (float)(d0[i] + s8[i]), pg[i]);
+                pu[i] = lg_fmaf(xd[i] * du, (float)(d1[i] + s8[i]), pu[i]);
+            }
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) { red[s][4 * h + i][n] = pg[i]; red[s][4 * h + i][32 + n] = pu[i]; }
     __syncthreads();
     for (int j = threadIdx.x >> 5; j < M; j += 16) {         // half-wavefront per row, one FFN column per lane
         const int i = threadIdx.x & 31;
