@@ -295,16 +295,23 @@ __device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChu
         for (int u = 0; u < LG_U; ++u) {
             if (it0 + u >= nit) break;
             const int it = it0 + u, b = c * nit + it;        // b: block of the natural order (for DUMP)
+            // the LDS reads of all M rows go out together, ahead of the first dot: left to itself the compiler
+            // interleaves them row by row and the wavefront waits out an LDS round trip per row
+            float2 ds[M]; int4 a0[M], a1[M];
             #pragma unroll
             for (int j = 0; j < M; ++j) {
-                const float2 ds = actds[j * nb + it * S + c];
+                ds[j] = actds[j * nb + it * S + c];
                 const int8_t *au = act + (size_t)j * k + (size_t)(it * 2 * S + c) * 16;
-                const int4 a0 = *(const int4 *)au, a1 = *(const int4 *)(au + S * 16);
+                a0[j] = *(const int4 *)au; a1[j] = *(const int4 *)(au + S * 16);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            #pragma unroll
+            for (int j = 0; j < M; ++j) {
                 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const int dot = lg_block_dot(cur.q[g][u], a0, a1, __float_as_int(ds.y));
+                    const int dot = lg_block_dot(cur.q[g][u], a0[j], a1[j], __float_as_int(ds[j].y));
                     if (DUMP) dots[((size_t)j * m + row[g]) * nb + b] = dot;
-                    acc[g][j] = lg_fmaf(ds.x * lg_h2f((uint16_t)cur.s[g][u]), (float)dot, acc[g][j]);
+                    acc[g][j] = lg_fmaf(ds[j].x * lg_h2f((uint16_t)cur.s[g][u]), (float)dot, acc[g][j]);
                 }
             }
         }
@@ -924,7 +931,6 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
     uint16_t *kt = (uint16_t *)(qs + (size_t)G * hd);         // [32][kst]
     uint16_t *vt = kt + 32 * kst;                             // [32][kst]
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
-    uint32_t *vmask = (uint32_t *)(es + G * 32);              // [G]
     const int kvh = blockIdx.y, j = blockIdx.z;
     const int pos0 = ctl->pos + a.pos_off, pj = pos0 + j;
     const int startj = lg_win_start(pj, a.window);
@@ -983,12 +989,9 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
             const float mx = lg_max_n(s, 32);
             const float e = valid ? lg_expf(s - mx) : 0.0f;
             const float l = lg_sum32(e);
-            const unsigned long long bal = __ballot(valid);
-            const uint32_t mask = (uint32_t)(threadIdx.x & 32 ? bal >> 32 : bal);
             if (hf == 0) {
                 es[g * 32 + sl] = e;
                 if (sl == 0) {
-                    vmask[g] = mask;
                     const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
                     a.pm[pi] = mx; a.pl[pi] = l;
                 }
@@ -997,19 +1000,30 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
     }
     __syncthreads();
     // acc[d] = sum over valid slots of e * V[slot][d]; thread = (head g, 4 dims)
+    // The valid slots of a tile are one run [lo, hi) (positions startj..pj), the same for every head of the
+    // row: 8 slots are read at a time, clamped to the tile, and the fma of a slot past the run is skipped
+    // by a wavefront-uniform test after all 16 reads are in flight.
+    const int lo = startj > t0 ? startj - t0 : 0, hi = pj - t0 + 1 < 32 ? pj - t0 + 1 : 32;
     for (int unit = threadIdx.x; unit < G * (hd >> 2); unit += LG_WG) {
         const int g = unit / (hd >> 2), d0 = (unit - g * (hd >> 2)) << 2;
-        const uint32_t mask = vmask[g];
         float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        #pragma unroll 8
-        for (int sl = 0; sl < 32; ++sl) {
-            if (!(mask >> sl & 1)) continue;
-            const float e = es[g * 32 + sl];
-            const uint2 v4 = *(const uint2 *)(vt + sl * kst + d0);
-            acc.x = lg_fmaf(e, lg_h2f((uint16_t)(v4.x & 0xFFFF)), acc.x);
-            acc.y = lg_fmaf(e, lg_h2f((uint16_t)(v4.x >> 16)), acc.y);
-            acc.z = lg_fmaf(e, lg_h2f((uint16_t)(v4.y & 0xFFFF)), acc.z);
-            acc.w = lg_fmaf(e, lg_h2f((uint16_t)(v4.y >> 16)), acc.w);
+        for (int sl0 = lo; sl0 < hi; sl0 += 8) {
+            float e8[8]; uint2 v8[8];
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int sl = sl0 + u < 32 ? sl0 + u : 31;
+                e8[u] = es[g * 32 + sl];
+                v8[u] = *(const uint2 *)(vt + sl * kst + d0);
+            }
+            #pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (sl0 + u < hi) {
+                    acc.x = lg_fmaf(e8[u], lg_h2f((uint16_t)(v8[u].x & 0xFFFF)), acc.x);
+                    acc.y = lg_fmaf(e8[u], lg_h2f((uint16_t)(v8[u].x >> 16)), acc.y);
+                    acc.z = lg_fmaf(e8[u], lg_h2f((uint16_t)(v8[u].y & 0xFFFF)), acc.z);
+                    acc.w = lg_fmaf(e8[u], lg_h2f((uint16_t)(v8[u].y >> 16)), acc.w);
+                }
+            }
         }
         const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
         *(float4 *)(a.pacc + pi * hd + d0) = acc;
