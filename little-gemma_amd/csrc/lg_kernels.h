@@ -175,7 +175,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
             uint32_t *blk = (uint32_t *)s.q + (size_t)(quad >> 3) * LG_MU_DWORDS;
             const int dw = quad & 7;
             blk[j * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))] = packed;
-            if ((t & 7) == 0) *(int2 *)(blk + 64 + 2 * j) = make_int2(__float_as_int(d), -8 * sum);
+            if ((t & 7) == 0) *(float2 *)(blk + 64 + 2 * j) = make_float2(d, 12582912.0f + (float)(8 * sum));
             continue;
         }
         *(uint32_t *)(s.q + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
 // tile keeps weight row l whole in lane l, so the two halves of the wavefront first trade 8 bytes each
 // (v_permlane32_swap): lane (n, h) then holds nibble bytes 8h..8h+7 of gate row n and of up row n, i.e.
 // K = 8h..8h+7 and 16+8h..16+8h+7.  The activation bytes are stored in that order (dwords 0 1 4 5 | 2 3 6 7
-// of a row's 32), 80 dwords per block: 8 row slots x 8 dwords, then 8 x {scale, -8*sum}.  Result register
+// of a row's 32), 80 dwords per block: 8 row slots x 8 dwords, then 8 x {scale, 12582912 + 8*sum as a float}.  Result register
 // i of lane (n, h) is draft row 4h+i of column n, so a lane applies 4 scale pairs per column, and the
 // per-block float work is 8 x (add, cvt, mul, fma) however many draft rows there are.
 // Each wavefront copies its own K segment of the activations into LDS once (wave-private, no barrier).
@@ -529,6 +529,12 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
     float pg[4] = { 0.0f, 0.0f, 0.0f, 0.0f }, pu[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+    // The accumulators start at the bit pattern of 1.5 * 2^23 = 12582912.0f: the integer dot (|dot| < 2^22) lands
+    // in the mantissa, the result read as a float is 12582912 + dot exactly, and subtracting the stored
+    // 12582912 + 8*sum gives (float)(dot - 8*sum) exactly, in one instruction per output.
+    lg_v16i magic;
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;
     const int arow = n < 8 ? n : 7;                           // operand rows past the 8 slots: any readable bytes
     for (int it0 = 0; it0 < nit; it0 += CH) {
         #pragma unroll
@@ -548,15 +554,14 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
             bg.x = s0.x & 0x0F0F0F0F; bg.y = s1.x & 0x0F0F0F0F; bg.z = (s0.x >> 4) & 0x0F0F0F0F; bg.w = (s1.x >> 4) & 0x0F0F0F0F;
             bu.x = s0.y & 0x0F0F0F0F; bu.y = s1.y & 0x0F0F0F0F; bu.z = (s0.y >> 4) & 0x0F0F0F0F; bu.w = (s1.y >> 4) & 0x0F0F0F0F;
             const float dg = lg_h2f((uint16_t)sd.x), du = lg_h2f((uint16_t)sd.y);
-            const lg_v16i z = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-            const lg_v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bg, z, 0, 0, 0);
-            const lg_v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bu, z, 0, 0, 0);
+            const lg_v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bg, magic, 0, 0, 0);
+            const lg_v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bu, magic, 0, 0, 0);
             const float xd[4] = { __int_as_float(sc0.x), __int_as_float(sc0.z), __int_as_float(sc1.x), __int_as_float(sc1.z) };
-            const int s8[4] = { sc0.y, sc0.w, sc1.y, sc1.w };
+            const float cf[4] = { __int_as_float(sc0.y), __int_as_float(sc0.w), __int_as_float(sc1.y), __int_as_float(sc1.w) };
             #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                pg[i] = lg_fmaf(xd[i] * dg, (float)(d0[i] + s8[i]), pg[i]);
-                pu[i] = lg_fmaf(xd[i] * du, (float)(d1[i] + s8[i]), pu[i]);
+                pg[i] = lg_fmaf(xd[i] * dg, __int_as_float(d0[i]) - cf[i], pg[i]);
+                pu[i] = lg_fmaf(xd[i] * du, __int_as_float(d1[i]) - cf[i], pu[i]);
             }
         }
     }

@@ -99,6 +99,9 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
     float p[16];
     #pragma unroll
     for (int i = 0; i < 16; ++i) p[i] = 0.0f;
+    lg_v16i magic, acc;
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;      // 12582912.0f
     fetch(0);
     for (int it0 = 0; it0 < nit; it0 += G::U) {
         unsigned char *cbase = smem + (size_t)((it0 / G::U) & 1) * G::U * G::step_bytes;
@@ -127,21 +130,25 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
             av[0] = (int)(a.x & 0x0F0F0F0Fu); av[1] = (int)(a.y & 0x0F0F0F0Fu);
             av[2] = (int)((a.x >> 4) & 0x0F0F0F0Fu); av[3] = (int)((a.y >> 4) & 0x0F0F0F0Fu);
             bv[0] = (int)b0[u].x; bv[1] = (int)b0[u].y; bv[2] = (int)b1[u].x; bv[3] = (int)b1[u].y;
-            lg_v16i acc = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc, 0, 0, 0);
+            // The accumulator starts at the bit pattern of 1.5 * 2^23: the integer dot (|dot| < 2^22) lands in the
+            // mantissa, so the result read as a float is 12582912 + dot exactly, and one float subtraction of
+            // 12582912 + 8*sum gives (float)(dot - 8*sum) exactly: one instruction per output instead of an
+            // integer subtract and a conversion.
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, magic, 0, 0, 0);
             const int corr = 8 * __float_as_int(xs[u].y);
+            const float cf = 12582912.0f + (float)corr;
             #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const float4 d4 = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
                 const float dv[4] = { d4.x, d4.y, d4.z, d4.w };
                 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int dot = acc[4 * g + j] - corr;
+                    const float fdot = __int_as_float(acc[4 * g + j]) - cf;
                     if (DUMP) {
                         const int row = 32 * rb + 8 * g + 4 * h + j;
-                        if (tile * LG_WIDE + n < rows) dots[((size_t)(tile * LG_WIDE + n) * m_total + row) * nb + (c * nit + it)] = dot;
+                        if (tile * LG_WIDE + n < rows) dots[((size_t)(tile * LG_WIDE + n) * m_total + row) * nb + (c * nit + it)] = (int)fdot;
                     }
-                    p[4 * g + j] = lg_fmaf(xs[u].x * dv[j], (float)dot, p[4 * g + j]);
+                    p[4 * g + j] = lg_fmaf(xs[u].x * dv[j], fdot, p[4 * g + j]);
                 }
             }
         }
