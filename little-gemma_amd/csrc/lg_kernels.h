@@ -3,7 +3,7 @@
 // One step is a graph of small kernels; a dependent kernel boundary costs ~1.5 us on MI355X, an
 // all-CU software barrier ten times that, so the step is NOT a persistent megakernel.  Per layer:
 //   rows(norm+q8) -> qkv -> qkv_post(norm,rope,KV write) -> attn tiles -> attn merge(+q8) -> o
-//   -> rows -> gate/up+GeGLU(+q8) -> down -> rows -> ple gate(+q8) -> ple proj
+//   -> rows -> gate/up+GeGLU(+q8) -> down -> rows+ple gate(+q8) -> ple proj
 // Every matmul reads its M activation rows already quantized (int8 + per-32 {scale,sum}) and
 // stages them in LDS once per workgroup; weights stream from HBM exactly once per step in
 // pre-tiled order (one 16-byte + one 2-byte load per lane per tile).  All kernels read the block
