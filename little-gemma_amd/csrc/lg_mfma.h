@@ -32,13 +32,17 @@ typedef int lg_v16i __attribute__((ext_vector_type(16)));
 
 #define LG_WIDE_WG 512                     // 8 wavefronts: two per SIMD, one K segment each
 
+#ifndef LG_WIDE_U
+#define LG_WIDE_U 1
+#endif
 struct MfmaGeo {
     static constexpr int AW_STRIDE = 33;   // uint2 per (segment, half) row of the operand store (32 + 1 pad)
     static constexpr size_t aw_bytes = (size_t)8 * 2 * AW_STRIDE * 8;
     static constexpr size_t dw_bytes = (size_t)8 * 32 * 4;
-    static constexpr int U = 5;            // steps per chunk: tiles and activation operands are requested a chunk ahead
+    static constexpr int U = LG_WIDE_U;    // steps per chunk: tiles and activation operands are requested a chunk ahead
     static constexpr size_t step_bytes = aw_bytes + dw_bytes;
-    static constexpr size_t lds_bytes = 2 * U * step_bytes;       // double-buffered chunks; the final exchange (32 KiB) reuses it
+    static constexpr size_t chunk_bytes = 2 * U * step_bytes;     // double-buffered chunks
+    static constexpr size_t lds_bytes = chunk_bytes > 32768 ? chunk_bytes : 32768;   // the final exchange (32 KiB) reuses it
 };
 static_assert(8 * 16 * 64 * 4 <= MfmaGeo::lds_bytes, "the final exchange must fit");
 
@@ -201,7 +205,7 @@ __device__ __forceinline__ void lg_wide_quant32(float *vbuf, int8_t *q, int kq, 
 // Gate/up with the GeGLU and the q8 of its result (see lg_k_geglu_t): row-block tiles, per 32 FFN
 // columns a block of 32 gate rows followed by the block of the 32 up rows.  grid = (n_ff/32, row tiles).
 template <int R>
-__global__ __launch_bounds__(LG_WIDE_WG) void lg_k_mm_geglu_wide(GegluArgs a, int rows) {
+__global__ __launch_bounds__(LG_WIDE_WG, 2) void lg_k_mm_geglu_wide(GegluArgs a, int rows) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float vbuf[32 * 33];
     float g[2], u[2];
