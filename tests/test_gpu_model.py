@@ -59,7 +59,8 @@ def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, gol
         gpu.close(); o.close()
 
 
-@pytest.mark.parametrize("name,rows", [("tiny", 2), ("tiny", 4), ("tiny", 5), ("tiny_full", 4), ("tiny_full", 8)])
+@pytest.mark.parametrize("name,rows", [("tiny", 2), ("tiny", 4), ("tiny", 5), ("tiny_full", 3), ("tiny_full", 4), ("tiny_full", 6),
+                                       ("tiny_full", 7), ("tiny_full", 8)])
 def test_verify_equals_decode_and_accept_counts(lg, ob, gpu_required, model_path, name, rows):
     """Row j of a verify block is bit-identical to a plain decode at pos+j (the reference's central
     invariant, src/cuda/model-cuda.cuh:520-526), and with drafts whose first mismatch is planted the
