@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel (gate/up + GeGLU at the E4B shape), from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised under profiles/ (scaled by the copy-kernel calibration given there):
 # reads 29.55 MB for M = 5 (29.36 MB for M = 1), writes 0.15 MB (0.03 MB).  Other shapes have no counter run.
-MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.55e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.36e6 + 0.03e6}
+MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.40e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.27e6 + 0.03e6}
 CTX = 2048
 WORKLOADS = {
     "e4b": ("E4B-shape q4_0 verify step (42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144, "
