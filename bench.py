@@ -141,6 +141,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--seed", type=int, default=7)
     ap.add_argument("--prefill", type=int, default=1024, help="positions of the prompt-processing measurement; 0 skips it")
+    ap.add_argument("--mtp-steps", type=int, default=24, help="steps of the draft-head loop measurement (4 chained device drafts + verify); 0 skips it")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU; the verify step is not sharded (run with --gpus 1)", file=sys.stderr)
@@ -157,7 +158,7 @@ def main():
         os.replace(path + ".tmp", path)
         log(f"wrote {path} in {time.time() - t0:.1f}s")
     total = a.steps + a.warmup
-    max_seq = max(ctx + (total + 2) * a.rows + 64, a.prefill + 64)
+    max_seq = max(ctx + (total + 2) * a.rows + 64, a.prefill + 64, ctx + (a.mtp_steps + 4) * a.rows + 64)
     t0 = time.time()
     gpu = lg.hiplib.HipBackend(path, max_seq, max_rows=max(a.rows, 1))
     log(f"weights on the device in {time.time() - t0:.1f}s")
@@ -227,6 +228,35 @@ def main():
         "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
                    "wall_ms_per_step": 1e3 * wall / a.steps, "plain_decode_ms_per_token_host_sync": decode_ms},
     }
+    # the loop a draft head drives (the reference's run.c with -mtp): per step K = rows-1 chained drafts on the
+    # device head (synthetic gemma4-assistant weights: its drafts are rarely accepted, the step cost does not
+    # depend on that), then the verify step; host clock around synchronous calls, from the seeded cache
+    if a.mtp_steps > 0 and a.rows >= 2:
+        apath = os.path.join(a.model_dir, f"lg_bench_{a.workload}_assistant.gguf")
+        if not os.path.exists(apath):
+            lg.synth.write_assistant(apath + ".tmp", **lg.synth.assistant_for(spec))
+            os.replace(apath + ".tmp", apath)
+        lg.hiplib.hip_check(H.lg_hip_kv_restore_prefix(gpu.dkv, ctx), "kv_restore_prefix")
+        head = gpu.mtp_open(apath)
+        tok, pos, t_draft, t_verify, emitted = first_tok, ctx, 0.0, 0.0, 0
+        tok = gpu.forward_next(tok, pos); pos += 1               # the head reads the target's hidden state of this token
+        for step in range(a.mtp_steps + 2):
+            t0 = time.time()
+            toks = [tok]
+            for j in range(1, a.rows):
+                d = gpu.mtp_draft(head, toks[-1], pos + j - 1, chain=j > 1)
+                toks.append(d if d >= 0 else toks[-1])
+            t1 = time.time()
+            adv, out = gpu.forward_spec(np.array(toks, np.int32), pos)
+            t2 = time.time()
+            if step >= 2:                                        # two untimed steps: graph captures of the head and its chain
+                t_draft += t1 - t0; t_verify += t2 - t1; emitted += adv
+            pos += adv; tok = int(out[adv - 1])
+        gpu.mtp_close(head)
+        line["mtp_loop"] = {"steps": a.mtp_steps, "drafts_per_step": a.rows - 1,
+                            "draft_ms_per_step": 1e3 * t_draft / a.mtp_steps, "verify_ms_per_step": 1e3 * t_verify / a.mtp_steps,
+                            "ms_per_step": 1e3 * (t_draft + t_verify) / a.mtp_steps, "tokens_per_step": emitted / a.mtp_steps,
+                            "head": "synthetic gemma4-assistant (4 blocks, 256 wide), host round trip per draft"}
     # prompt processing on the matrix cores: 32-row blocks through the int8 MFMA kernels (a fresh cache, host clock
     # around a synchronised call; the first call captures the graph and is not timed)
     if a.prefill > 0:
