@@ -931,9 +931,13 @@ __device__ __forceinline__ int lg_win_start(int pos, int window) {
 __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int hd = a.hd, G = a.H / a.nkv;
-    const int kst = hd + 8;                                   // padded K/V tile row (halves)
+    const int kst = hd + 8;                                   // padded V tile row (halves): 16-byte rows, read along the row
+    // K is read down a column (32 lanes = 32 key slots, the same two dims): an odd row stride in dwords spreads
+    // the slots over all 32 banks (a 16-byte-aligned stride leaves them 4 to a bank, and the score loop is
+    // bound by exactly these reads); the price is 4-byte stores when the tile is staged
+    const int ksk = hd + 2;                                   // K tile row (halves)
     float *qs = (float *)smem;                                // [G][hd]
-    uint16_t *kt = (uint16_t *)(qs + (size_t)G * hd);         // [32][kst]
+    uint16_t *kt = (uint16_t *)(qs + (size_t)G * hd);         // [32][ksk]
     uint16_t *vt = kt + 32 * kst;                             // [32][kst]
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
     const int kvh = blockIdx.y, j = blockIdx.z;
@@ -949,15 +953,15 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
         const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
         for (int i0 = threadIdx.x; i0 < nk8; i0 += 4 * LG_WG) {
             // element u of the batch: LDS offset (halves) in `lo`, cache offset in `go`, validity in `ok`
-            auto place = [&](int u, int &lo, size_t &go, bool &ok) {
+            auto place = [&](int u, int &lo, int &lk, size_t &go, bool &ok) {
                 const int idx = min(i0 + u * LG_WG, nk8 - 1);
                 const int sl = idx / per_row, e0 = (idx - sl * per_row) << 3, t = t0 + sl;
                 ok = t >= startj && t <= pj;
-                lo = sl * kst + e0;
+                lo = sl * kst + e0; lk = sl * ksk + e0;
                 go = (size_t)((ok ? t : pj) % a.seq) * a.kv_dim + (size_t)kvh * hd + e0;
             };
-            int l0, l1, l2, l3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3;
-            place(0, l0, g0, ok0); place(1, l1, g1, ok1); place(2, l2, g2, ok2); place(3, l3, g3, ok3);
+            int l0, l1, l2, l3, m0, m1, m2, m3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3;
+            place(0, l0, m0, g0, ok0); place(1, l1, m1, g1, ok1); place(2, l2, m2, g2, ok2); place(3, l3, m3, g3, ok3);
             const uint4 k0 = a.kc4(g0), k1 = a.kc4(g1), k2 = a.kc4(g2), k3 = a.kc4(g3);
             const uint4 v0 = a.vc4(g0), v1 = a.vc4(g1), v2 = a.vc4(g2), v3 = a.vc4(g3);
             __builtin_amdgcn_sched_barrier(0);
@@ -965,10 +969,14 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
                 const uint32_t mk = ok ? 0xFFFFFFFFu : 0u;
                 return make_uint4(v.x & mk, v.y & mk, v.z & mk, v.w & mk);
             };
-            *(uint4 *)(kt + l0) = keep(k0, ok0);  *(uint4 *)(vt + l0) = keep(v0, ok0);
-            *(uint4 *)(kt + l1) = keep(k1, ok1);  *(uint4 *)(vt + l1) = keep(v1, ok1);
-            *(uint4 *)(kt + l2) = keep(k2, ok2);  *(uint4 *)(vt + l2) = keep(v2, ok2);
-            *(uint4 *)(kt + l3) = keep(k3, ok3);  *(uint4 *)(vt + l3) = keep(v3, ok3);
+            auto putk = [&](int lk, uint4 v) {               // four 4-byte stores: K rows are only 4-byte aligned
+                uint32_t *d = (uint32_t *)(kt + lk);
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+            };
+            putk(m0, keep(k0, ok0));  *(uint4 *)(vt + l0) = keep(v0, ok0);
+            putk(m1, keep(k1, ok1));  *(uint4 *)(vt + l1) = keep(v1, ok1);
+            putk(m2, keep(k2, ok2));  *(uint4 *)(vt + l2) = keep(v2, ok2);
+            putk(m3, keep(k3, ok3));  *(uint4 *)(vt + l3) = keep(v3, ok3);
         }
     }
     __syncthreads();
@@ -978,7 +986,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
         for (int unit = part; unit < 2 * G; unit += LG_WG / 32) {
             const int g = unit >> 1, hf = unit & 1;
             const float *qv = qs + (size_t)g * hd + 2 * hf;
-            const uint16_t *kr = kt + sl * kst + 2 * hf;
+            const uint16_t *kr = kt + sl * ksk + 2 * hf;
             float ax = 0.0f, ay = 0.0f;                       // chains 2hf and 2hf+1
             for (int i = 0; i < hd; i += 8) {
                 const float2 q0 = *(const float2 *)(qv + i), q1 = *(const float2 *)(qv + i + 4);
