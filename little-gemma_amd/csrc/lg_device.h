@@ -76,15 +76,22 @@ __device__ __forceinline__ float lg_sum16(float v) {
     v = v + lg_dpp_f<LG_DPP_MIRROR16>(v);
     return v;
 }
+// Lane l and lane l^16 (l^32): v_permlane16_swap (v_permlane32_swap) with the value as both operands leaves
+// the even rows (the lower half) in one result and the odd rows (the upper half) in the other, each in every
+// lane of the pair; combining the two results gives v[l] (+) v[l^16] in one VALU step, where a shuffle through
+// the LDS crossbar costs an LDS round trip.  The combination is commutative, so the order of the pair is free.
+typedef unsigned lg_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ lg_u2 lg_pair16(uint32_t v) { return __builtin_amdgcn_permlane16_swap(v, v, false, false); }
+__device__ __forceinline__ lg_u2 lg_pair32(uint32_t v) { return __builtin_amdgcn_permlane32_swap(v, v, false, false); }
+__device__ __forceinline__ float lg_add_x16(float v) { const lg_u2 r = lg_pair16(__float_as_uint(v)); return __uint_as_float(r.x) + __uint_as_float(r.y); }
+__device__ __forceinline__ float lg_add_x32(float v) { const lg_u2 r = lg_pair32(__float_as_uint(v)); return __uint_as_float(r.x) + __uint_as_float(r.y); }
 __device__ __forceinline__ float lg_sum32(float v) {
     v = lg_sum16(v);
-    v = v + __shfl_xor(v, 16);
-    return v;
+    return lg_add_x16(v);
 }
 __device__ __forceinline__ float lg_wave_sum64(float v) {
     v = lg_sum32(v);
-    v = v + __shfl_xor(v, 32);
-    return v;
+    return lg_add_x32(v);
 }
 template <int S>
 __device__ __forceinline__ float lg_sum_seg(float v) {       // S = 8 or 32 adjacent lanes
@@ -100,8 +107,8 @@ __device__ __forceinline__ float lg_max8(float v) {
 __device__ __forceinline__ float lg_max_n(float v, int n) {       // n = 8, 32 or 64 lanes
     v = lg_max8(v);
     if (n >= 16) v = fmaxf(v, lg_dpp_f<LG_DPP_MIRROR16>(v));
-    if (n >= 32) v = fmaxf(v, __shfl_xor(v, 16));
-    if (n >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+    if (n >= 32) { const lg_u2 r = lg_pair16(__float_as_uint(v)); v = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y)); }
+    if (n >= 64) { const lg_u2 r = lg_pair32(__float_as_uint(v)); v = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y)); }
     return v;
 }
 __device__ __forceinline__ int lg_isum_n(int v, int n) {          // n = 8 or 32 lanes
@@ -109,7 +116,7 @@ __device__ __forceinline__ int lg_isum_n(int v, int n) {          // n = 8 or 32
     v += lg_dpp_i<LG_DPP_SWAP2>(v);
     v += lg_dpp_i<LG_DPP_MIRROR8>(v);
     if (n >= 16) v += lg_dpp_i<LG_DPP_MIRROR16>(v);
-    if (n >= 32) v += __shfl_xor(v, 16);
+    if (n >= 32) { const lg_u2 r = lg_pair16((uint32_t)v); v = (int)r.x + (int)r.y; }
     return v;
 }
 

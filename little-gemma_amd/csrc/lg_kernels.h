@@ -996,8 +996,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
                 ax = lg_fmaf(q1.x, lg_h2f((uint16_t)(k1 & 0xFFFF)), ax);
                 ay = lg_fmaf(q1.y, lg_h2f((uint16_t)(k1 >> 16)), ay);
             }
-            const float mine = ax + ay, other = __shfl_xor(mine, 32);
-            float s = hf ? other + mine : mine + other;       // (a0+a1) + (a2+a3)
+            float s = lg_add_x32(ax + ay);                     // (a0+a1) + (a2+a3): the two halves sit 32 lanes apart
             if (!valid) s = -INFINITY;
             const float mx = lg_max_n(s, 32);
             const float e = valid ? lg_expf(s - mx) : 0.0f;
