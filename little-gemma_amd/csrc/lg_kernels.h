@@ -45,9 +45,10 @@ struct RowArgs {
 };
 
 // Sum over the 256 lanes of a workgroup in adjacent-pair tree order; every thread gets the result.
+// `scratch4` must not be in use by an earlier call that other wavefronts may still be reading: each call
+// site has its own four floats, so one barrier is enough.
 __device__ __forceinline__ float lg_block_sum256(float v, float *scratch4) {
     v = lg_wave_sum64(v);
-    __syncthreads();
     if ((threadIdx.x & 63) == 0) scratch4[threadIdx.x >> 6] = v;
     __syncthreads();
     return (scratch4[0] + scratch4[1]) + (scratch4[2] + scratch4[3]);
@@ -81,7 +82,7 @@ __device__ __forceinline__ size_t lg_q8_ds_idx(int k, int j, int b) {
 #define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
-    __shared__ float red[4];
+    __shared__ float red[2][4];
     const int t = threadIdx.x, j = blockIdx.x;
     const int E = s.E, nq = E >> 2;                          // float4 quads in a row; thread t owns quads t + 256*v
     float4 xv[LG_ROWV], dv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         float ss = 0.0f;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
-        ss = lg_block_sum256(ss, red);
+        ss = lg_block_sum256(ss, red[0]);
         const float sc = 1.0f / sqrtf(ss / (float)E + s.eps);
         const bool has_os = s.os != nullptr;
         const float osv = has_os ? s.os[0] : 1.0f;
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         float ss = 0.0f;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(xv[v], ss);
-        ss = lg_block_sum256(ss, red);
+        ss = lg_block_sum256(ss, red[1]);
         const float sc = 1.0f / sqrtf(ss / (float)E + s.eps);
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
