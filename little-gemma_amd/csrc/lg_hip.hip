@@ -614,6 +614,17 @@ struct Launcher {
 #define LAUNCH(cls, kernel, grid, block, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { lx.begin(cls); \
     hipLaunchKernelGGL(kernel, grid, block, lds, lx.m->stream, __VA_ARGS__); lx.end(); } } while (0)
 
+// Compute units of the current device (asked once).
+static int cu_count() {
+    static int n = -1;
+    if (n < 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) v = 0;
+        n = v;
+    }
+    return n;
+}
+
 // Plain matmul launch: picks the segment count from k and the workgroup shape from the row count
 // (small matrices get one wavefront per workgroup so that every CU has work).
 template <int M, bool DUMP>
@@ -628,7 +639,10 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
     } else {
     const size_t lds = lds_mm(M, a.k);
     if (S == 32) {
-        const int W = 4;
+        // 4 wavefronts (8 rows) per workgroup, or 5 when that makes exactly one workgroup per CU (2560 rows on 256 CUs):
+        // with 320 workgroups a quarter of the CUs would hold two of them and the kernel would wait for those
+        const int cus = cu_count();
+        const int W = (ngroups % 5 == 0 && ngroups / 5 <= cus && ngroups / 4 > cus) ? 5 : 4;
         LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
     } else if (ngroups >= 4096) {
         const int W = 4;

@@ -345,7 +345,7 @@ struct MmArgs {
 // Plain matmul: out[j][i] f32.  blockDim = 64*W wavefronts, each wavefront takes G neighbouring
 // row groups (G*64/S rows); grid covers ceil(groups / (W*G)) workgroups.
 template <int M, int S, int G, bool DUMP>
-__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm(MmArgs a) {
+__global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
