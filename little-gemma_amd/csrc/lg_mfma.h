@@ -129,7 +129,13 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
             const int it = it0 + u;
             const uint2 *aw = (const uint2 *)(cbase + (size_t)u * G::step_bytes);
             const float *dwf = (const float *)((const unsigned char *)aw + G::aw_bytes);
+            // operand and the 16 weight scales of this lane's outputs: all five LDS reads go out together, ahead of the
+            // MFMA (interleaved with the epilogue, as the compiler would have them, each costs an LDS round trip)
             const uint2 a = aw[(wave * 2 + h) * G::AW_STRIDE + n];
+            float4 d4[4];
+            #pragma unroll
+            for (int g = 0; g < 4; ++g) d4[g] = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
+            __builtin_amdgcn_sched_barrier(0);
             lg_v4i av, bv;
             av[0] = (int)(a.x & 0x0F0F0F0Fu); av[1] = (int)(a.y & 0x0F0F0F0Fu);
             av[2] = (int)((a.x >> 4) & 0x0F0F0F0Fu); av[3] = (int)((a.y >> 4) & 0x0F0F0F0Fu);
@@ -143,8 +149,7 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
             const float cf = 12582912.0f + (float)corr;
             #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const float4 d4 = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
-                const float dv[4] = { d4.x, d4.y, d4.z, d4.w };
+                const float dv[4] = { d4[g].x, d4[g].y, d4[g].z, d4[g].w };
                 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float fdot = __int_as_float(acc[4 * g + j]) - cf;
