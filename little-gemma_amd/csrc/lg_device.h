@@ -36,14 +36,21 @@ __host__ __device__ static inline int lg_segments(int k) { return (k >> 5) > 128
 // = w%2) lives at unit it*2S + half*S + c, and the block's {scale,sum} pair at it*S + c, with
 // c = b / nit, it = b % nit.  A wavefront's LDS reads are then consecutive 16-byte units (no bank
 // conflicts), and producers write this order directly.
-struct ActLayout { int S, nit; };
-__host__ __device__ static inline ActLayout lg_act_layout(int k) { const int S = lg_segments(k); return { S, (k >> 5) / S }; }
+// b / nit is taken as (b * inv) >> 16 with inv = 65536 / nit + 1: exact for b < 65536 / nit (a row has at most
+// a few hundred blocks), and two instructions per lane where a division by a run-time value costs about
+// fifteen; the layout itself is wavefront-uniform, so its own division runs on the scalar unit.
+struct ActLayout { int S, nit; unsigned inv; };
+__host__ __device__ static inline ActLayout lg_act_layout(int k) {
+    const int S = lg_segments(k), nit = (k >> 5) / S;
+    return { S, nit, 65536u / (unsigned)nit + 1u };
+}
+__host__ __device__ static inline int lg_act_seg(ActLayout a, int b) { return (int)(((unsigned)b * a.inv) >> 16); }
 __host__ __device__ static inline int lg_act_unit(ActLayout a, int w) {
-    const int b = w >> 1, c = b / a.nit, it = b - c * a.nit;
+    const int b = w >> 1, c = lg_act_seg(a, b), it = b - c * a.nit;
     return it * 2 * a.S + (w & 1) * a.S + c;
 }
 __host__ __device__ static inline int lg_act_block(ActLayout a, int b) {
-    const int c = b / a.nit, it = b - c * a.nit;
+    const int c = lg_act_seg(a, b), it = b - c * a.nit;
     return it * a.S + c;
 }
 
