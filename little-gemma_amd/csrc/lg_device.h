@@ -135,13 +135,23 @@ __device__ __forceinline__ float lg_sumsq4(float4 v, float acc) {
     return acc;
 }
 
+// amax / 127.0f for amax >= 0, in three instructions: with r = the float nearest to 1/127, q0 = amax * r,
+// the residual amax - 127*q0 is exact in one fma and the corrected quotient fma(residual, r, q0) equals the
+// correctly rounded IEEE quotient for every non-negative finite float (checked exhaustively on a CPU, all
+// 2,139,095,040 of them, subnormals included); the generic division sequence costs about ten instructions.
+__device__ __forceinline__ float lg_div127(float amax) {
+    const float r = 1.0f / 127.0f;
+    const float q0 = amax * r;
+    return lg_fmaf(lg_fmaf(-127.0f, q0, amax), r, q0);
+}
+
 // q8 quantization of 32 consecutive values held as one float4 in each of 8 adjacent lanes:
 // amax, d = amax/127, id = 1/d (0 when d == 0), q = rint_even(x*id), sum of q.
 // Returns the 4 packed int8; *d_out / *sum_out are the same in all 8 lanes.
 __device__ __forceinline__ uint32_t lg_quant4_8lanes(float4 h, float *d_out, int *sum_out) {
     float amax = fmaxf(fmaxf(fabsf(h.x), fabsf(h.y)), fmaxf(fabsf(h.z), fabsf(h.w)));
     amax = lg_max_n(amax, 8);
-    const float d = amax / 127.0f;
+    const float d = lg_div127(amax);
     const float id = d > 0.0f ? 1.0f / d : 0.0f;
     const int q0 = (int)lg_rintf(h.x * id), q1 = (int)lg_rintf(h.y * id);
     const int q2 = (int)lg_rintf(h.z * id), q3 = (int)lg_rintf(h.w * id);
@@ -153,7 +163,7 @@ __device__ __forceinline__ uint32_t lg_quant4_8lanes(float4 h, float *d_out, int
 // Same for 32 values held one per lane in 32 adjacent lanes (half a wavefront).
 __device__ __forceinline__ int lg_quant1_32lanes(float h, float *d_out, int *sum_out) {
     const float amax = lg_max_n(fabsf(h), 32);
-    const float d = amax / 127.0f;
+    const float d = lg_div127(amax);
     const float id = d > 0.0f ? 1.0f / d : 0.0f;
     const int q = (int)lg_rintf(h * id);
     *d_out = d;

@@ -193,3 +193,42 @@ def test_ring_rows(ob):
     assert L.lgo_ring_rows(512, 300) == 300                     # never more rows than positions
     for w in (100, 128, 511, 512, 1000):
         assert L.lgo_ring_rows(w, 1 << 20) % 32 == 0 and L.lgo_ring_rows(w, 1 << 20) >= w + 128 - 1
+
+
+def test_division_by_127_in_three_instructions_is_the_ieee_quotient():
+    """The device quantizer forms amax/127 as fma(fma(-127, q0, amax), r, q0) with q0 = amax*r, r = fl(1/127).
+    Exact rational arithmetic with one rounding per operation (what mul and fma do) must land on the
+    correctly rounded quotient: edge values and a seeded sample here; the full sweep over every non-negative
+    finite float was run once offline (0 mismatches)."""
+    from fractions import Fraction
+
+    def fl(x):                       # nearest float32 to a rational, ties to even, subnormals included
+        if x == 0:
+            return Fraction(0)
+        if x < 0:
+            return -fl(-x)
+        e = x.numerator.bit_length() - x.denominator.bit_length()
+        if Fraction(2) ** e > x:
+            e -= 1                   # 2^e <= x < 2^(e+1)
+        e = max(e, -126)             # below the normal range the spacing stays 2^-149
+        q = Fraction(2) ** (e - 23)
+        n = x / q
+        lo = n.numerator // n.denominator
+        rem = n - lo
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+            lo += 1
+        return lo * q
+
+    r = fl(Fraction(1, 127))
+    assert float(r) == float(np.float32(1.0) / np.float32(127.0))
+    rng = np.random.default_rng(127)
+    bits = np.concatenate([
+        np.array([0, 1, 2, 126, 127, 128, 0x007FFFFF, 0x00800000, 0x00800001, 0x3F800000, 0x42FE0000, 0x7F7FFFFF], np.uint32),
+        rng.integers(0, 0x7F800000, 3000, dtype=np.uint32),
+        rng.integers(0, 0x01000000, 500, dtype=np.uint32)])           # dense around the subnormal boundary
+    for b in bits:
+        a = Fraction(float(np.array([b], np.uint32).view(np.float32)[0]))
+        q0 = fl(a * r)
+        e = fl(a - 127 * q0)
+        q = fl(e * r + q0)
+        assert q == fl(a / 127), hex(int(b))
