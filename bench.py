@@ -34,8 +34,11 @@ CTX = 2048
 WORKLOADS = {
     "e4b": ("E4B-shape q4_0 verify step (42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144, "
             "5 sliding-512 : 1 global), ctx 2048", lg.synth.E4B),
+    "g12b": ("12B-shape q4_0 verify step (48 layers, d 3840, 16/8 heads x 256, FFN 15360, no PLE, vocab 262144, "
+             "5 sliding-1024 : 1 global), ctx 8192", lg.synth.G12B),
     "tiny": ("tiny 4-layer shape (plumbing check only: fits in cache, no bandwidth claim)", lg.synth.TINY),
 }
+WORKLOAD_CTX = {"e4b": CTX, "g12b": 8192, "tiny": 256}
 
 
 def log(*a):
@@ -150,7 +153,7 @@ def main():
     if rank != 0:
         return
     desc, spec = WORKLOADS[a.workload]
-    ctx = CTX if a.workload == "e4b" else 256
+    ctx = WORKLOAD_CTX[a.workload]
     path = os.path.join(a.model_dir, f"lg_bench_{a.workload}_seed{spec['seed']}.gguf")
     if not os.path.exists(path):
         t0 = time.time()
@@ -215,7 +218,8 @@ def main():
                 "launches_per_step": dom["launches"]}
     step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9
     line = {
-        "metric": "verified tok/s (E4B-shape q4_0, block-4, ctx 2048) + achieved HBM GB/s vs peak",
+        "metric": ("verified tok/s (E4B-shape q4_0, block-4, ctx 2048) + achieved HBM GB/s vs peak" if a.workload == "e4b" else
+                   f"verified tok/s ({a.workload} shape q4_0, {a.rows} rows, ctx {ctx}) + achieved HBM GB/s vs peak"),
         "value": value, "unit": "verified tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms / a.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 x int4 -> int32 block dots, f32 accumulate", "data": "synthetic",

@@ -579,6 +579,12 @@ extern "C" int lg_hip_kv_restore_prefix(lg_hip_kv *kv, int n) {
 
 // ---- launching --------------------------------------------------------------------------------
 static size_t lds_mm(int M, int k) { return (size_t)M * k + (size_t)M * (k / 32) * 8; }
+// lg_k_attn: queries of the G heads, K and V tiles, exponentials; with the q/k/v preparation fused in, a head
+// vector of staging per wavefront (16-byte aligned)
+static size_t attn_lds(int G, int hd, bool fused_post) {
+    const size_t b = (size_t)G * hd * 4 + (size_t)2 * 32 * (hd + 8) * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
+    return fused_post ? ((b + 15) & ~(size_t)15) + (size_t)(LG_WG / 64) * hd * 4 : b;
+}
 
 // Kernels that want more than the default dynamic LDS limit have it raised once per (kernel, size).
 template <typename K>
@@ -711,9 +717,12 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
         rows(y.attn_norm, nullptr);
+        bool fused_post = false;
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
             launch_mm<M, false>(lx, KC_QKV, a);
+            // blocks of the model itself, up to LG_HIP_MAX_ROWS rows: the attention kernel does this part as well
+            fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
             QkvPostArgs p{};
             p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
             p.H = H; p.nkv = y.nkv; p.hd = y.hd;
@@ -721,16 +730,23 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             p.q_rot = m->q_rot;
             p.kc = y.owns ? kv->k[L] : nullptr; p.vc = y.owns ? kv->v[L] : nullptr;
             p.seq = kv->seq[y.src]; p.kv_dim = y.kd; p.eps = m->eps;
-            LAUNCH(KC_QKVPOST, lg_k_qkv_post, dim3(H + (y.owns ? 2 * y.nkv : 0), M), dim3(64), 0, p, m->ctl);
+            if (!fused_post) LAUNCH(KC_QKVPOST, lg_k_qkv_post, dim3(H + (y.owns ? 2 * y.nkv : 0), M), dim3(64), 0, p, m->ctl);
         }
         {   // attention tiles + merge
-            const int G = H / y.nkv, kst = y.hd + 8;
+            const int G = H / y.nkv;
             AttnArgs a{};
             a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
-            const size_t lds = (size_t)G * y.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
-            LAUNCH(KC_ATTN, lg_k_attn, dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), lds, a, m->ctl);
+            if (fused_post) {
+                a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
+                a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
+                a.kcw = y.owns ? kv->k[L] : nullptr; a.vcw = y.owns ? kv->v[L] : nullptr; a.eps = m->eps;
+                if (y.hd <= 256) LAUNCH(KC_ATTN, (lg_k_attn<true, 1>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
+                else             LAUNCH(KC_ATTN, (lg_k_attn<true, 2>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
+            } else {
+                LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
+            }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
             LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
@@ -1169,15 +1185,14 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
 
 template <int M>
 static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl, int tiles, int repeats, float *kernel_ms) {
-    const int G = a.H / a.nkv, kst = a.hd + 8;
-    const size_t lds = (size_t)G * a.hd * 4 + (size_t)2 * 32 * kst * 2 + (size_t)G * 32 * 4 + (size_t)G * 4;
-    int rc = set_lds(lg_k_attn, lds);
+    const size_t lds = attn_lds(a.H / a.nkv, a.hd, false);
+    int rc = set_lds(lg_k_attn<false, 1>, lds);
     if (rc) return rc;
     hipEvent_t e0, e1;
     HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
     for (int r = 0; r < repeats + 1; ++r) {
         if (r == 1) HIP_TRY(hipEventRecord(e0, st));
-        hipLaunchKernelGGL(lg_k_attn, dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
+        hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
         hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
     }
     HIP_TRY(hipEventRecord(e1, st));

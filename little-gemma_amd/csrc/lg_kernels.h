@@ -854,46 +854,91 @@ struct QkvPostArgs {
     int seq, kv_dim;
     float eps;
 };
-__global__ __launch_bounds__(64) void lg_k_qkv_post(QkvPostArgs a, const StepCtl *ctl) {
-    __shared__ float vec[512];
-    const int lane = threadIdx.x, job = blockIdx.x, j = blockIdx.y, hd = a.hd, half = hd >> 1;
-    const int pos = ctl->pos + j;
-    const bool isq = job < a.H, isv = job >= a.H + a.nkv;
-    const int head = isq ? job : (job - a.H) % a.nkv;
-    const float *src = a.qkv + (size_t)j * a.ld + (isq ? (size_t)head * hd : (size_t)(isv ? a.v_off : a.k_off) + (size_t)head * hd);
-    const float *w = isq ? a.q_norm : (isv ? nullptr : a.k_norm);
-    float4 xv[2], wv[2];
-    float ss0 = 0.0f, ss1 = 0.0f;                            // lanes l and l+64 of the 256-lane sum order
+// One head vector (hd <= 512 floats) per wavefront, in two steps so that a wavefront with several vectors to do
+// has all their loads in flight first.  lg_head_load: 4 consecutive elements per lane (and 4 more at +256).
+// lg_head_finish: rmsnorm (weighted by `w`, or plain when w == nullptr) in the 256-lane sum order, then NeoX
+// rotary at position `pos` when `rope`; the result lands in vec[0..hd), LDS private to the wavefront.
+// NV = 1 serves hd <= 256 with half the registers.
+template <int NV> struct HeadVec { float4 x[NV]; };
+template <int NV>
+__device__ __forceinline__ HeadVec<NV> lg_head_load(const float *src, int hd) {
+    const int lane = threadIdx.x & 63;
+    HeadVec<NV> h;
     #pragma unroll
-    for (int v = 0; v < 2; ++v) {
+    for (int v = 0; v < NV; ++v) {
         const int e0 = 256 * v + 4 * lane;
-        if (e0 < hd) { xv[v] = *(const float4 *)(src + e0); if (w) wv[v] = *(const float4 *)(w + e0); }
+        h.x[v] = e0 < hd ? *(const float4 *)(src + e0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
-    if (4 * lane < hd) ss0 = lg_sumsq4(xv[0], 0.0f);
-    if (256 + 4 * lane < hd) ss1 = lg_sumsq4(xv[1], 0.0f);
-    const float ss = lg_wave_sum64(ss0) + lg_wave_sum64(ss1);
-    const float sc = 1.0f / sqrtf(ss / (float)hd + a.eps);
+    return h;
+}
+// The rotary table entries of the pairs this lane rotates (p = lane + 64 i), loaded ahead of their use.
+template <int NV> struct RopeVals { float tab[2 * NV], ff[2 * NV]; };
+template <int NV>
+__device__ __forceinline__ RopeVals<NV> lg_rope_load(const float *rope_tab, const float *rope_ff, int hd) {
+    const int lane = threadIdx.x & 63, half = hd >> 1;
+    RopeVals<NV> r;
     #pragma unroll
-    for (int v = 0; v < 2; ++v) {
+    for (int i = 0; i < 2 * NV; ++i) {
+        const int p = lane + 64 * i;
+        r.tab[i] = p < half ? rope_tab[p] : 0.0f;
+        r.ff[i] = (p < half && rope_ff) ? rope_ff[p] : 1.0f;
+    }
+    return r;
+}
+__device__ __forceinline__ void lg_wave_lds_sync() {
+    // LDS serves one wavefront's accesses in order; the fences keep the compiler from reordering around it
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+template <int NV>
+__device__ __forceinline__ void lg_head_finish(HeadVec<NV> h, HeadVec<NV> w, bool weighted, int hd, float eps, bool rope, int pos,
+                                               const RopeVals<NV> &rv, float *vec) {
+    const int lane = threadIdx.x & 63, half = hd >> 1;
+    float ss0 = 0.0f, ss1 = 0.0f;                            // lanes l and l+64 of the 256-lane sum order
+    if (4 * lane < hd) ss0 = lg_sumsq4(h.x[0], 0.0f);
+    if (NV > 1 && 256 + 4 * lane < hd) ss1 = lg_sumsq4(h.x[NV - 1], 0.0f);
+    const float ss = NV > 1 ? lg_wave_sum64(ss0) + lg_wave_sum64(ss1) : lg_wave_sum64(ss0);    // ss1 == 0 adds nothing
+    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+    #pragma unroll
+    for (int v = 0; v < NV; ++v) {
         const int e0 = 256 * v + 4 * lane;
         if (e0 >= hd) continue;
+        const float4 x = h.x[v], ww = w.x[v];
         float4 r;
-        if (w) r = make_float4(xv[v].x * sc * wv[v].x, xv[v].y * sc * wv[v].y, xv[v].z * sc * wv[v].z, xv[v].w * sc * wv[v].w);
-        else r = make_float4(xv[v].x * sc, xv[v].y * sc, xv[v].z * sc, xv[v].w * sc);
-        vec[e0] = r.x; vec[e0 + 1] = r.y; vec[e0 + 2] = r.z; vec[e0 + 3] = r.w;
+        if (weighted) r = make_float4(x.x * sc * ww.x, x.y * sc * ww.y, x.z * sc * ww.z, x.w * sc * ww.w);
+        else r = make_float4(x.x * sc, x.y * sc, x.z * sc, x.w * sc);
+        *(float4 *)(vec + e0) = r;
     }
-    __syncthreads();
-    if (!isv) {
-        for (int p = lane; p < half; p += 64) {
-            const float ang = (float)pos * a.rope_tab[p] / (a.rope_ff ? a.rope_ff[p] : 1.0f);
+    lg_wave_lds_sync();
+    if (rope) {
+        #pragma unroll
+        for (int i = 0; i < 2 * NV; ++i) {
+            const int p = lane + 64 * i;
+            if (p >= half) continue;
+            const float ang = (float)pos * rv.tab[i] / rv.ff[i];
             float sn, cs;
             lg_sincosf(ang, &sn, &cs);
             const float x0 = vec[p], x1 = vec[p + half];
             vec[p] = x0 * cs - x1 * sn;
             vec[p + half] = x0 * sn + x1 * cs;
         }
-        __syncthreads();
+        lg_wave_lds_sync();
     }
+}
+
+__global__ __launch_bounds__(64) void lg_k_qkv_post(QkvPostArgs a, const StepCtl *ctl) {
+    __shared__ __align__(16) float vec[512];
+    const int lane = threadIdx.x, job = blockIdx.x, j = blockIdx.y, hd = a.hd;
+    const int pos = ctl->pos + j;
+    const bool isq = job < a.H, isv = job >= a.H + a.nkv;
+    const int head = isq ? job : (job - a.H) % a.nkv;
+    const float *src = a.qkv + (size_t)j * a.ld + (isq ? (size_t)head * hd : (size_t)(isv ? a.v_off : a.k_off) + (size_t)head * hd);
+    const float *w = isq ? a.q_norm : (isv ? nullptr : a.k_norm);
+    const HeadVec<2> h = lg_head_load<2>(src, hd);
+    const HeadVec<2> wv = w ? lg_head_load<2>(w, hd) : h;
+    const RopeVals<2> rv = lg_rope_load<2>(a.rope_tab, a.rope_ff, hd);
+    lg_head_finish<2>(h, wv, w != nullptr, hd, a.eps, !isv, pos, rv, vec);
     if (isq) {
         float *dst = a.q_rot + (size_t)j * a.H * hd + (size_t)head * hd;
         for (int e = lane; e < hd; e += 64) dst[e] = vec[e];
@@ -918,6 +963,12 @@ struct AttnArgs {
     float *pm, *pl, *pacc;   // partials: [M*H][tiles_max], [M*H][tiles_max][hd]
     int tiles_max;
     int pos_off;             // added to the step position: -1 for a draft head, whose query at pos sees keys < pos
+    // lg_k_attn<true> only: the raw q/k/v projections of the block and what lg_k_qkv_post would apply to them
+    const float *qkv;        // [M][ld]: q at 0, k at k_off, v at v_off
+    int ld, k_off, v_off;
+    const float *q_norm, *k_norm, *rope_tab, *rope_ff;
+    uint16_t *kcw, *vcw;     // this layer's own cache, to receive the block's rows (nullptr: it reads another layer's)
+    float eps;
     __device__ __forceinline__ uint4 kc4(size_t off) const { return *(const uint4 *)(kc + off); }
     __device__ __forceinline__ uint4 vc4(size_t off) const { return *(const uint4 *)(vc + off); }
 };
@@ -929,7 +980,16 @@ __device__ __forceinline__ int lg_win_start(int pos, int window) {
 // One workgroup per (tile, kv head, draft row): the G = H/nkv query heads of the kv head's group.
 // The score of (query g, key slot) is split over two lanes of the same wavefront (lane and lane^32):
 // each runs two of the four partial chains, and the halves meet as (a0+a1)+(a2+a3).
-__global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
+//
+// FQ: the block's raw projections are normed and rotated here instead of by lg_k_qkv_post (one launch less per
+// layer; blocks of up to LG_HIP_MAX_ROWS_DEV rows; pos_off == 0 unless the layer owns no cache).  Every workgroup prepares its own row's G
+// queries (wavefront g = head g).  The block's own K/V rows are not in the cache yet: a workgroup whose tile
+// holds some of them builds the ones its row may see straight into the LDS tile (wavefronts 0,2: K rows,
+// 1,3: V rows), and the workgroups of the last row, which see all of them, also store them to the cache.
+// The ring has at least LG_WIDE_ROWS spare rows, so no row another workgroup still reads is overwritten.
+#define LG_ATTN_JOBS ((LG_HIP_MAX_ROWS_DEV + 1) / 2)       // K (or V) rows one wavefront may have to build
+template <bool FQ, int NV>
+__global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int hd = a.hd, G = a.H / a.nkv;
     const int kst = hd + 8;                                   // padded V tile row (halves): 16-byte rows, read along the row
@@ -941,28 +1001,76 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
     uint16_t *kt = (uint16_t *)(qs + (size_t)G * hd);         // [32][ksk]
     uint16_t *vt = kt + 32 * kst;                             // [32][kst]
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
+    float *hv = (float *)(smem + (((size_t)((unsigned char *)(es + G * 32 + G) - smem) + 15) & ~(size_t)15));   // FQ: [4 wavefronts][hd] staging
     const int kvh = blockIdx.y, j = blockIdx.z;
     const int pos0 = ctl->pos + a.pos_off, pj = pos0 + j;
     const int startj = lg_win_start(pj, a.window);
     const int n = (lg_win_start(pos0, a.window) >> 5) + blockIdx.x;
     if (n < (startj >> 5) || n > (pj >> 5)) return;           // tile outside this row's keys
     const int t0 = n << 5;
+    // FQ: positions tnew..pj of this tile are rows of the block itself (none when the layer reads another's cache)
+    const int tnew = (FQ && a.kcw) ? ctl->pos : 0x7FFFFFFF;
     {   // stage q (G heads of this row) and the tile's K/V rows; loads are issued in groups ahead of
         // the LDS stores (named temporaries + scheduling barrier, see lg_copy_batched)
-        const float *qrow = a.q + (size_t)j * a.H * hd + (size_t)kvh * G * hd;
-        lg_copy_batched<float4>((const float4 *)qrow, (float4 *)qs, G * (hd >> 2));
+        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        HeadVec<NV> hq[2], hj[LG_ATTN_JOBS], wq, wk;
+        RopeVals<NV> rv;
+        int njobs = 0, r0 = 0;
+        if (FQ) {                                             // all loads of this wavefront's vectors first
+            const float *qrow = a.qkv + (size_t)j * a.ld + (size_t)kvh * G * hd;
+            #pragma unroll
+            for (int u = 0; u < 2; ++u) if (wv + 4 * u < G) hq[u] = lg_head_load<NV>(qrow + (size_t)(wv + 4 * u) * hd, hd);
+            wq = lg_head_load<NV>(a.q_norm, hd);
+            rv = lg_rope_load<NV>(a.rope_tab, a.rope_ff, hd);
+            const int rlo = t0 > tnew ? t0 - tnew : 0, rhi = (t0 + 31 < pj ? t0 + 31 : pj) - tnew;   // block rows in this tile
+            if (pj >= tnew && rhi >= rlo) { njobs = rhi - rlo + 1; r0 = rlo; }
+            wk = ((wv & 1) || njobs == 0) ? wq : lg_head_load<NV>(a.k_norm, hd);   // no K rows to build: k_norm may not exist
+            #pragma unroll
+            for (int u = 0; u < LG_ATTN_JOBS; ++u) {
+                const int rr = (wv >> 1) + 2 * u;
+                if (rr < njobs) hj[u] = lg_head_load<NV>(a.qkv + (size_t)(r0 + rr) * a.ld + ((wv & 1) ? a.v_off : a.k_off) + (size_t)kvh * hd, hd);
+            }
+        } else {
+            const float *qrow = a.q + (size_t)j * a.H * hd + (size_t)kvh * G * hd;
+            lg_copy_batched<float4>((const float4 *)qrow, (float4 *)qs, G * (hd >> 2));
+        }
+        auto prepare = [&]() {                                // queries, then this wavefront's K or V rows of the block
+            #pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (wv + 4 * u < G)
+                    lg_head_finish<NV>(hq[u], wq, true, hd, a.eps, true, ctl->pos + j, rv, qs + (size_t)(wv + 4 * u) * hd);
+            float *vec = hv + (size_t)wv * hd;
+            #pragma unroll
+            for (int u = 0; u < LG_ATTN_JOBS; ++u) {
+                const int rr = (wv >> 1) + 2 * u;
+                if (rr >= njobs) continue;
+                const bool isv = wv & 1;
+                const int t = tnew + r0 + rr, sl = t - t0;
+                lg_head_finish<NV>(hj[u], wk, !isv, hd, a.eps, !isv, t, rv, vec);
+                uint16_t *row = isv ? vt + sl * kst : kt + sl * ksk;
+                uint16_t *crow = (j == (int)gridDim.z - 1) ? (isv ? a.vcw : a.kcw) + (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd : nullptr;
+                for (int e = 2 * lane; e < hd; e += 128) {
+                    const uint32_t two = (uint32_t)lg_f2h(vec[e]) | ((uint32_t)lg_f2h(vec[e + 1]) << 16);
+                    *(uint32_t *)(row + e) = two;
+                    if (crow) *(uint32_t *)(crow + e) = two;
+                }
+                lg_wave_lds_sync();                           // vec is reused by the next row
+            }
+        };
         const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
         for (int i0 = threadIdx.x; i0 < nk8; i0 += 4 * LG_WG) {
             // element u of the batch: LDS offset (halves) in `lo`, cache offset in `go`, validity in `ok`
-            auto place = [&](int u, int &lo, int &lk, size_t &go, bool &ok) {
+            auto place = [&](int u, int &lo, int &lk, size_t &go, bool &ok, bool &own) {
                 const int idx = min(i0 + u * LG_WG, nk8 - 1);
                 const int sl = idx / per_row, e0 = (idx - sl * per_row) << 3, t = t0 + sl;
                 ok = t >= startj && t <= pj;
+                own = ok && t >= tnew;                        // a row of the block: built by `prepare`, not read from the cache
+                ok = ok && !own;
                 lo = sl * kst + e0; lk = sl * ksk + e0;
                 go = (size_t)((ok ? t : pj) % a.seq) * a.kv_dim + (size_t)kvh * hd + e0;
             };
-            int l0, l1, l2, l3, m0, m1, m2, m3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3;
-            place(0, l0, m0, g0, ok0); place(1, l1, m1, g1, ok1); place(2, l2, m2, g2, ok2); place(3, l3, m3, g3, ok3);
+            int l0, l1, l2, l3, m0, m1, m2, m3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3, ow0, ow1, ow2, ow3;
+            place(0, l0, m0, g0, ok0, ow0); place(1, l1, m1, g1, ok1, ow1); place(2, l2, m2, g2, ok2, ow2); place(3, l3, m3, g3, ok3, ow3);
             const uint4 k0 = a.kc4(g0), k1 = a.kc4(g1), k2 = a.kc4(g2), k3 = a.kc4(g3);
             const uint4 v0 = a.vc4(g0), v1 = a.vc4(g1), v2 = a.vc4(g2), v3 = a.vc4(g3);
             __builtin_amdgcn_sched_barrier(0);
@@ -974,11 +1082,12 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn(AttnArgs a, const StepCtl *ct
                 uint32_t *d = (uint32_t *)(kt + lk);
                 d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
             };
-            putk(m0, keep(k0, ok0));  *(uint4 *)(vt + l0) = keep(v0, ok0);
-            putk(m1, keep(k1, ok1));  *(uint4 *)(vt + l1) = keep(v1, ok1);
-            putk(m2, keep(k2, ok2));  *(uint4 *)(vt + l2) = keep(v2, ok2);
-            putk(m3, keep(k3, ok3));  *(uint4 *)(vt + l3) = keep(v3, ok3);
+            if (!ow0) { putk(m0, keep(k0, ok0));  *(uint4 *)(vt + l0) = keep(v0, ok0); }
+            if (!ow1) { putk(m1, keep(k1, ok1));  *(uint4 *)(vt + l1) = keep(v1, ok1); }
+            if (!ow2) { putk(m2, keep(k2, ok2));  *(uint4 *)(vt + l2) = keep(v2, ok2); }
+            if (!ow3) { putk(m3, keep(k3, ok3));  *(uint4 *)(vt + l3) = keep(v3, ok3); }
         }
+        if (FQ) prepare();                                    // its loads were issued ahead of the tile's
     }
     __syncthreads();
     {   // scores, tile max, exp, tile sum
