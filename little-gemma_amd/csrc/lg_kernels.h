@@ -1002,10 +1002,11 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
     uint16_t *vt = kt + 32 * kst;                             // [32][kst]
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
     float *hv = (float *)(smem + (((size_t)((unsigned char *)(es + G * 32 + G) - smem) + 15) & ~(size_t)15));   // FQ: [4 wavefronts][hd] staging
-    const int kvh = blockIdx.y, j = blockIdx.z;
+    // dispatched last rows and last tiles first: those hold the block's own K/V rows, the longest workgroups
+    const int kvh = blockIdx.y, j = (int)gridDim.z - 1 - (int)blockIdx.z, bx = (int)gridDim.x - 1 - (int)blockIdx.x;
     const int pos0 = ctl->pos + a.pos_off, pj = pos0 + j;
     const int startj = lg_win_start(pj, a.window);
-    const int n = (lg_win_start(pos0, a.window) >> 5) + blockIdx.x;
+    const int n = (lg_win_start(pos0, a.window) >> 5) + bx;
     if (n < (startj >> 5) || n > (pj >> 5)) return;           // tile outside this row's keys
     const int t0 = n << 5;
     // FQ: positions tnew..pj of this tile are rows of the block itself (none when the layer reads another's cache)
@@ -1048,7 +1049,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
                 const int t = tnew + r0 + rr, sl = t - t0;
                 lg_head_finish<NV>(hj[u], wk, !isv, hd, a.eps, !isv, t, rv, vec);
                 uint16_t *row = isv ? vt + sl * kst : kt + sl * ksk;
-                uint16_t *crow = (j == (int)gridDim.z - 1) ? (isv ? a.vcw : a.kcw) + (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd : nullptr;
+                uint16_t *crow = (blockIdx.z == 0) ? (isv ? a.vcw : a.kcw) + (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd : nullptr;
                 for (int e = 2 * lane; e < hd; e += 128) {
                     const uint32_t two = (uint32_t)lg_f2h(vec[e]) | ((uint32_t)lg_f2h(vec[e + 1]) << 16);
                     *(uint32_t *)(row + e) = two;
@@ -1114,7 +1115,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
             if (hf == 0) {
                 es[g * 32 + sl] = e;
                 if (sl == 0) {
-                    const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
+                    const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + bx;
                     a.pm[pi] = mx; a.pl[pi] = l;
                 }
             }
@@ -1147,7 +1148,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
                 }
             }
         }
-        const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + blockIdx.x;
+        const size_t pi = ((size_t)j * a.H + kvh * G + g) * a.tiles_max + bx;
         *(float4 *)(a.pacc + pi * hd + d0) = acc;
     }
 }
