@@ -891,40 +891,58 @@ __device__ __forceinline__ void lg_wave_lds_sync() {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+// rmsnorm of a head vector (weighted by `w`, or plain) in the 256-lane sum order; the result stays in registers.
 template <int NV>
-__device__ __forceinline__ void lg_head_finish(HeadVec<NV> h, HeadVec<NV> w, bool weighted, int hd, float eps, bool rope, int pos,
-                                               const RopeVals<NV> &rv, float *vec) {
-    const int lane = threadIdx.x & 63, half = hd >> 1;
+__device__ __forceinline__ HeadVec<NV> lg_head_norm(HeadVec<NV> h, HeadVec<NV> w, bool weighted, int hd, float eps) {
+    const int lane = threadIdx.x & 63;
     float ss0 = 0.0f, ss1 = 0.0f;                            // lanes l and l+64 of the 256-lane sum order
     if (4 * lane < hd) ss0 = lg_sumsq4(h.x[0], 0.0f);
     if (NV > 1 && 256 + 4 * lane < hd) ss1 = lg_sumsq4(h.x[NV - 1], 0.0f);
     const float ss = NV > 1 ? lg_wave_sum64(ss0) + lg_wave_sum64(ss1) : lg_wave_sum64(ss0);    // ss1 == 0 adds nothing
     const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+    HeadVec<NV> r;
     #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int e0 = 256 * v + 4 * lane;
-        if (e0 >= hd) continue;
         const float4 x = h.x[v], ww = w.x[v];
-        float4 r;
-        if (weighted) r = make_float4(x.x * sc * ww.x, x.y * sc * ww.y, x.z * sc * ww.z, x.w * sc * ww.w);
-        else r = make_float4(x.x * sc, x.y * sc, x.z * sc, x.w * sc);
-        *(float4 *)(vec + e0) = r;
+        if (weighted) r.x[v] = make_float4(x.x * sc * ww.x, x.y * sc * ww.y, x.z * sc * ww.z, x.w * sc * ww.w);
+        else r.x[v] = make_float4(x.x * sc, x.y * sc, x.z * sc, x.w * sc);
     }
+    return r;
+}
+template <int NV>
+__device__ __forceinline__ void lg_head_store(const HeadVec<NV> &r, int hd, float *vec) {
+    const int lane = threadIdx.x & 63;
+    #pragma unroll
+    for (int v = 0; v < NV; ++v) if (256 * v + 4 * lane < hd) *(float4 *)(vec + 256 * v + 4 * lane) = r.x[v];
     lg_wave_lds_sync();
-    if (rope) {
-        #pragma unroll
-        for (int i = 0; i < 2 * NV; ++i) {
-            const int p = lane + 64 * i;
-            if (p >= half) continue;
-            const float ang = (float)pos * rv.tab[i] / rv.ff[i];
-            float sn, cs;
-            lg_sincosf(ang, &sn, &cs);
-            const float x0 = vec[p], x1 = vec[p + half];
-            vec[p] = x0 * cs - x1 * sn;
-            vec[p + half] = x0 * sn + x1 * cs;
-        }
-        lg_wave_lds_sync();
+}
+// NeoX rotary at position `pos` of a normed vector: it goes through vec[0..hd) (LDS private to the wavefront,
+// the pairs (p, p + hd/2) sit in different lanes), and out(p, lo, hi) receives the rotated pair p = lane + 64 i.
+template <int NV, typename Out>
+__device__ __forceinline__ void lg_head_rope(const HeadVec<NV> &r, int hd, int pos, const RopeVals<NV> &rv, float *vec, Out out) {
+    const int lane = threadIdx.x & 63, half = hd >> 1;
+    lg_head_store<NV>(r, hd, vec);
+    #pragma unroll
+    for (int i = 0; i < 2 * NV; ++i) {
+        const int p = lane + 64 * i;
+        if (p >= half) continue;
+        const float ang = (float)pos * rv.tab[i] / rv.ff[i];
+        float sn, cs;
+        lg_sincosf(ang, &sn, &cs);
+        const float x0 = vec[p], x1 = vec[p + half];
+        out(p, x0 * cs - x1 * sn, x0 * sn + x1 * cs);
     }
+}
+// Both steps with the result left in vec.
+template <int NV>
+__device__ __forceinline__ void lg_head_finish(HeadVec<NV> h, HeadVec<NV> w, bool weighted, int hd, float eps, bool rope, int pos,
+                                               const RopeVals<NV> &rv, float *vec) {
+    const HeadVec<NV> r = lg_head_norm<NV>(h, w, weighted, hd, eps);
+    if (rope) {
+        const int half = hd >> 1;
+        lg_head_rope<NV>(r, hd, pos, rv, vec, [&](int p, float lo, float hi) { vec[p] = lo; vec[p + half] = hi; });
+        lg_wave_lds_sync();
+    } else lg_head_store<NV>(r, hd, vec);
 }
 
 __global__ __launch_bounds__(64) void lg_k_qkv_post(QkvPostArgs a, const StepCtl *ctl) {
@@ -1039,23 +1057,36 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
             #pragma unroll
             for (int u = 0; u < 2; ++u)
                 if (wv + 4 * u < G)
-                    lg_head_finish<NV>(hq[u], wq, true, hd, a.eps, true, ctl->pos + j, rv, qs + (size_t)(wv + 4 * u) * hd);
+                    lg_head_finish<NV>(hq[u], wq, true, hd, a.eps, true, ctl->pos + j, rv, qs + (size_t)(wv + 4 * u) * hd);   // in place
             float *vec = hv + (size_t)wv * hd;
+            const int half = hd >> 1;
             #pragma unroll
             for (int u = 0; u < LG_ATTN_JOBS; ++u) {
                 const int rr = (wv >> 1) + 2 * u;
                 if (rr >= njobs) continue;
                 const bool isv = wv & 1;
                 const int t = tnew + r0 + rr, sl = t - t0;
-                lg_head_finish<NV>(hj[u], wk, !isv, hd, a.eps, !isv, t, rv, vec);
-                uint16_t *row = isv ? vt + sl * kst : kt + sl * ksk;
-                uint16_t *crow = (blockIdx.z == 0) ? (isv ? a.vcw : a.kcw) + (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd : nullptr;
-                for (int e = 2 * lane; e < hd; e += 128) {
-                    const uint32_t two = (uint32_t)lg_f2h(vec[e]) | ((uint32_t)lg_f2h(vec[e + 1]) << 16);
-                    *(uint32_t *)(row + e) = two;
-                    if (crow) *(uint32_t *)(crow + e) = two;
+                const HeadVec<NV> r = lg_head_norm<NV>(hj[u], wk, !isv, hd, a.eps);
+                const size_t coff = (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd;
+                const bool wr_cache = blockIdx.z == 0;       // the last row's workgroups see every row of the block
+                if (isv) {                                    // V: no rotary, straight from the registers
+                    #pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        const int e0 = 256 * v + 4 * lane;
+                        if (e0 >= hd) continue;
+                        const uint2 h4 = make_uint2((uint32_t)lg_f2h(r.x[v].x) | ((uint32_t)lg_f2h(r.x[v].y) << 16),
+                                                    (uint32_t)lg_f2h(r.x[v].z) | ((uint32_t)lg_f2h(r.x[v].w) << 16));
+                        *(uint2 *)(vt + sl * kst + e0) = h4;
+                        if (wr_cache) *(uint2 *)(a.vcw + coff + e0) = h4;
+                    }
+                } else {
+                    uint16_t *row = kt + sl * ksk, *crow = a.kcw + coff;
+                    lg_head_rope<NV>(r, hd, t, rv, vec, [&](int p, float lo, float hi) {
+                        const uint16_t hl = lg_f2h(lo), hh = lg_f2h(hi);
+                        row[p] = hl; row[p + half] = hh;
+                        if (wr_cache) { crow[p] = hl; crow[p + half] = hh; }
+                    });
                 }
-                lg_wave_lds_sync();                           // vec is reused by the next row
             }
         };
         const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
