@@ -175,6 +175,10 @@ __device__ __forceinline__ float lg_h2f(uint16_t h) {
     return __half2float(__ushort_as_half(h));
 }
 __device__ __forceinline__ uint16_t lg_f2h(float f) {
+    // The value converted is the binary32 one.  Without the barrier the compiler folds a multiply that produced f
+    // into one multiply-and-convert instruction (v_fma_mixlo_f16), which rounds once instead of twice and differs
+    // from the stored-then-converted value in rare tie cases.
+    asm("" : "+v"(f));
     return __half_as_ushort(__float2half_rn(f));
 }
 

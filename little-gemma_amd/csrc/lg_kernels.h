@@ -1002,10 +1002,10 @@ __device__ __forceinline__ int lg_win_start(int pos, int window) {
 // FQ: the block's raw projections are normed and rotated here instead of by lg_k_qkv_post (one launch less per
 // layer; blocks of up to LG_HIP_MAX_ROWS_DEV rows; pos_off == 0 unless the layer owns no cache).  Every workgroup prepares its own row's G
 // queries (wavefront g = head g).  The block's own K/V rows are not in the cache yet: a workgroup whose tile
-// holds some of them builds the ones its row may see straight into the LDS tile (wavefronts 0,2: K rows,
-// 1,3: V rows), and the workgroups of the last row, which see all of them, also store them to the cache.
+// holds some of them builds the ones its row may see straight into the LDS tile (K row r by wavefront r % 4,
+// V row r by wavefront 3 - r % 4), and the workgroups of the last row, which see all of them, also store them to the cache.
 // The ring has at least LG_WIDE_ROWS spare rows, so no row another workgroup still reads is overwritten.
-#define LG_ATTN_JOBS ((LG_HIP_MAX_ROWS_DEV + 1) / 2)       // K (or V) rows one wavefront may have to build
+#define LG_ATTN_JOBS (2 * ((LG_HIP_MAX_ROWS_DEV + 3) / 4)) // K and V rows one wavefront may have to build
 template <bool FQ, int NV>
 __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -1043,11 +1043,12 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
             rv = lg_rope_load<NV>(a.rope_tab, a.rope_ff, hd);
             const int rlo = t0 > tnew ? t0 - tnew : 0, rhi = (t0 + 31 < pj ? t0 + 31 : pj) - tnew;   // block rows in this tile
             if (pj >= tnew && rhi >= rlo) { njobs = rhi - rlo + 1; r0 = rlo; }
-            wk = ((wv & 1) || njobs == 0) ? wq : lg_head_load<NV>(a.k_norm, hd);   // no K rows to build: k_norm may not exist
+            wk = njobs == 0 ? wq : lg_head_load<NV>(a.k_norm, hd);   // no K rows to build: k_norm may not exist
             #pragma unroll
-            for (int u = 0; u < LG_ATTN_JOBS; ++u) {
-                const int rr = (wv >> 1) + 2 * u;
-                if (rr < njobs) hj[u] = lg_head_load<NV>(a.qkv + (size_t)(r0 + rr) * a.ld + ((wv & 1) ? a.v_off : a.k_off) + (size_t)kvh * hd, hd);
+            for (int u = 0; u < LG_ATTN_JOBS; ++u) {          // slots 0,1: K rows wv, wv+4; slots 2,3: V rows 3-wv, 7-wv
+                const bool isv = u >= LG_ATTN_JOBS / 2;
+                const int rr = (isv ? 3 - wv : wv) + 4 * (u & 1);
+                if (rr < njobs) hj[u] = lg_head_load<NV>(a.qkv + (size_t)(r0 + rr) * a.ld + (isv ? a.v_off : a.k_off) + (size_t)kvh * hd, hd);
             }
         } else {
             const float *qrow = a.q + (size_t)j * a.H * hd + (size_t)kvh * G * hd;
@@ -1062,9 +1063,9 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
             const int half = hd >> 1;
             #pragma unroll
             for (int u = 0; u < LG_ATTN_JOBS; ++u) {
-                const int rr = (wv >> 1) + 2 * u;
+                const bool isv = u >= LG_ATTN_JOBS / 2;
+                const int rr = (isv ? 3 - wv : wv) + 4 * (u & 1);
                 if (rr >= njobs) continue;
-                const bool isv = wv & 1;
                 const int t = tnew + r0 + rr, sl = t - t0;
                 const HeadVec<NV> r = lg_head_norm<NV>(hj[u], wk, !isv, hd, a.eps);
                 const size_t coff = (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * hd;
