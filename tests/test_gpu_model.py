@@ -59,13 +59,16 @@ def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, gol
         gpu.close(); o.close()
 
 
-@pytest.mark.parametrize("name,rows", [("tiny", 2), ("tiny", 4), ("tiny", 5), ("tiny_full", 3), ("tiny_full", 4), ("tiny_full", 6),
-                                       ("tiny_full", 7), ("tiny_full", 8)])
-def test_verify_equals_decode_and_accept_counts(lg, ob, gpu_required, model_path, name, rows):
+@pytest.mark.parametrize("name,rows,over", [("tiny", 2, {}), ("tiny", 4, {}), ("tiny", 5, {}), ("tiny_full", 3, {}), ("tiny_full", 4, {}),
+                                            ("tiny_full", 6, {}), ("tiny_full", 7, {}), ("tiny_full", 8, {}),
+                                            ("tiny", 5, {"head_dim_full": 512}), ("tiny_full", 8, {"head_dim_full": 256})])
+def test_verify_equals_decode_and_accept_counts(lg, ob, gpu_required, model_path, name, rows, over):
     """Row j of a verify block is bit-identical to a plain decode at pos+j (the reference's central
     invariant, src/cuda/model-cuda.cuh:520-526), and with drafts whose first mismatch is planted the
-    accepted count is known in advance (the acceptance tripwire, bench/mtp-accept.ps1:1-4)."""
-    path, spec = model_path(name)
+    accepted count is known in advance (the acceptance tripwire, bench/mtp-accept.ps1:1-4).  The last two
+    cases widen the heads of the global layers (512: two registers per lane in the attention kernel's
+    query/key preparation; 256: one, full)."""
+    path, spec = model_path(name, **over)
     V = spec["n_vocab"]
     rng = np.random.default_rng(rows)
     prompt = rng.integers(0, V, 150).astype(np.int32)           # beyond the 128-wide window: the ring has wrapped
