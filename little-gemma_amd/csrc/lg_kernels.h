@@ -1213,25 +1213,34 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
         __syncthreads();
         for (int n = threadIdx.x; n < cn; n += LG_WG) wts[n] = lg_expf(a.pm[base + c0 + n] - mx);
         __syncthreads();
-        for (int n0 = 0; n0 < cn; n0 += 8) {                   // 8 independent loads in flight, fma in tile order
-            float pl8[8], pa8[2][8];
+        // a batch of partials is one memory round trip (they were written by other CUs a moment ago), so the
+        // batch is made large enough to hold all the tiles of a sliding layer; fma in tile order
+        constexpr int U = 24;
+        for (int n0 = 0; n0 < cn; n0 += U) {
+            float plu[U], pau[U], pbu[U];                     // sums, dims 0..255, dims 256..511 (hd = 512 only)
+            const bool wide = hd > LG_WG;
             #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int n = n0 + u < cn ? n0 + u : cn - 1;
-                pl8[u] = a.pl[base + c0 + n];
+                plu[u] = a.pl[base + c0 + n];
+                pau[u] = (int)threadIdx.x < hd ? a.pacc[(base + c0 + n) * hd + threadIdx.x] : 0.0f;
+            }
+            if (wide) {
                 #pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2) {
-                    const int d = h2 * LG_WG + threadIdx.x;
-                    pa8[h2][u] = d < hd ? a.pacc[(base + c0 + n) * hd + d] : 0.0f;
+                for (int u = 0; u < U; ++u) {
+                    const int n = n0 + u < cn ? n0 + u : cn - 1;
+                    pbu[u] = a.pacc[(base + c0 + n) * hd + LG_WG + threadIdx.x];
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);                // every load of the batch issued before the first fma waits
             #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (n0 + u >= cn) break;
-                const float wn = wts[n0 + u];
-                L = lg_fmaf(pl8[u], wn, L);
-                o[0] = lg_fmaf(pa8[0][u], wn, o[0]);
-                o[1] = lg_fmaf(pa8[1][u], wn, o[1]);
+            for (int u = 0; u < U; ++u) {
+                if (n0 + u < cn) {                            // (a guard, not a break: the arrays stay in registers)
+                    const float wn = wts[n0 + u];
+                    L = lg_fmaf(plu[u], wn, L);
+                    o[0] = lg_fmaf(pau[u], wn, o[0]);
+                    if (wide) o[1] = lg_fmaf(pbu[u], wn, o[1]);
+                }
             }
         }
     }
