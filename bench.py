@@ -217,6 +217,17 @@ def main():
                 "bytes_per_launch": dom["bytes"] / max(dom["launches"], 1), "ms_per_launch": dom["ms"] / max(dom["launches"], 1),
                 "launches_per_step": dom["launches"]}
     step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9
+    # matrix-core utilisation of the verify step's one MFMA GEMM (gate/up for blocks of 4..8 rows): the weights of a
+    # launch (bytes / 0.5625 elements) times the block's rows are the useful MACs, the 8 row slots of the tiles the
+    # issued ones.  It is a bandwidth-bound kernel: the figure says how far the matrix cores are from mattering.
+    mfma = None
+    gu = next((c for c in prof if c["name"] == "gate_up_geglu" and c["launches"] > 0), None)
+    if gu and 4 <= a.rows <= 8:
+        w_elems = gu["bytes"] / gu["launches"] / (18.0 / 32.0)
+        sec = gu["ms"] / gu["launches"] * 1e-3
+        mfma = {"kernel": "gate_up_geglu (v_mfma_i32_32x32x32_i8, activations as the 8-row operand)",
+                "useful_int8_TOPs": 2.0 * w_elems * a.rows / sec / 1e12, "issued_int8_TOPs": 2.0 * w_elems * 8 / sec / 1e12,
+                "mfma_peak_TOPs": 5000.0, "mfma_utilisation": 2.0 * w_elems * a.rows / sec / 5.0e15}
     line = {
         "metric": ("verified tok/s (E4B-shape q4_0, block-4, ctx 2048) + achieved HBM GB/s vs peak" if a.workload == "e4b" else
                    f"verified tok/s ({a.workload} shape q4_0, {a.rows} rows, ctx {ctx}) + achieved HBM GB/s vs peak"),
@@ -228,6 +239,7 @@ def main():
         "roofline": roofline,
         "step_hbm": {"bytes_per_step": step_bytes, "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": step_gbs / HBM_PEAK_GBS},
+        "verify_mfma": mfma,
         "kernel_classes": [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in c.items()} for c in prof],
         "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
                    "wall_ms_per_step": 1e3 * wall / a.steps, "plain_decode_ms_per_token_host_sync": decode_ms},
