@@ -156,3 +156,14 @@ def test_model_init_reports_missing_tensors(lg, ob, tmp_path):
     assert H.lg_gw_commit(w) == 0 and H.lg_gw_close(w) == 0
     with pytest.raises(RuntimeError):
         ob.Oracle(p)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The verify step is not sharded: bench.py --gpus N with N > 1 exits with a message that says so
+    (before anything touches a device)."""
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr
+    assert r.stdout.strip() == ""
