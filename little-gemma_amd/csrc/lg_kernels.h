@@ -636,6 +636,7 @@ struct RowsPleGateArgs {
     float          eps;
 };
 #define LG_RPG_WG 1024
+#define LG_RPG_SPLIT 7                                       // draft rows from which the gate matmul is split over two sets of wavefronts
 template <int M>
 __global__ __launch_bounds__(LG_RPG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -647,8 +648,11 @@ __global__ __launch_bounds__(LG_RPG_WG) void lg_k_rows_plegate(RowsPleGateArgs a
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
     const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + (wave & 3)) * nit * LG_TILE };
     const int row[1] = { 0 };
+    // the gate matmul: wavefronts 0..3 take one group of 8 gate rows each; from LG_RPG_SPLIT draft rows up, wavefronts 4..7 take
+    // the same groups for the second half of the draft rows (the registers of all M rows do not fit 128 per lane)
+    constexpr int MA = M >= LG_RPG_SPLIT ? (M + 1) / 2 : M, MB = M - MA;
     WChunk<1> first;
-    if (wave < 4) lg_mm_fetch<1>(first, wg, 0, nit, lane);
+    if (wave < (MB ? 8 : 4)) lg_mm_fetch<1>(first, wg, 0, nit, lane);
     for (int j = wave; j < M; j += LG_RPG_WG / 64)
         if (lane < 32) ipl[j][lane] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + lane];
     {
@@ -701,10 +705,16 @@ __global__ __launch_bounds__(LG_RPG_WG) void lg_k_rows_plegate(RowsPleGateArgs a
     }
     __syncthreads();
     if (wave < 4) {
-        float acc[1][M];
-        lg_mm_groups<M, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
+        float acc[1][MA];
+        lg_mm_groups<MA, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
         const int c = lane & 7, r = lane >> 3;
-        if (c < M) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<M>(acc[0], c)) * ipl[c][wave * 8 + r];
+        if (c < MA) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<MA>(acc[0], c)) * ipl[c][wave * 8 + r];
+    } else if (MB > 0 && wave < 8) {
+        constexpr int MBB = MB > 0 ? MB : 1;
+        float acc[1][MBB];
+        lg_mm_groups<MBB, 8, 1, false>(wg, first, nit, lq + (size_t)MA * E, lds + (size_t)MA * (E >> 5), E, acc, lane, nullptr, 0, row);
+        const int c = lane & 7, r = lane >> 3;
+        if (c < MBB) gbuf[MA + c][(wave & 3) * 8 + r] = lg_gelu(lg_pick<MBB>(acc[0], c)) * ipl[MA + c][(wave & 3) * 8 + r];
     }
     __syncthreads();
     for (int j = threadIdx.x >> 5; j < M; j += LG_RPG_WG / 32) {
