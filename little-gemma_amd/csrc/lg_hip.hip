@@ -780,7 +780,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             } else {
                 // the residual update after ffn_down and its q8 happen inside the gate kernel (no rows kernel here)
                 RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps };
-                LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32), dim3(LG_RPG_WG), lds_mm(M, E), r);
+                LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32, M), dim3(LG_WG), lds_mm(1, E), r);
                 cur ^= 1;
                 pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
             }

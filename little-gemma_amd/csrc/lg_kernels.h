@@ -625,102 +625,69 @@ struct PleGateArgs {
 };
 // Verify blocks (wide blocks: lg_k_mm_plegate_wide): the row work that precedes the matmul is folded in,
 // i.e. the residual update x += rmsnorm(dout) * w_post and the q8 of the new x (what lg_k_rows does
-// between two other matmuls).  Each of the ple/32 workgroups repeats the update of all M rows: the matmul needs every row
-// whole, and a kernel boundary costs more than the repeated work.  1024 threads: four groups of 256, a
-// group takes rows g, g+4 with the lane assignment and summation order of lg_k_rows; the quantized rows
-// go straight to LDS, workgroup 0 also writes the new residual; wavefronts 0..3 then run the matmul.
+// between two other matmuls).  One workgroup per (block of 32 gate rows, draft row): it updates and quantizes
+// its one row (lane assignment and summation order of lg_k_rows; the quantized row goes straight to LDS, the
+// workgroups of gate block 0 also write the new residual), then its four wavefronts take 8 gate rows each
+// against that row.  The ple/32 workgroups of a draft row repeat its row work, which costs less than a kernel
+// boundary; splitting the draft rows over workgroups keeps what one CU has to pull in (row, previous output,
+// norm weights, 32 gate rows) near 76 KB at the E4B shape.
 struct RowsPleGateArgs {
     PleGateArgs    g;
     const float   *x, *dout, *w_post;   // [M][E] residual, [M][E] ffn_down output, [E]
     float         *x_out;               // [M][E]
     float          eps;
 };
-#define LG_RPG_WG 1024
-#define LG_RPG_SPLIT 7                                       // draft rows from which the gate matmul is split over two sets of wavefronts
 template <int M>
-__global__ __launch_bounds__(LG_RPG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
+__global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    int8_t *lq = (int8_t *)smem;
-    float2 *lds = (float2 *)(smem + (size_t)M * a.g.k);
-    __shared__ float gbuf[LG_HIP_MAX_ROWS_DEV][32];
-    __shared__ float ipl[LG_HIP_MAX_ROWS_DEV][32];
-    __shared__ float red[LG_HIP_MAX_ROWS_DEV][4];
+    int8_t *lq = (int8_t *)smem;                              // one row: [E] int8, then [E/32] {scale, sum}
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
-    const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + (wave & 3)) * nit * LG_TILE };
+    float2 *lds = (float2 *)(smem + (size_t)E);
+    __shared__ float gbuf[32], ipl[32], red[4];
+    const int j = blockIdx.y;
+    const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
     const int row[1] = { 0 };
-    // the gate matmul: wavefronts 0..3 take one group of 8 gate rows each; from LG_RPG_SPLIT draft rows up, wavefronts 4..7 take
-    // the same groups for the second half of the draft rows (the registers of all M rows do not fit 128 per lane)
-    constexpr int MA = M >= LG_RPG_SPLIT ? (M + 1) / 2 : M, MB = M - MA;
     WChunk<1> first;
-    if (wave < (MB ? 8 : 4)) lg_mm_fetch<1>(first, wg, 0, nit, lane);
-    for (int j = wave; j < M; j += LG_RPG_WG / 64)
-        if (lane < 32) ipl[j][lane] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + lane];
+    lg_mm_fetch<1>(first, wg, 0, nit, lane);
+    if (threadIdx.x < 32) ipl[threadIdx.x] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + threadIdx.x];
     {
-        constexpr int RJ = (M + 3) / 4;                       // rows per group
-        const int t = threadIdx.x & 255, grp = threadIdx.x >> 8, gw = wave & 3, nq = E >> 2;
-        float4 xv[RJ][LG_ROWV], dv[RJ][LG_ROWV], wp[LG_ROWV];
-        const float4 *wr = (const float4 *)a.w_post;
+        const int t = threadIdx.x, nq = E >> 2;
+        float4 xv[LG_ROWV], dv[LG_ROWV], wp[LG_ROWV];
+        const float4 *wr = (const float4 *)a.w_post, *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) wp[v] = wr[t + 256 * v];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; dv[v] = dr[t + 256 * v]; wp[v] = wr[t + 256 * v]; }
+        float ss = 0.0f;
         #pragma unroll
-        for (int r = 0; r < RJ; ++r) {
-            const int j = grp + 4 * r;
-            if (j >= M) break;                                // uniform per wavefront
-            const float4 *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
-            #pragma unroll
-            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[r][v] = xr[t + 256 * v]; dv[r][v] = dr[t + 256 * v]; }
-        }
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
+        ss = lg_block_sum256(ss, red);
+        const float sc = 1.0f / sqrtf(ss / (float)E + a.eps);
         #pragma unroll
-        for (int r = 0; r < RJ; ++r) {
-            const int j = grp + 4 * r;
-            if (j >= M) break;
-            float ss = 0.0f;
-            #pragma unroll
-            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[r][v], ss);
-            ss = lg_wave_sum64(ss);
-            if (lane == 0) red[j][gw] = ss;
-        }
-        __syncthreads();
-        #pragma unroll
-        for (int r = 0; r < RJ; ++r) {
-            const int j = grp + 4 * r;
-            if (j >= M) break;
-            const float ss = (red[j][0] + red[j][1]) + (red[j][2] + red[j][3]);
-            const float sc = 1.0f / sqrtf(ss / (float)E + a.eps);
-            #pragma unroll
-            for (int v = 0; v < LG_ROWV; ++v) {
-                if (t + 256 * v >= nq) break;                 // nq is a multiple of 64: whole wavefronts
-                const float4 w = wp[v], d = dv[r][v];
-                float4 x = xv[r][v];
+        for (int v = 0; v < LG_ROWV; ++v) {
+            if (t + 256 * v < nq) {                           // nq is a multiple of 64: whole wavefronts
+                const float4 w = wp[v], d = dv[v];
+                float4 x = xv[v];
                 x.x = x.x + d.x * sc * w.x;  x.y = x.y + d.y * sc * w.y;
                 x.z = x.z + d.z * sc * w.z;  x.w = x.w + d.w * sc * w.w;
                 if (blockIdx.x == 0) ((float4 *)(a.x_out + (size_t)j * E))[t + 256 * v] = x;
                 float dq; int sum;
                 const uint32_t packed = lg_quant4_8lanes(x, &dq, &sum);
                 const int quad = t + 256 * v;
-                *(uint32_t *)(lq + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
-                if ((t & 7) == 0) lds[lg_q8_ds_idx<M>(E, j, quad >> 3)] = make_float2(dq, __int_as_float(sum));
+                *(uint32_t *)(lq + lg_q8_off<1>(E, 0, quad >> 2, (quad & 3) * 4)) = packed;
+                if ((t & 7) == 0) lds[lg_q8_ds_idx<1>(E, 0, quad >> 3)] = make_float2(dq, __int_as_float(sum));
             }
         }
     }
     __syncthreads();
-    if (wave < 4) {
-        float acc[1][MA];
-        lg_mm_groups<MA, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
-        const int c = lane & 7, r = lane >> 3;
-        if (c < MA) gbuf[c][wave * 8 + r] = lg_gelu(lg_pick<MA>(acc[0], c)) * ipl[c][wave * 8 + r];
-    } else if (MB > 0 && wave < 8) {
-        constexpr int MBB = MB > 0 ? MB : 1;
-        float acc[1][MBB];
-        lg_mm_groups<MBB, 8, 1, false>(wg, first, nit, lq + (size_t)MA * E, lds + (size_t)MA * (E >> 5), E, acc, lane, nullptr, 0, row);
-        const int c = lane & 7, r = lane >> 3;
-        if (c < MBB) gbuf[MA + c][(wave & 3) * 8 + r] = lg_gelu(lg_pick<MBB>(acc[0], c)) * ipl[MA + c][(wave & 3) * 8 + r];
+    {
+        float acc[1][1];
+        lg_mm_groups<1, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
+        if ((lane & 7) == 0) gbuf[wave * 8 + (lane >> 3)] = lg_gelu(acc[0][0]) * ipl[wave * 8 + (lane >> 3)];
     }
     __syncthreads();
-    for (int j = threadIdx.x >> 5; j < M; j += LG_RPG_WG / 32) {
-        const int i = threadIdx.x & 31;
+    if (threadIdx.x < 32) {
+        const int i = threadIdx.x;
         float d; int sum;
-        const int q = lg_quant1_32lanes(gbuf[j][i], &d, &sum);
+        const int q = lg_quant1_32lanes(gbuf[i], &d, &sum);
         const ActLayout lay = lg_act_layout(ple);
         a.g.pq[(size_t)j * ple + lg_act_unit(lay, blockIdx.x * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
         if (i == 0) lg_q8_ds<M>(a.g.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, blockIdx.x)] = make_float2(d, __int_as_float(sum));
