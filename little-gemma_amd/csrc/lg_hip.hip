@@ -654,7 +654,10 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
         const int W = 4;
         LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
     } else {
-        const int W = ngroups >= 1024 ? 2 : 1;
+        // Two row groups per workgroup when there are very many groups, and for blocks of 4+ rows when one group per
+        // workgroup would leave some CUs with two of them: their activations (16 KB at M = 5) are then staged twice
+        // on the CUs that set the kernel's time.  (Short rows, k < 1024, have too little to stage for that to matter.)
+        const int W = (ngroups >= 1024 || (M >= 4 && a.k >= 1024 && ngroups > cu_count())) ? 2 : 1;
         LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
     }
     }
