@@ -244,6 +244,20 @@ def main():
         "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
                    "wall_ms_per_step": 1e3 * wall / a.steps, "plain_decode_ms_per_token_host_sync": decode_ms},
     }
+    # the same model and cache at the reference's "block-4" width (LG_MTP_N = 4: the chosen token + 3 drafts,
+    # include/model.h:179-183) when the headline ran at another width: same greedy chain, same draft model
+    if a.rows != 4 and a.workload == "e4b":
+        blocks4, expect4 = build_schedule(greedy, first_tok, 4, total, info["n_vocab"], a.seed)
+        lg.hiplib.hip_check(H.lg_hip_kv_restore_prefix(gpu.dkv, ctx), "kv_restore_prefix")
+        gpu.schedule(blocks4, ctx)
+        if a.warmup:
+            gpu.schedule_time(a.warmup)
+        ms4 = gpu.schedule_time(a.steps)
+        _, adv4, _ = gpu.schedule_wait()
+        line["block4"] = {"verify_rows": 4, "drafts": 3, "ms_per_step": ms4 / a.steps,
+                          "value": int(adv4[a.warmup:].sum()) / (ms4 * 1e-3), "unit": "verified tok/s",
+                          "mean_accepted_per_step": float(adv4[a.warmup:].mean()),
+                          "accept_counts_as_scheduled": bool(np.array_equal(adv4, expect4))}
     # the loop a draft head drives (the reference's run.c with -mtp): per step K = rows-1 chained drafts on the
     # device head (synthetic gemma4-assistant weights: its drafts are rarely accepted, the step cost does not
     # depend on that), then the verify step; host clock around synchronous calls, from the seeded cache
@@ -268,8 +282,18 @@ def main():
             if step >= 2:                                        # two untimed steps: graph captures of the head and its chain
                 t_draft += t1 - t0; t_verify += t2 - t1; emitted += adv
             pos += adv; tok = int(out[adv - 1])
+        # the same rounds kept on the device (lg_hip_mtp_rounds: one graph per round, the host waits once at the end)
+        lg.hiplib.hip_check(H.lg_hip_kv_restore_prefix(gpu.dkv, ctx), "kv_restore_prefix")
+        tok = gpu.forward_next(first_tok, ctx)
+        gpu.mtp_rounds(head, tok, ctx + 1, a.rows, 2)             # captures the round
+        lg.hiplib.hip_check(H.lg_hip_kv_restore_prefix(gpu.dkv, ctx), "kv_restore_prefix")
+        tok = gpu.forward_next(first_tok, ctx)
+        t0 = time.time()
+        _, _, radv, _ = gpu.mtp_rounds(head, tok, ctx + 1, a.rows, a.mtp_steps)
+        t_rounds = time.time() - t0
         gpu.mtp_close(head)
-        line["mtp_loop"] = {"steps": a.mtp_steps, "drafts_per_step": a.rows - 1,
+        line["mtp_loop"] = {"device_rounds_ms_per_step": 1e3 * t_rounds / a.mtp_steps,
+                            "device_rounds_tokens_per_step": float(radv.mean()),"steps": a.mtp_steps, "drafts_per_step": a.rows - 1,
                             "draft_ms_per_step": 1e3 * t_draft / a.mtp_steps, "verify_ms_per_step": 1e3 * t_verify / a.mtp_steps,
                             "ms_per_step": 1e3 * (t_draft + t_verify) / a.mtp_steps, "tokens_per_step": emitted / a.mtp_steps,
                             "head": "synthetic gemma4-assistant (4 blocks, 256 wide), host round trip per draft"}

@@ -117,6 +117,20 @@ int  lg_hip_draft_create(lg_hip_model *target, const struct lg_hip_config *cfg, 
  * head's post-norm hidden (inner width); lg_hip_get_logits(head, 0) its logits when stored. */
 int  lg_hip_draft_step(lg_hip_model *head, lg_hip_kv *target_kv, int token, int pos, int chain, int32_t *tok_out);
 
+/* Whole speculative rounds on the device: the loop the reference drives from the host with one
+ * synchronisation per draft and per verify step (mtp_step, src/run.c:54-71, inside the generation
+ * loop :737-768).  Round r verifies the block [chosen, d1..d(n_rows-1)] whose drafts the head
+ * proposes (d1 from the target's hidden state, the others chained), accepts, and takes the greedy
+ * successor of the last accepted row as the next round's chosen token; tokens and positions move
+ * between head and target in device memory, one captured graph per round, and the host waits
+ * once, after n_rounds.  token = the first chosen token, to sit at position pos; the target's
+ * hidden state must be that of the token before it (as for lg_hip_draft_step with chain = 0).
+ * Out: blocks[n_rounds][n_rows] as verified, out[n_rounds][n_rows] greedy successors,
+ * adv[n_rounds]; round r emitted blocks[r][0..adv[r]-1] and *final_pos = pos + sum(adv).
+ * The cache must hold pos + n_rows*n_rounds positions (every block may be accepted whole). */
+int  lg_hip_mtp_rounds(lg_hip_model *head, lg_hip_kv *target_kv, int token, int pos, int n_rows, int n_rounds,
+                       int32_t *blocks, int32_t *out, int32_t *adv, int32_t *final_pos);
+
 /* ---- device-resident stepping: the same step with no host round trip between steps.
  * A schedule is n_steps blocks of n_rows tokens built by the caller (drafts come from a draft
  * head or, in the benchmark, are prepared in advance); each step verifies block `step`, writes

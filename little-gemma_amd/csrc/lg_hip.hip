@@ -937,6 +937,78 @@ extern "C" int lg_hip_draft_step(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     return 0;
 }
 
+// One speculative round with no host involvement: K = rows-1 drafts (the first from the target's hidden state, the
+// others chained), the link kernels that move their tokens, and the verify step.
+static int enqueue_round(lg_hip_model *d, lg_hip_kv *kv, int rows, bool dry) {
+    lg_hip_model *t = d->target;
+    LinkArgs a{ d->ctl, t->ctl, d->sched, d->out, t->sched, t->out, t->adv, rows, 0 };
+    int rc = 0;
+    for (int j = 1; j <= rows && !rc; ++j) {
+        a.phase = j;
+        if (!dry) hipLaunchKernelGGL(lg_k_link, dim3(1), dim3(1), 0, t->stream, a);
+        if (j == rows) break;
+        d->draft_chain = j > 1;
+        rc = enqueue_step_rows(d, kv, 1, true, dry);
+        d->draft_chain = false;
+    }
+    if (!rc) rc = enqueue_step_rows(t, kv, rows, true, dry);
+    a.phase = 0;
+    if (!rc && !dry) hipLaunchKernelGGL(lg_k_link, dim3(1), dim3(1), 0, t->stream, a);
+    if (!rc && !dry) { hipError_t e = hipGetLastError(); if (e != hipSuccess) rc = fail(-100 - (int)e, "mtp_rounds: launch failed: %s", hipGetErrorString(e)); }
+    return rc;
+}
+
+extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int pos, int rows, int n_rounds,
+                                 int32_t *blocks, int32_t *out, int32_t *adv, int32_t *final_pos) {
+    if (!d || !kv || !d->target || !d->committed || kv->m != d->target) return fail(-1, "mtp_rounds: bad draft / cache pointer");
+    lg_hip_model *t = d->target;
+    if (!blocks || !out || !adv) return fail(-1, "mtp_rounds: null output");
+    if (rows < 2 || rows > t->max_rows) return fail(-2, "mtp_rounds: blocks of %d rows; the target was committed for 2..%d", rows, t->max_rows);
+    if (rows > 2 && !d->w_post) return fail(-4, "mtp_rounds: this head has no post-projection, drafts cannot chain");
+    if (n_rounds < 1 || n_rounds + 1 > t->sched_cap) return fail(-2, "mtp_rounds: %d rounds (limit %d)", n_rounds, t->sched_cap - 1);
+    if (token < 0 || token >= t->n_vocab) return fail(-2, "mtp_rounds: token id %d outside the target vocabulary of %d", token, t->n_vocab);
+    // every round may accept its whole block, so the last one may start rows*(n_rounds-1) positions on
+    if (pos < 1 || (long long)pos + (long long)rows * n_rounds > kv->max_seq) return fail(-2, "mtp_rounds: positions %d..%lld do not fit a cache of %d", pos, (long long)pos + (long long)rows * n_rounds - 1, kv->max_seq);
+    if (d->H > t->max_rows * t->H) return fail(-2, "mtp_rounds: %d draft heads do not fit the target's attention scratch", d->H);
+    HIP_TRY(hipSetDevice(t->device));
+    int rc;
+    int32_t tk = token;
+    if ((rc = load_block(t, &tk, 1, pos))) return rc;
+    if (!t->use_graph || t->prof.on || d->prof.on) {
+        for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
+    } else {
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "");
+        auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
+        if (it == d->graphs.end()) {
+            hipGraph_t graph = nullptr;
+            hipGraphExec_t exec = nullptr;
+            if ((rc = enqueue_round(d, kv, rows, true))) return rc;
+            HIP_TRY(hipStreamBeginCapture(t->stream, hipStreamCaptureModeThreadLocal));
+            rc = enqueue_round(d, kv, rows, false);
+            hipError_t e = hipStreamEndCapture(t->stream, &graph);
+            if (rc) { if (graph) (void)hipGraphDestroy(graph); return rc; }
+            if (e != hipSuccess) return fail(-100 - (int)e, "hipStreamEndCapture: %s", hipGetErrorString(e));
+            e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(graph);
+            if (e != hipSuccess) return fail(-100 - (int)e, "hipGraphInstantiate: %s", hipGetErrorString(e));
+            it = d->graphs.emplace(key, exec).first;
+        }
+        for (int r = 0; r < n_rounds; ++r) HIP_TRY(hipGraphLaunch(it->second, t->stream));
+    }
+    HIP_TRY(hipStreamSynchronize(t->stream));
+    StepCtl c;
+    HIP_TRY(hipMemcpy(&c, t->ctl, sizeof c, hipMemcpyDeviceToHost));
+    if (c.step != n_rounds) return fail(-9, "mtp_rounds: %d of %d rounds ran", c.step, n_rounds);
+    HIP_TRY(hipMemcpy(blocks, t->sched, (size_t)n_rounds * rows * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(out, t->out, (size_t)n_rounds * rows * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(adv, t->adv, (size_t)n_rounds * 4, hipMemcpyDeviceToHost));
+    if (final_pos) *final_pos = c.pos;
+    t->last_rows = rows; t->last_adv = adv[n_rounds - 1];
+    t->sched_steps = 0;
+    d->last_rows = 1; d->last_adv = 1;
+    return 0;
+}
+
 extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int pos0) {
     if (n <= 0) return 0;
     if (!m) return fail(-1, "prefill: null model");

@@ -816,6 +816,36 @@ __global__ __launch_bounds__(LG_WG) void lg_k_accept(AcceptArgs a, StepCtl *ctl)
 // Prefill blocks skip the head: only the position advances.
 __global__ void lg_k_advance(StepCtl *ctl, int rows) { ctl->pos += rows; ctl->step += 1; }
 
+// Glue of a speculative round that stays on the device (the host loop it replaces: src/run.c:54-71): one thread
+// moves tokens between the draft head's and the target's step state, so that K chained drafts and the verify
+// step that checks them run back to back with no copy to the host.
+//   phase 1..K   (before draft `phase`): the head's input token = the block's chosen token (phase 1) or the head's
+//                previous draft, which also becomes row phase-1 of the target's block; the head drafts for
+//                position pos + phase - 1 (src/run.c:60-66).
+//   phase K+1    (before the verify step): the last draft becomes row K of the block.
+//   phase 0      (after the verify step, whose accept kernel has advanced pos and step): the greedy successor of
+//                the last accepted row is the next block's chosen token (src/run.c:569-574).
+struct LinkArgs {
+    StepCtl *hctl; const StepCtl *tctl;
+    int32_t *hsched; const int32_t *hout;        // head: token slot 0, drafted token 0
+    int32_t *tsched; const int32_t *tout, *tadv; // target: [steps][M] blocks, [steps][M] successors, [steps]
+    int M, phase;
+};
+__global__ void lg_k_link(LinkArgs a) {
+    const int s = a.tctl->step;
+    if (a.phase == 0) {
+        a.tsched[(size_t)s * a.M] = a.tout[(size_t)(s - 1) * a.M + a.tadv[s - 1] - 1];
+        return;
+    }
+    const int tok = a.phase == 1 ? a.tsched[(size_t)s * a.M] : a.hout[0];
+    if (a.phase > 1) a.tsched[(size_t)s * a.M + a.phase - 1] = tok;
+    if (a.phase < a.M) {
+        a.hsched[0] = tok;
+        a.hctl->pos = a.tctl->pos + a.phase - 1;
+        a.hctl->step = 0;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // After the q/k/v projection: per-head rmsnorm (q and k weighted, v plain), rotary on q and k,
 // f16 round and store of the block's K/V rows into the ring (src/cuda/prefill-kernel.cuh:403-421).

@@ -69,6 +69,7 @@ def load_hip():
     L.lg_hip_get_hidden.argtypes = [C.c_void_p, f32p]
     L.lg_hip_get_logits.argtypes = [C.c_void_p, C.c_int, f32p]
     L.lg_hip_set_option.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+    L.lg_hip_mtp_rounds.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, i32p, i32p, i32p, C.POINTER(C.c_int32)]
     L.lg_hip_schedule_load.argtypes = [C.c_void_p, i32p, C.c_int, C.c_int, C.c_int]
     L.lg_hip_schedule_run.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
     L.lg_hip_schedule_wait.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32)]
@@ -128,6 +129,9 @@ def load_backend():
     B.lg_session_mtp_hidden.argtypes = [C.c_void_p, C.c_void_p, f32p]
     B.lg_session_mtp_logits.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
     B.lg_session_generate_mtp.argtypes = [C.c_void_p, C.c_void_p, i32p, C.c_int, C.c_int, C.c_int, i32p] + [C.POINTER(C.c_int)] * 3
+    B.lg_session_generate_mtp_rounds.argtypes = [C.c_void_p, C.c_void_p, i32p, C.c_int, C.c_int, C.c_int, C.c_int, i32p] + [C.POINTER(C.c_int)] * 3
+    B.lg_mtp_device.argtypes = [C.c_void_p, C.c_void_p]
+    B.lg_mtp_device.restype = C.c_void_p
     _backend = B
     return B
 
@@ -232,6 +236,28 @@ class HipBackend:
         if n < 0:
             raise HipError("generate_mtp rejected its arguments")
         return emitted[:n], steps.value, nd.value, na.value
+
+    def generate_mtp_rounds(self, t, prompt, n_gen, rows, batch):
+        """generate_mtp with `batch` speculative rounds at a time kept on the device."""
+        p = np.ascontiguousarray(prompt, np.int32)
+        emitted = np.zeros(n_gen, np.int32)
+        steps, nd, na = C.c_int(0), C.c_int(0), C.c_int(0)
+        n = self.B.lg_session_generate_mtp_rounds(self.s, t, p, len(p), n_gen, rows, batch, emitted, C.byref(steps), C.byref(nd), C.byref(na))
+        if n < 0:
+            raise HipError("generate_mtp_rounds rejected its arguments")
+        return emitted[:n], steps.value, nd.value, na.value
+
+    def mtp_rounds(self, t, token, pos, rows, n_rounds):
+        """n_rounds device-resident speculative rounds through the C ABI: (blocks, out, adv, final_pos)."""
+        d = self.B.lg_mtp_device(t, self.model)
+        if not d:
+            raise HipError("the draft head is not on the device")
+        blocks = np.zeros((n_rounds, rows), np.int32)
+        out = np.zeros((n_rounds, rows), np.int32)
+        adv = np.zeros(n_rounds, np.int32)
+        fp = C.c_int32(0)
+        hip_check(self.H.lg_hip_mtp_rounds(d, self.dkv, int(token), int(pos), rows, n_rounds, blocks, out, adv, C.byref(fp)), "mtp_rounds")
+        return blocks, out, adv, fp.value
 
     def last_hidden(self, n_embd):
         h = np.zeros(n_embd, np.float32)

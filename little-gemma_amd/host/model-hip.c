@@ -225,6 +225,18 @@ int  mtp_draft_device(struct mtp *t, const struct model *m, const struct kvcache
 int  mtp_draft_chain_device(struct mtp *t, const struct model *m, const struct kvcache *kv, int token, int pos) {
     return draft_on_device(t, m, kv, token, pos, 1);
 }
+/* n_rounds speculative rounds with no host round trip in between (draft, chained drafts, verify, accept, next
+ * chosen token: the body of the reference's loop, src/run.c:54-71 and :559-574, kept on the device).  Returns 0,
+ * or -1 when the head is unavailable or cannot chain: the caller then drives the loop itself. */
+int lg_model_mtp_rounds(struct mtp *t, const struct model *m, struct kvcache *kv, int token, int pos, int rows,
+                        int n_rounds, int *blocks, int *out, int *adv) {
+    lg_hip_model *d = draft_model(t, m);
+    if (!d) return -1;
+    int rc = lg_hip_mtp_rounds(d, device_kv(kv), token, pos, rows, n_rounds, blocks, out, adv, NULL);
+    if (rc == -4) return -1;                       /* no post-projection */
+    if (rc != 0) die("mtp_rounds");
+    return 0;
+}
 void mtp_free_device(struct mtp *t) {
     if (t->cuda && t->cuda != (void *)-1) lg_hip_model_destroy((lg_hip_model *)t->cuda);
     t->cuda = NULL;

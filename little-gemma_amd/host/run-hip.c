@@ -1,16 +1,19 @@
 /* run-hip — the reference CLI's generation path on the gfx950 backend, for token ids.
  *
  * The reference's `run` takes text (-p) and a draft-head file (-mtp) and prints text
- * (src/run.c:697-842).  Tokenizer, chat template and the draft head are outside this build, so
- * run-hip keeps the flags and the loop (prefill, first token, plain or block-LG_MTP_N speculative
- * greedy steps, the same stderr statistics lines) but takes the prompt as token ids and, for
- * -mtp, a file of draft token ids in place of a draft head:
+ * (src/run.c:697-842).  Tokenizer and chat template are outside this build, so run-hip keeps the
+ * flags and the loop (prefill, first token, plain or block-LG_MTP_N speculative greedy steps, the
+ * same stderr statistics lines) but takes the prompt as token ids and prints token ids:
  *
- *   run-hip -m model.gguf -p 12,7,99,4 [-n 256] [-mtp drafts.txt | -mtp self]
+ *   run-hip -m model.gguf -p 12,7,99,4 [-n 256] [-mtp assistant.gguf [-rounds R] | -mtp drafts.txt | -mtp self]
  *
- * -mtp self runs the plain path first and replays its own output as (perfect) drafts: the check
- * the reference does by hand — output with and without -mtp must be byte-identical
- * (docs/mtp.md:16-19) — as one command.  Output: generated token ids on stdout, one line.
+ * -mtp assistant.gguf drafts with a gemma4-assistant head on the device, like the reference's -mtp
+ * (src/run.c:719), after a plain greedy run of the same prompt: the two outputs must be
+ * byte-identical (docs/mtp.md:16-19) and the exit status says whether they were.  -rounds R keeps R
+ * speculative rounds on the device between host waits (default 8); 0 waits after every draft and
+ * every verify step, as the reference's loop does.  -mtp drafts.txt replays a file of draft token
+ * ids instead of a head; -mtp self replays the plain run's own output as (perfect) drafts.
+ * Output: generated token ids on stdout, one line.
  */
 #include <stdio.h>
 #include <stdlib.h>
@@ -41,15 +44,18 @@ static int parse_ids(const char *s, int *out, int cap) {
 
 int main(int argc, char **argv) {
     const char *model = NULL, *prompt = NULL, *mtp = NULL;
-    int n_gen = 256;
+    int n_gen = 256, rounds = 8;
     for (int i = 1; i < argc; i++) {
         if (!strcmp(argv[i], "-m") && i + 1 < argc) model = argv[++i];
         else if (!strcmp(argv[i], "-p") && i + 1 < argc) prompt = argv[++i];
         else if (!strcmp(argv[i], "-mtp") && i + 1 < argc) mtp = argv[++i];
         else if (!strcmp(argv[i], "-n") && i + 1 < argc) n_gen = atoi(argv[++i]);
+        else if (!strcmp(argv[i], "-rounds") && i + 1 < argc) rounds = atoi(argv[++i]);
     }
     if (!model || !prompt) {
-        printf("Usage: %s -m <model.gguf> -p <id,id,...> [-n N] [-mtp <assistant.gguf> | -mtp <draft-ids.txt> | -mtp self]\n"
+        printf("Usage: %s -m <model.gguf> -p <id,id,...> [-n N] [-mtp <assistant.gguf> [-rounds R] | -mtp <draft-ids.txt> | -mtp self]\n"
+               "       -rounds R: speculative rounds kept on the device between host waits (default 8; 0 = one wait per draft\n"
+               "       and per verify step, like the reference's loop)\n"
                "       (built with LG_MTP_N=%d: speculative blocks verify %d tokens per step)\n", argv[0], LG_MTP_N, LG_MTP_N);
         return 1;
     }
@@ -79,7 +85,8 @@ int main(int argc, char **argv) {
             if (lg_session_kv(s, max_seq) != 0) return 1;
             int steps = 0, nd = 0, na = 0;
             double t0 = now_sec();
-            int g = lg_session_generate_mtp(s, head, ids, n_prompt, n_gen, LG_MTP_N, emitted, &steps, &nd, &na);
+            int g = rounds > 0 ? lg_session_generate_mtp_rounds(s, head, ids, n_prompt, n_gen, LG_MTP_N, rounds, emitted, &steps, &nd, &na)
+                               : lg_session_generate_mtp(s, head, ids, n_prompt, n_gen, LG_MTP_N, emitted, &steps, &nd, &na);
             double dt = now_sec() - t0;
             for (int i = 0; i < g; i++) printf("%s%d", i ? "," : "", emitted[i]);
             printf("\n");

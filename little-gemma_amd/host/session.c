@@ -7,6 +7,8 @@
 
 int lg_model_forward_spec_n(struct model *m, struct kvcache *kv, const int *toks, int rows, int pos, int *out);
 lg_hip_model *lg_mtp_device(struct mtp *t, const struct model *m);
+int lg_model_mtp_rounds(struct mtp *t, const struct model *m, struct kvcache *kv, int token, int pos, int rows,
+                        int n_rounds, int *blocks, int *out, int *adv);
 
 struct lg_session { struct gguf_context *ctx; struct model m; struct kvcache kv; int has_kv; };
 
@@ -124,6 +126,64 @@ int lg_session_generate_mtp(struct lg_session *s, struct mtp *t, const int *prom
         for (int e = 1; e < adv && g < n_gen; e++) emitted[g++] = toks[e];
         best = out[adv - 1];
     }
+    if (steps) *steps = n_steps;
+    if (n_draft) *n_draft = nd;
+    if (n_accept) *n_accept = na;
+    return g;
+}
+
+/* The same loop with `batch` rounds at a time kept on the device (drafts, verify, accept and the next chosen token
+ * never visit the host inside a batch).  Tokens, step and draft counts are those of lg_session_generate_mtp as long
+ * as both run whole rounds; near the end of the cache, or when the head cannot chain, the rest of the generation
+ * goes through the host-driven rounds.  A batch may run rounds past n_gen: their tokens are dropped and not counted. */
+int lg_session_generate_mtp_rounds(struct lg_session *s, struct mtp *t, const int *prompt, int n_prompt, int n_gen, int rows,
+                                   int batch, int *emitted, int *steps, int *n_draft, int *n_accept) {
+    if (n_prompt < 1 || !s->has_kv || rows < 2 || rows > 16 || batch < 1) return -1;
+    int *blocks = malloc((size_t)batch * rows * 2 * sizeof(int)), *adv = malloc((size_t)batch * sizeof(int));
+    if (!blocks || !adv) { free(blocks); free(adv); return -1; }
+    int *out = blocks + (size_t)batch * rows;
+    model_prefill(&s->m, &s->kv, prompt, n_prompt - 1, 0);
+    int pos = n_prompt - 1, g = 0, n_steps = 0, nd = 0, na = 0, on_device = 1;
+    int best = model_forward_next(&s->m, &s->kv, prompt[n_prompt - 1], pos++);
+    while (g < n_gen) {
+        emitted[g++] = best;
+        if (g >= n_gen) break;
+        /* rounds still wanted: each emits at least one token; rounds that fit: each may take `rows` positions */
+        int want = n_gen - g < batch ? n_gen - g : batch;
+        int fit = (s->kv.max_seq - pos) / rows;
+        int n = want < fit ? want : fit;
+        if (on_device && n >= 1) {
+            if (lg_model_mtp_rounds(t, &s->m, &s->kv, best, pos, rows, n, blocks, out, adv) == 0) {
+                for (int r = 0; r < n && g < n_gen; r++) {
+                    const int *toks = blocks + (size_t)r * rows, a = adv[r];
+                    if (r > 0) emitted[g++] = toks[0];              /* the chosen token of a later round */
+                    if (g >= n_gen) break;                          /* that round's drafts are past the end: not counted */
+                    n_steps++; nd += rows - 1; na += a - 1;
+                    pos += a;
+                    for (int e = 1; e < a && g < n_gen; e++) emitted[g++] = toks[e];
+                    best = out[(size_t)r * rows + a - 1];
+                }
+                if (g >= n_gen) break;
+                continue;                                           /* `best` opens the next batch */
+            }
+            on_device = 0;                                          /* refused: host-driven rounds from here on */
+        }
+        if (pos + rows - 1 >= s->kv.max_seq) { best = model_forward_next(&s->m, &s->kv, best, pos++); n_steps++; continue; }
+        int toks[16], o[16];
+        toks[0] = best;
+        int d = mtp_draft(t, &s->m, &s->kv, best, pos);
+        toks[1] = d >= 0 ? d : best;
+        for (int j = 2; j < rows; j++) {
+            int dj = mtp_draft_chain(t, &s->m, &s->kv, toks[j - 1], pos + j - 1);
+            toks[j] = dj >= 0 ? dj : toks[j - 1];
+        }
+        int a = lg_model_forward_spec_n(&s->m, &s->kv, toks, rows, pos, o);
+        n_steps++; nd += rows - 1; na += a - 1;
+        pos += a;
+        for (int e = 1; e < a && g < n_gen; e++) emitted[g++] = toks[e];
+        best = o[a - 1];
+    }
+    free(blocks); free(adv);
     if (steps) *steps = n_steps;
     if (n_draft) *n_draft = nd;
     if (n_accept) *n_accept = na;

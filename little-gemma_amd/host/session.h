@@ -39,4 +39,8 @@ int  lg_session_mtp_hidden(struct lg_session *s, struct mtp *t, float *dst);
 int  lg_session_mtp_logits(struct lg_session *s, struct mtp *t, int on, float *dst);
 int  lg_session_generate_mtp(struct lg_session *s, struct mtp *t, const int *prompt, int n_prompt, int n_gen, int rows,
                              int *emitted, int *steps, int *n_draft, int *n_accept);
+/* The same generation with `batch` rounds at a time kept on the device (lg_hip_mtp_rounds): the host
+ * waits once per batch instead of once per draft and per verify step. */
+int  lg_session_generate_mtp_rounds(struct lg_session *s, struct mtp *t, const int *prompt, int n_prompt, int n_gen, int rows,
+                                    int batch, int *emitted, int *steps, int *n_draft, int *n_accept);
 #endif
