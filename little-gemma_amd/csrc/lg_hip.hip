@@ -1181,21 +1181,26 @@ static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, cons
     shim.stream = st;
     Launcher lx{ &shim, false };
     if (ddots) launch_mm<M, true>(lx, 0, a);
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
-    a.dots = nullptr;
-    launch_mm<M, false>(lx, 0, a);           // warm-up, also the result
-    HIP_TRY(hipEventRecord(e0, st));
-    for (int r = 0; r < repeats; ++r) launch_mm<M, false>(lx, 0, a);
-    if (lx.rc) return lx.rc;
-    HIP_TRY(hipEventRecord(e1, st));
-    HIP_TRY(hipStreamSynchronize(st));
-    HIP_TRY(hipGetLastError());
-    float t = 0;
-    if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
-    if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
-    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-    return 0;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        a.dots = nullptr;
+        launch_mm<M, false>(lx, 0, a);           // warm-up, also the result
+        HIP_TRY(hipEventRecord(e0, st));
+        for (int r = 0; r < repeats; ++r) launch_mm<M, false>(lx, 0, a);
+        if (lx.rc) return lx.rc;
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipGetLastError());
+        float t = 0;
+        if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+        if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+        return 0;
+    };
+    const int rc = body();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
 }
 
 extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *x, int rows, float *out, int32_t *dots,
