@@ -167,6 +167,18 @@ int  lg_hip_matmul_q4q8(const void *w, int k, int m, const float *x, int rows, f
 int  lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, int rows, int n_head,
                       int n_head_kv, int hd, int seq, int window, int pos, float *out,
                       int repeats, float *kernel_ms);
+/* The same attention for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  q, kc, vc and out
+ * are DEVICE pointers on the current device; the kernels' working memory (step state, tile partials)
+ * lives in a static device array of lg_hip_attention_noalloc_limit() bytes (8 MiB, held by every GPU
+ * the library runs on until the process ends), so the call allocates and frees nothing.  Shapes whose
+ * partials do not fit (rows * n_head * key tiles * hd * 4 bytes, plus small change) are refused with
+ * -2.  The launches go to `stream` (a hipStream_t, NULL = the default stream) and the call returns
+ * without waiting: out is valid once the stream has passed them.  All calls on one GPU share the
+ * array, so two calls that overlap in time on one GPU race; calls on one stream are ordered. */
+int    lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, const uint16_t *d_vc, int rows, int n_head,
+                                int n_head_kv, int hd, int seq, int window, int pos, float *d_out, void *stream);
+size_t lg_hip_attention_noalloc_limit(void);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
 int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 */

@@ -1263,26 +1263,37 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     return 0;
 }
 
+// the two launches of an isolated attention: tile partials, then the ordered merge
+template <int M>
+static void enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs &g, StepCtl *ctl, int tiles, size_t lds) {
+    hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
+    hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
+}
+
 template <int M>
 static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl, int tiles, int repeats, float *kernel_ms) {
     const size_t lds = attn_lds(a.H / a.nkv, a.hd, false);
     int rc = set_lds(lg_k_attn<false, 1>, lds);
     if (rc) return rc;
-    hipEvent_t e0, e1;
-    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
-    for (int r = 0; r < repeats + 1; ++r) {
-        if (r == 1) HIP_TRY(hipEventRecord(e0, st));
-        hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
-        hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
-    }
-    HIP_TRY(hipEventRecord(e1, st));
-    HIP_TRY(hipStreamSynchronize(st));
-    HIP_TRY(hipGetLastError());
-    float t = 0;
-    if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
-    if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
-    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-    return 0;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        for (int r = 0; r < repeats + 1; ++r) {
+            if (r == 1) HIP_TRY(hipEventRecord(e0, st));
+            enqueue_attention<M>(st, a, g, ctl, tiles, lds);
+        }
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipGetLastError());
+        float t = 0;
+        if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+        if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+        return 0;
+    };
+    rc = body();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    return rc;
 }
 
 extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, int rows, int n_head, int n_head_kv,
@@ -1324,5 +1335,73 @@ extern "C" int lg_hip_attention(const float *q, const uint16_t *kc, const uint16
     (void)hipStreamDestroy(st);
     if (rc) return rc;
     HIP_TRY(hipMemcpy(out, dxf, (size_t)rows * qd * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// ---- attention for callers that cannot allocate ---------------------------------------------------
+// lg_hip_attention with every buffer given by the caller as DEVICE memory, and the kernels' own working
+// memory (step state, tile partials, the q8 copy of the result that the merge kernel also writes) in a
+// static device array instead of hipMalloc'ed scratch: nothing is allocated or freed, the launches are
+// left on the caller's stream and the call returns without waiting.
+#define LG_NOALLOC_BYTES (8u << 20)
+#define LG_NOALLOC_DEVICES 16
+static __device__ __align__(256) unsigned char lg_noalloc_scratch[LG_NOALLOC_BYTES];
+// the array's device address, asked once per device (each device holds its own copy at its own address)
+static unsigned char *g_noalloc_ptr[LG_NOALLOC_DEVICES];
+
+__global__ void lg_k_set_ctl(StepCtl *ctl, int pos) { ctl->pos = pos; ctl->step = 0; ctl->err = 0; ctl->pad = 0; }
+
+static size_t up256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+extern "C" size_t lg_hip_attention_noalloc_limit(void) { return LG_NOALLOC_BYTES; }
+
+extern "C" int lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, const uint16_t *d_vc, int rows, int n_head,
+                                        int n_head_kv, int hd, int seq, int window, int pos, float *d_out, void *stream) {
+    if (!d_q || !d_kc || !d_vc || !d_out) return fail(-1, "attention_noalloc: null argument");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || n_head_kv < 1 || n_head % n_head_kv || n_head / n_head_kv > 8 ||
+        (hd != 64 && hd != 128 && hd != 256 && hd != 512) || pos < 0 || seq < 1)
+        return fail(-2, "attention_noalloc: unsupported shape");
+    if (window > 0 ? seq < window + rows - 1 && seq < pos + rows : seq < pos + rows)
+        return fail(-2, "attention_noalloc: a cache of %d rows cannot hold the keys of positions up to %d", seq, pos + rows - 1);
+    const int qd = n_head * hd;
+    const int start0 = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int tiles = ((pos + rows - 1) >> 5) - (start0 >> 5) + 1;
+    const size_t slots = (size_t)rows * n_head * tiles;
+    const size_t o_pm = 256, o_pl = o_pm + up256(slots * 4), o_pacc = o_pl + up256(slots * 4),
+                 o_xq = o_pacc + up256(slots * hd * 4), need = o_xq + up256((size_t)rows * qd * 5 / 4);
+    if (need > LG_NOALLOC_BYTES)
+        return fail(-2, "attention_noalloc: %d rows x %d heads x %d key tiles of %d need %zu bytes of working memory; the built-in array holds %u",
+                    rows, n_head, tiles, hd, need, LG_NOALLOC_BYTES);
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= LG_NOALLOC_DEVICES) return fail(-3, "attention_noalloc: device %d (0..%d are served)", dev, LG_NOALLOC_DEVICES - 1);
+    if (!g_noalloc_ptr[dev]) {
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(lg_noalloc_scratch)));
+        if (!p) return fail(-3, "attention_noalloc: the working array has no address on device %d", dev);
+        g_noalloc_ptr[dev] = (unsigned char *)p;
+    }
+    unsigned char *base = g_noalloc_ptr[dev];
+    StepCtl *ctl = (StepCtl *)base;
+    float *dpm = (float *)(base + o_pm), *dpl = (float *)(base + o_pl), *dpacc = (float *)(base + o_pacc);
+    int8_t *dxq = (int8_t *)(base + o_xq);
+    AttnArgs a{};
+    a.q = d_q; a.H = n_head; a.nkv = n_head_kv; a.hd = hd;
+    a.kc = d_kc; a.vc = d_vc; a.seq = seq; a.kv_dim = n_head_kv * hd; a.window = window;
+    a.pm = dpm; a.pl = dpl; a.pacc = dpacc; a.tiles_max = tiles;
+    MergeArgs g{ dpm, dpl, dpacc, tiles, n_head, hd, window, 0, dxq, d_out };
+    const size_t lds = attn_lds(n_head / n_head_kv, hd, false);
+    int rc = set_lds(lg_k_attn<false, 1>, lds);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    // every tile slot that the merge reads is written by the tile kernel of the same call, so nothing has to be
+    // cleared; only the step state is set, by a kernel (a caller may be capturing this stream)
+    hipLaunchKernelGGL(lg_k_set_ctl, dim3(1), dim3(1), 0, st, ctl, pos);
+    switch (rows) {
+#define CASE(M) case M: enqueue_attention<M>(st, a, g, ctl, tiles, lds); break;
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+    }
+    HIP_TRY(hipGetLastError());
     return 0;
 }
