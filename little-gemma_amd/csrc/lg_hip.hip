@@ -16,8 +16,10 @@
 #include "../../include/lg_hip.h"
 #include "lg_kernels.h"
 #include "lg_mfma.h"
+#include "lg_fused.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
+#define LG_FUSE_ROWS_MAX 2         // widest block whose q/k/v matmul does the preceding row work itself
 
 // ---- errors -----------------------------------------------------------------------------------
 static thread_local char g_err[512] = "";
@@ -154,7 +156,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -202,6 +204,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     m->head_dim.assign(c->head_dim, c->head_dim + c->n_layer);
     m->n_head_kv.assign(c->n_head_kv, c->n_head_kv + c->n_layer);
     if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
+    if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
     *out = m;
@@ -653,6 +656,14 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
     } else if (ngroups >= 4096) {
         const int W = 4;
         LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
+    } else if (M >= 4 && a.k >= 2048 && !DUMP) {
+        // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over four wavefronts
+        if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
+            static const int kp = getenv("LG_KP") ? atoi(getenv("LG_KP")) : 2;
+            const size_t l2 = ((lds + 15) & ~(size_t)15) + (size_t)2 * M * 64 * 4;
+            if (kp == 4) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, a);
+            else         LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
+        }
     } else {
         // Two row groups per workgroup when there are very many groups, and for blocks of 4+ rows when one group per
         // workgroup would leave some CUs with two of them: their activations (16 KB at M = 5) are then staged twice
@@ -703,9 +714,40 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os; s.dparts = pend_parts;
         s.w_pre = w_pre; s.h_out = h_out;
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
-        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M), dim3(LG_WG), 0, s, m->ctl);
+        // verify blocks: the tail of the row work (store, norm weight, q8) cut over one workgroup per float4 of a lane
+        const int slices = M <= LG_HIP_MAX_ROWS ? (E + 1023) / 1024 : 1;
+        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, s, m->ctl);
         if (s.x_out) cur ^= 1;
         have_x = true; pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+    };
+
+    // The same row work done by the workgroups of the matmul that consumes it (lg_fused.h): verify-width blocks
+    // whose residual is already in memory.  NV = float4 per lane of a row.
+    const int NVr = (E + 1023) / 1024;
+    // (blocks of one or two rows: wider ones pay more for the repeated row work than for the launch, see lg_fused.h)
+    auto can_fuse = [&]() { return M <= LG_FUSE_ROWS_MAX && have_x && m->fuse_rows && pend_parts == 1; };
+    auto row_work = [&](const float *w_pre) {
+        RowWork r{ m->x[cur], pend_dout, pend_w, pend_os, m->x[cur ^ 1], w_pre, E, m->eps };
+        return r;
+    };
+    auto row_work_done = [&]() {
+        if (pend_dout) cur ^= 1;
+        pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+    };
+    auto rows_mm = [&](const float *w_pre, const MmArgs &a, int cls) {      // rows(w_pre) then an 8-segment matmul of the result
+        if constexpr (M <= LG_FUSE_ROWS_MAX) {
+            constexpr int NW = 1;
+            RowsMmArgs f{ a, row_work(w_pre) };
+            const dim3 grid((a.m / 8 + NW - 1) / NW);
+            const size_t lds = lds_mm(M, a.k);
+            switch (NVr) {
+                case 1: LAUNCH(cls, (lg_k_rows_mm<M, 1, NW>), grid, dim3(LG_WG), lds, f); break;
+                case 2: LAUNCH(cls, (lg_k_rows_mm<M, 2, NW>), grid, dim3(LG_WG), lds, f); break;
+                case 3: LAUNCH(cls, (lg_k_rows_mm<M, 3, NW>), grid, dim3(LG_WG), lds, f); break;
+                default: LAUNCH(cls, (lg_k_rows_mm<M, 4, NW>), grid, dim3(LG_WG), lds, f); break;
+            }
+            row_work_done();
+        }
     };
 
     if (m->ple) {
@@ -719,11 +761,11 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
-        rows(y.attn_norm, nullptr);
         bool fused_post = false;
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
-            launch_mm<M, false>(lx, KC_QKV, a);
+            if (can_fuse()) rows_mm(y.attn_norm, a, KC_QKV);
+            else { rows(y.attn_norm, nullptr); launch_mm<M, false>(lx, KC_QKV, a); }
             // blocks of the model itself, up to LG_HIP_MAX_ROWS rows: the attention kernel does this part as well
             fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
             QkvPostArgs p{};
@@ -762,8 +804,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             // verify blocks: 1..3 rows through v_dot4 with scalar operands, 4..8 rows through the matrix cores
             // (its float work per tile does not grow with the row count); each has its own activation order
             constexpr bool mfma = M >= 4 && M <= LG_HIP_MAX_ROWS;
-            rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
+            rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
             else if constexpr (mfma)
@@ -832,7 +874,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -866,6 +908,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     if (!strcmp(name, "store_logits")) m->store_logits = value != 0;
     else if (!strcmp(name, "use_graph")) m->use_graph = value != 0;
     else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
+    else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
 }
@@ -977,7 +1020,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v");
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;

@@ -84,6 +84,9 @@ template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
     __shared__ float red[2][4];
     const int t = threadIdx.x, j = blockIdx.x;
+    // gridDim.y > 1: every workgroup of a row forms the row's sums, workgroup y stores and quantizes only the
+    // float4 t + 256*y of each lane (the tail of the kernel is the longest part of it and splits freely)
+    const int vs = gridDim.y > 1 ? (int)blockIdx.y : -1;
     const int E = s.E, nq = E >> 2;                          // float4 quads in a row; thread t owns quads t + 256*v
     float4 xv[LG_ROWV], dv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
     // issue every load up front: one memory round trip for the whole row
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
     if (s.x_out) {
         float4 *xo = (float4 *)(s.x_out + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) xo[t + 256 * v] = xv[v];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq && (vs < 0 || v == vs)) xo[t + 256 * v] = xv[v];
     }
     if (s.w_pre) {
         float ss = 0.0f;
@@ -156,13 +159,14 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
     if (s.h_out) {
         float4 *ho = (float4 *)(s.h_out + (size_t)j * E);
         #pragma unroll
-        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ho[t + 256 * v] = xv[v];
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq && (vs < 0 || v == vs)) ho[t + 256 * v] = xv[v];
     }
     float2 *dsb = lg_q8_ds<M>(s.q, E);
     #pragma unroll
     for (int v = 0; v < LG_ROWV; ++v) {
         // nq is a multiple of 64, so a whole wavefront is either inside the row or outside it
         if (t + 256 * v >= nq) break;
+        if (vs >= 0 && v != vs) continue;
         float d; int sum;
         const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
         const int quad = t + 256 * v;                        // 4 values = a quarter of a 16-byte unit
@@ -521,8 +525,15 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
     fetch(0);
     unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
     {
+        // four loads in flight per lane before the first store (left as a plain loop the copy is one round trip per 16 bytes)
         const uint4 *src = (const uint4 *)(a.q_in + (size_t)s * nit * (LG_MU_DWORDS * 4));
-        for (int i = lane; i < nit * (LG_MU_DWORDS / 4); i += 64) ((uint4 *)la)[i] = src[i];
+        const int nu = nit * (LG_MU_DWORDS / 4);
+        for (int i0 = lane; i0 < nu; i0 += 256) {
+            const int i1 = min(i0 + 64, nu - 1), i2 = min(i0 + 128, nu - 1), i3 = min(i0 + 192, nu - 1);
+            const uint4 t0 = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
+            __builtin_amdgcn_sched_barrier(0);
+            ((uint4 *)la)[i0] = t0; ((uint4 *)la)[i1] = t1; ((uint4 *)la)[i2] = t2; ((uint4 *)la)[i3] = t3;
+        }
         // read back below by other lanes of this wavefront only: LDS serves a wavefront's accesses in order,
         // the fences keep the compiler from moving the reads above the writes
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -646,9 +657,15 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     __shared__ float gbuf[32], ipl[32], red[4];
     const int j = blockIdx.y;
     const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
-    const int row[1] = { 0 };
-    WChunk<1> first;
-    lg_mm_fetch<1>(first, wg, 0, nit, lane);
+    // the whole row group (nit <= 16 tiles) is requested before anything else: with this few workgroups the kernel
+    // is a chain of memory round trips, and fetching the tiles two at a time adds one per pair
+    uint4 wq[LG_MAXV]; uint32_t wsc[LG_MAXV];
+    #pragma unroll
+    for (int u = 0; u < LG_MAXV; ++u) {
+        const int it = u < nit ? u : nit - 1;
+        wq[u] = *(const uint4 *)(wg[0] + (size_t)it * LG_TILE + lane * 16);
+        wsc[u] = *(const uint16_t *)(wg[0] + (size_t)it * LG_TILE + 1024 + lane * 2);
+    }
     if (threadIdx.x < 32) ipl[threadIdx.x] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + threadIdx.x];
     {
         const int t = threadIdx.x, nq = E >> 2;
@@ -679,9 +696,19 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     }
     __syncthreads();
     {
-        float acc[1][1];
-        lg_mm_groups<1, 8, 1, false>(wg, first, nit, lq, lds, E, acc, lane, nullptr, 0, row);
-        if ((lane & 7) == 0) gbuf[wave * 8 + (lane >> 3)] = lg_gelu(acc[0][0]) * ipl[wave * 8 + (lane >> 3)];
+        const int c = lane & 7;
+        float p = 0.0f;
+        #pragma unroll
+        for (int u = 0; u < LG_MAXV; ++u) {
+            if (u < nit) {                                    // (a guard, not a break: the arrays stay in registers)
+                const float2 ds = lds[u * 8 + c];
+                const int8_t *au = lq + (size_t)(u * 16 + c) * 16;
+                const int dot = lg_block_dot(wq[u], *(const int4 *)au, *(const int4 *)(au + 8 * 16), __float_as_int(ds.y));
+                p = lg_fmaf(ds.x * lg_h2f((uint16_t)wsc[u]), (float)dot, p);
+            }
+        }
+        p = lg_sum_seg<8>(p);
+        if (c == 0) gbuf[wave * 8 + (lane >> 3)] = lg_gelu(p) * ipl[wave * 8 + (lane >> 3)];
     }
     __syncthreads();
     if (threadIdx.x < 32) {
