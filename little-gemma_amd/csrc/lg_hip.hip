@@ -783,14 +783,17 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
+            // tiles a block of this layer can touch: a sliding layer needs only its window's, not the cache's
+            int tiles = kv->tiles_max;
+            if (window > 0 && M <= LG_HIP_MAX_ROWS) { const int t = (window + M - 1 + 31) / 32 + 1; if (t < tiles) tiles = t; }
             if (fused_post) {
                 a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
                 a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
                 a.kcw = y.owns ? kv->k[L] : nullptr; a.vcw = y.owns ? kv->v[L] : nullptr; a.eps = m->eps;
-                if (y.hd <= 256) LAUNCH(KC_ATTN, (lg_k_attn<true, 1>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
-                else             LAUNCH(KC_ATTN, (lg_k_attn<true, 2>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
+                if (y.hd <= 256) LAUNCH(KC_ATTN, (lg_k_attn<true, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
+                else             LAUNCH(KC_ATTN, (lg_k_attn<true, 2>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
             } else {
-                LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(kv->tiles_max, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
+                LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
             LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
