@@ -11,7 +11,7 @@ import subprocess
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-REF, I8, I8_LIBM = 0, 1, 2
+REF, I8, I8_LIBM, I8_F32 = 0, 1, 2, 3
 ORDER_SEG, ORDER_CUDA32 = 0, 1
 _lib = None
 _ref = {}

@@ -17,17 +17,20 @@
  *   lgo_forward(LGO_I8 / _LIBM)    built from the pinned primitives above.  The reference's CUDA int8 path
  *                                  it restates cannot run without an NVIDIA device: PARITY UNPINNED for the
  *                                  last bits of its float sums (this file fixes its own summation orders).
- *                                  The composition (quantization points, op order) is held by the measured
- *                                  gap to LGO_REF staying inside the q8 noise band and by spec == decode
- *                                  (tests/test_oracle_model.py).
+ *                                  The composition (quantization points, op order) is held by LGO_I8_F32: the
+ *                                  same function with the quantization switched off agrees with LGO_REF to
+ *                                  float reordering noise (1e-3 relative L2 of the logits at every step, every
+ *                                  argmax equal), and with it on stays inside the q8 noise band; plus
+ *                                  spec == decode (tests/test_oracle_model.py).
  *   lgo_mtp_draft(LGO_REF)         bit-identical tokens, hidden state and logits against the reference's host
  *                                  draft head (src/mtp.c, in oracle/_ref) and its committed fixtures
  *                                  (tests/test_oracle_draft.py), including that file's f16 subnormal reading
  *   lgo_mtp_draft(LGO_I8), lgo_mtp_post   same code path with q8 activations and this build's orders; the
  *                                  reference's device draft (f16 weights, CUDA sums) cannot run here: PARITY
  *                                  UNPINNED for its last bits and for the chained draft's post-projection,
- *                                  which has no CPU counterpart in the reference.  Held by the gap to LGO_REF
- *                                  and by the key-range test (a draft at pos reads positions < pos only).
+ *                                  which has no CPU counterpart in the reference.  Held by LGO_I8_F32 (same
+ *                                  code path, quantization off) agreeing with LGO_REF to 1e-3, by the q8 gap to
+ *                                  LGO_REF and by the key-range test (a draft at pos reads positions < pos only).
  *   lgo_forward_spec_all           equal to lgo_forward_spec in adv, out[0..adv-1] and hidden
  */
 #define _GNU_SOURCE
@@ -194,9 +197,15 @@ void lgo_rope(float *v, int d, int pos, const float *tab, const float *ff, int e
  *   score = (a0+a1)+(a2+a3) with a_c the fma chain over dims i%4==c; m = max; e = exp(s-m);
  *   l = adjacent tree over the 32 key slots; acc[d] = fma chain over slots ascending;
  *   tiles merged ascending with weights exp(m_tile - M), then out = acc / L. */
+static float kvf(const void *base, size_t i, int f16) {
+    return f16 ? lg_f16_to_f32(((const uint16_t *)base)[i]) : ((const float *)base)[i];
+}
+static void attention_tiled(float *out, const float *q, const void *kc, const void *vc, int f16,
+                            int hd, int kv_dim, int kvh, int seq, int start, int pos, int exact);
 void lgo_attention_f16(float *out, const float *q, const uint16_t *kc, const uint16_t *vc,
                        int hd, int kv_dim, int kvh, int seq, int start, int pos, int tiled, int exact) {
-    if (!tiled) {
+    if (tiled) { attention_tiled(out, q, kc, vc, 1, hd, kv_dim, kvh, seq, start, pos, exact); return; }
+    {
         int T = pos - start + 1;
         float *att = malloc((size_t)T * sizeof(float));
         float mx = -INFINITY;
@@ -217,8 +226,11 @@ void lgo_attention_f16(float *out, const float *q, const uint16_t *kc, const uin
             for (int i = 0; i < hd; i++) out[i] += a * lg_f16_to_f32(vr[i]);
         }
         free(att);
-        return;
     }
+}
+/* the tiled order over a cache of binary16 (f16 = 1) or float rows */
+static void attention_tiled(float *out, const float *q, const void *kc, const void *vc, int f16,
+                            int hd, int kv_dim, int kvh, int seq, int start, int pos, int exact) {
     const int TK = 32, n_lo = start / TK, n_hi = pos / TK, nt = n_hi - n_lo + 1;
     float *tm = malloc((size_t)nt * sizeof(float)), *tl = malloc((size_t)nt * sizeof(float));
     float *tacc = malloc((size_t)nt * hd * sizeof(float));
@@ -230,9 +242,9 @@ void lgo_attention_f16(float *out, const float *q, const uint16_t *kc, const uin
             int t = n * TK + sl;
             valid[sl] = t >= start && t <= pos;
             if (!valid[sl]) continue;
-            const uint16_t *kr = kc + (size_t)(t % seq) * kv_dim + (size_t)kvh * hd;
+            const size_t ko = (size_t)(t % seq) * kv_dim + (size_t)kvh * hd;
             float a[4] = { 0, 0, 0, 0 };
-            for (int i = 0; i < hd; i++) a[i & 3] = lg_fmaf(q[i], lg_f16_to_f32(kr[i]), a[i & 3]);
+            for (int i = 0; i < hd; i++) a[i & 3] = lg_fmaf(q[i], kvf(kc, ko + i, f16), a[i & 3]);
             sc[sl] = (a[0] + a[1]) + (a[2] + a[3]);
             if (sc[sl] > m) m = sc[sl];
         }
@@ -243,8 +255,8 @@ void lgo_attention_f16(float *out, const float *q, const uint16_t *kc, const uin
         for (int sl = 0; sl < TK; sl++) {
             if (!valid[sl]) continue;
             int t = n * TK + sl;
-            const uint16_t *vr = vc + (size_t)(t % seq) * kv_dim + (size_t)kvh * hd;
-            for (int i = 0; i < hd; i++) acc[i] = lg_fmaf(e[sl], lg_f16_to_f32(vr[i]), acc[i]);
+            const size_t vo = (size_t)(t % seq) * kv_dim + (size_t)kvh * hd;
+            for (int i = 0; i < hd; i++) acc[i] = lg_fmaf(e[sl], kvf(vc, vo + i, f16), acc[i]);
         }
         tm[n - n_lo] = m;
         tl[n - n_lo] = tree_sum(e, 32);
@@ -392,10 +404,11 @@ struct lgo_kv *lgo_kv_new(const struct lgo_model *o, int max_seq, int mode) {
         kv->kv_dim[L] = o->m.n_head_kv[L] * o->m.head_dim[L];
         if (L >= c->n_kv_start) continue;
         int seq = max_seq, local = o->m.is_local[L] && c->sliding_window > 0;
-        if (mode == LGO_REF) { if (local && c->sliding_window < max_seq) seq = c->sliding_window; }
+        const int reflike = mode == LGO_REF || mode == LGO_I8_F32;
+        if (reflike) { if (local && c->sliding_window < max_seq) seq = c->sliding_window; }
         else if (local) seq = lgo_ring_rows(c->sliding_window, max_seq);
         kv->seq[L] = seq;
-        kv->f16[L] = mode == LGO_REF ? !o->m.is_local[L] : 1;
+        kv->f16[L] = reflike ? !o->m.is_local[L] : 1;
         size_t n = (size_t)seq * kv->kv_dim[L];
         kv->k[L] = calloc(n, kv->f16[L] ? 2 : 4);
         kv->v[L] = calloc(n, kv->f16[L] ? 2 : 4);
@@ -560,14 +573,20 @@ static int forward_ref(struct lgo_model *o, struct lgo_kv *kv, int token, int po
  * loop, src/cuda/model-cuda.cuh:1121-1147 PLE build, src/cuda/mtp-kernel.cuh:21-30 head), one row.
  * Every matmul input is quantized once where the reference quantizes it; sums and elementary functions
  * follow this build's definitions when exact = 1. */
-struct qact { int8_t *q; float *d; };
-static void quant_into(struct qact *a, const float *x, int n) { lgo_quant_q8(x, n, a->q, a->d, NULL); }
+struct qact { int8_t *q; float *d; float *f; int noq; };
+/* noq: the quantization is switched off and the matmul takes the f32 vector itself (LGO_I8_F32): the same op
+ * sequence, norm / attention orders and elementary functions, without the int8 rounding of the activations */
+static void quant_into(struct qact *a, const float *x, int n) {
+    if (a->noq) memcpy(a->f, x, (size_t)n * 4);
+    else lgo_quant_q8(x, n, a->q, a->d, NULL);
+}
 static void mm(const struct gguf_tensor *w, int k, int mrows, const struct qact *a, float *out) {
     if (w->type != GGML_TYPE_Q4_0) { fprintf(stderr, "oracle: matmul weight %s is %s, only q4_0 is on the int8 path\n", w->name, ggml_type_name(w->type)); abort(); }
-    lgo_matmul_q4q8(w->data, k, mrows, a->q, a->d, 1, out, NULL, LGO_ORDER_SEG);
+    if (a->noq) lgo_matmul_f32(w->data, w->type, k, mrows, a->f, out);
+    else lgo_matmul_q4q8(w->data, k, mrows, a->q, a->d, 1, out, NULL, LGO_ORDER_SEG);
 }
 
-static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos, int exact, float *logits, float *hidden) {
+static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos, int exact, int noq, float *logits, float *hidden) {
     const struct model *m = &o->m;
     const struct config *c = &m->cfg;
     const int E = c->n_embd, H = c->n_head, ple = c->n_embd_per_layer;
@@ -580,7 +599,7 @@ static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos
     int widest = E;
     if (c->n_ff > widest) widest = c->n_ff;
     if (H * maxhd > widest) widest = H * maxhd;
-    struct qact a = { malloc((size_t)widest), malloc((size_t)widest / 32 * 4) };
+    struct qact a = { malloc((size_t)widest), malloc((size_t)widest / 32 * 4), malloc((size_t)widest * 4), noq };
     float *x = dequantize_row(o->token_embd, token, E);
     const float es = sqrtf((float)E);
     for (int i = 0; i < E; i++) x[i] = x[i] * es;
@@ -634,15 +653,20 @@ static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos
                 lgo_rope(kb + hh * hd, hd, pos, tab, ff, exact);
             }
             const int row = pos % kv->seq[L];
-            uint16_t *kr = (uint16_t *)kv->k[L] + (size_t)row * kd, *vr = (uint16_t *)kv->v[L] + (size_t)row * kd;
-            for (int i = 0; i < kd; i++) { kr[i] = lg_f32_to_f16(kb[i]); vr[i] = lg_f32_to_f16(vb[i]); }
+            if (kv->f16[L]) {
+                uint16_t *kr = (uint16_t *)kv->k[L] + (size_t)row * kd, *vr = (uint16_t *)kv->v[L] + (size_t)row * kd;
+                for (int i = 0; i < kd; i++) { kr[i] = lg_f32_to_f16(kb[i]); vr[i] = lg_f32_to_f16(vb[i]); }
+            } else {                                          /* LGO_I8_F32: the reference's f32 sliding rings */
+                memcpy((float *)kv->k[L] + (size_t)row * kd, kb, (size_t)kd * 4);
+                memcpy((float *)kv->v[L] + (size_t)row * kd, vb, (size_t)kd * 4);
+            }
         }
         const int start = (local && c->sliding_window > 0 && pos - c->sliding_window + 1 > 0) ? pos - c->sliding_window + 1 : 0;
         const int gqa = H / nkv;
         #pragma omp parallel for schedule(static)
         for (int hh = 0; hh < H; hh++)
-            lgo_attention_f16(xb + hh * hd, q + hh * hd, kv->k[src], kv->v[src], hd, kd, hh / gqa,
-                              kv->seq[src], start, pos, 1, exact);
+            attention_tiled(xb + hh * hd, q + hh * hd, kv->k[src], kv->v[src], kv->f16[src], hd, kd, hh / gqa,
+                            kv->seq[src], start, pos, exact);
         quant_into(&a, xb, qd);
         mm(y->wo, qd, E, &a, ob);
         lgo_rmsnorm(ob, ob, y->post_attn, E, eps, 1);
@@ -690,18 +714,18 @@ static int forward_i8(struct lgo_model *o, struct lgo_kv *kv, int token, int pos
         best = 0;
         for (int v = 1; v < c->n_vocab; v++) if (logits[v] > logits[best]) best = v;
     }
-    free(a.q); free(a.d);
+    free(a.q); free(a.d); free(a.f);
     free(x); free(h); free(q); free(kb); free(vb); free(xb); free(ob); free(g1); free(g2); free(pg); free(ipl);
     return best;
 }
 
 int lgo_forward(struct lgo_model *o, struct lgo_kv *kv, int token, int pos, int mode, float *logits, float *hidden) {
     if (token < 0 || token >= o->m.cfg.n_vocab || pos < 0 || pos >= kv->max_seq) return -1;
-    if ((mode == LGO_REF) != (kv->mode == LGO_REF)) { fprintf(stderr, "oracle: kv cache was created for another mode\n"); return -1; }
+    if ((mode == LGO_REF || mode == LGO_I8_F32) != (kv->mode == LGO_REF || kv->mode == LGO_I8_F32)) { fprintf(stderr, "oracle: kv cache was created for another mode\n"); return -1; }
     float *own = NULL;
     if (!logits) logits = own = malloc((size_t)o->m.cfg.n_vocab * 4);
     int best = mode == LGO_REF ? forward_ref(o, kv, token, pos, logits, hidden)
-                               : forward_i8(o, kv, token, pos, mode == LGO_I8, logits, hidden);
+                               : forward_i8(o, kv, token, pos, mode != LGO_I8_LIBM, mode == LGO_I8_F32, logits, hidden);
     free(own);
     return best;
 }
@@ -711,7 +735,7 @@ int lgo_forward(struct lgo_model *o, struct lgo_kv *kv, int token, int pos, int 
 void lgo_prefill(struct lgo_model *o, struct lgo_kv *kv, const int *tokens, int n, int pos0, int mode) {
     for (int i = 0; i < n; i++) {
         if (mode == LGO_REF) forward_ref(o, kv, tokens[i], pos0 + i, NULL, NULL);
-        else forward_i8(o, kv, tokens[i], pos0 + i, mode == LGO_I8, NULL, NULL);
+        else forward_i8(o, kv, tokens[i], pos0 + i, mode != LGO_I8_LIBM, mode == LGO_I8_F32, NULL, NULL);
     }
 }
 
@@ -826,15 +850,15 @@ int lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv
                   const float *h_prev, int mode, float *hidden_out, float *logits_out) {
     const struct model *m = &target->m;
     const struct config *c = &m->cfg;
-    const int ni = t->n_inner, nb = t->n_bb, ref = mode == LGO_REF, exact = mode == LGO_I8;
+    const int ni = t->n_inner, nb = t->n_bb, ref = mode == LGO_REF, exact = mode == LGO_I8 || mode == LGO_I8_F32, noq = mode == LGO_I8_F32;
     const float eps = t->eps;
     if (pos < 1 || token < 0 || token >= c->n_vocab) return -1;
-    if (ref != (kv->mode == LGO_REF)) { fprintf(stderr, "oracle: kv cache was created for another mode\n"); return -1; }
+    if ((ref || noq) != (kv->mode == LGO_REF || kv->mode == LGO_I8_F32)) { fprintf(stderr, "oracle: kv cache was created for another mode\n"); return -1; }
     int qmax = 0, widest = 2 * nb;
     for (int L = 0; L < t->n_layer; L++) if (t->n_head * t->l[L].hd > qmax) qmax = t->n_head * t->l[L].hd;
     if (qmax > widest) widest = qmax;
     if (t->n_ff > widest) widest = t->n_ff;
-    struct qact a = { malloc((size_t)widest), malloc((size_t)widest / 32 * 4) };
+    struct qact a = { malloc((size_t)widest), malloc((size_t)widest / 32 * 4), malloc((size_t)widest * 4), noq };
     float *cat = malloc((size_t)2 * nb * 4), *x = malloc((size_t)ni * 4), *h = malloc((size_t)ni * 4);
     float *q = malloc((size_t)qmax * 4), *xb = malloc((size_t)qmax * 4), *o = malloc((size_t)ni * 4);
     float *g1 = malloc((size_t)t->n_ff * 4), *g2 = malloc((size_t)t->n_ff * 4), *att = malloc((size_t)(pos + 1) * 4);
@@ -894,7 +918,7 @@ int lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv
             /* a query at pos-1 with the window one shorter: keys max(0, pos-window+1) .. pos-1 */
             #pragma omp parallel for schedule(static)
             for (int hh = 0; hh < t->n_head; hh++)
-                lgo_attention_f16(xb + hh * hd, q + hh * hd, kv->k[src], kv->v[src], hd, kd, hh / gqa, seq, start, pos - 1, 1, exact);
+                attention_tiled(xb + hh * hd, q + hh * hd, kv->k[src], kv->v[src], kv->f16[src], hd, kd, hh / gqa, seq, start, pos - 1, exact);
         }
         if (ref) lgo_matmul_f32(b->o->data, b->o->type, qd, ni, xb, o);
         else { quant_into(&a, xb, qd); mm(b->o, qd, ni, &a, o); }
@@ -926,7 +950,7 @@ int lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv
     int best = 0;
     for (int v = 1; v < t->n_vocab; v++) if (logits[v] > logits[best]) best = v;
     if (!logits_out) free(logits);
-    free(a.q); free(a.d); free(cat); free(x); free(h); free(q); free(xb); free(o); free(g1); free(g2); free(att); free(tab);
+    free(a.q); free(a.d); free(a.f); free(cat); free(x); free(h); free(q); free(xb); free(o); free(g1); free(g2); free(att); free(tab);
     return best;
 }
 
@@ -935,10 +959,10 @@ int lgo_mtp_draft(struct lgo_mtp *t, struct lgo_model *target, struct lgo_kv *kv
 int lgo_mtp_post(struct lgo_mtp *t, const float *hidden, int mode, float *h_out) {
     if (!t->post) return -1;
     if (mode == LGO_REF) { lgo_matmul_f32(t->post->data, t->post->type, t->n_inner, t->n_bb, hidden, h_out); return 0; }
-    struct qact a = { malloc((size_t)t->n_inner), malloc((size_t)t->n_inner / 32 * 4) };
+    struct qact a = { malloc((size_t)t->n_inner), malloc((size_t)t->n_inner / 32 * 4), malloc((size_t)t->n_inner * 4), mode == LGO_I8_F32 };
     quant_into(&a, hidden, t->n_inner);
     mm(t->post, t->n_inner, t->n_bb, &a, h_out);
-    free(a.q); free(a.d);
+    free(a.q); free(a.d); free(a.f);
     return 0;
 }
 

@@ -20,6 +20,9 @@ enum lgo_mode {
                          points, exact int32 block dots, f16 KV everywhere; float orders and elementary
                          functions as this build defines them (include/lg_math.h) */
     LGO_I8_LIBM = 2,  /* LGO_I8 with libm elementary functions: measures what lg_math.h changes */
+    LGO_I8_F32  = 3,  /* LGO_I8's op sequence, orders and functions with the activation quantization switched off
+                         (f32 activations into a serial f32 dot): differs from LGO_REF by float reordering and
+                         f16 sliding rings only, so the gap to LGO_REF pins the composition to reorder noise */
 };
 
 /* f32 combine order of the q4_0 x q8 matmul */

@@ -108,6 +108,36 @@ def test_int8_draft_stays_near_ref(lg, ob, model_path, model_dir, blocks, limit)
         d.close(); o.close()
 
 
+@pytest.mark.parametrize("blocks", [1, 4])
+def test_f32_variant_of_the_int8_draft_sequence_matches_ref_to_reorder_noise(lg, ob, model_path, model_dir, blocks):
+    """The int8-class draft with its quantization switched off (I8_F32: same op sequence, tile attention over
+    keys < pos, this build's norm orders and functions, f32 activations) must sit within float reordering
+    noise of the reference host draft: 1e-3 relative L2, same argmax.  The wide band of the q8 test above
+    cannot tell a misplaced op from int8 noise; this one can."""
+    path, spec = model_path("tiny_full")
+    head = head_path(lg, model_dir, "tiny_full", spec, n_layer=blocks, n_full=1)
+    o = ob.Oracle(path)
+    d = o.mtp_open(head)
+    try:
+        rng = np.random.default_rng(29)
+        prompt = rng.integers(0, spec["n_vocab"], 150).astype(np.int32)       # past the 128-row sliding window
+        kr, kf = o.kv_new(200, ob.REF), o.kv_new(200, ob.I8_F32)
+        o.prefill(kr, prompt[:-1], 0, ob.REF); o.prefill(kf, prompt[:-1], 0, ob.I8_F32)
+        tok, pos, gaps = int(prompt[-1]), 149, []
+        for _ in range(8):
+            best, _, hid = o.forward(kr, tok, pos, ob.REF, want_logits=True, want_hidden=True)
+            o.forward(kf, tok, pos, ob.I8_F32)
+            pos += 1
+            t0, _, l0 = d.draft(kr, best, pos, hid, ob.REF, want_logits=True)
+            t1, _, l1 = d.draft(kf, best, pos, hid, ob.I8_F32, want_logits=True)
+            gaps.append(np.linalg.norm(l1 - l0) / np.linalg.norm(l0))
+            assert t0 == t1
+            tok = best
+        assert max(gaps) <= 1e-3, gaps
+    finally:
+        d.close(); o.close()
+
+
 def test_draft_sees_only_positions_before_its_own(lg, ob, model_path, model_dir):
     """The cache row at the draft position (and later ones) must not influence the draft: overwrite
     them with noise and the int8-class draft is unchanged; change the row just before and it moves."""

@@ -95,6 +95,33 @@ def test_int8_class_stays_in_the_q8_noise_band_of_ref(ob, model_path, name):
         o.close()
 
 
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+def test_f32_variant_of_the_int8_sequence_matches_ref_to_reorder_noise(ob, model_path, name):
+    """I8_F32 runs forward_i8's exact op sequence (quantization points, PLE build, residual and scale placement,
+    tile attention, this build's norm orders and elementary functions) with the quantization switched off and
+    the reference's cache precision (f32 sliding rings).  What is left between it and REF is float reordering:
+    teacher-forced on the REF tokens the logits agree to 1e-3 relative L2 at every step and every argmax is the
+    same.  Any misplaced op in the shared sequence shows here at O(1e-1), far above the bar."""
+    path, spec = model_path(name)
+    o = ob.Oracle(path)
+    try:
+        rng = np.random.default_rng(spec["seed"] + 1)
+        prompt = rng.integers(0, spec["n_vocab"], 140).astype(np.int32)
+        kr, kf = o.kv_new(220, ob.REF), o.kv_new(220, ob.I8_F32)
+        o.prefill(kr, prompt[:-1], 0, ob.REF); o.prefill(kf, prompt[:-1], 0, ob.I8_F32)
+        tok, pos, gaps = int(prompt[-1]), 139, []
+        for _ in range(32):
+            b0, l0, h0 = o.forward(kr, tok, pos, ob.REF, want_hidden=True)
+            b1, l1, h1 = o.forward(kf, tok, pos, ob.I8_F32, want_hidden=True)
+            gaps.append(np.linalg.norm(l1 - l0) / np.linalg.norm(l0))
+            assert b0 == b1
+            assert np.linalg.norm(h1 - h0) <= 1e-3 * np.linalg.norm(h0)
+            tok, pos = b0, pos + 1
+        assert max(gaps) <= 1e-3, gaps
+    finally:
+        o.close()
+
+
 def test_int8_class_sequential_spec_equals_plain_decode(ob, model_path):
     """verify == decode by construction in the oracle: the block form is the same forwards."""
     path, spec = model_path("tiny")
