@@ -133,6 +133,7 @@ struct Profile {
 struct lg_hip_model {
     int device = 0;
     hipStream_t stream = nullptr;
+    bool owns_stream = true;           // false for a draft head: it runs on its target's stream and never destroys it
     // config
     int n_layer = 0, E = 0, H = 0, n_vocab = 0, window = 0, ple = 0, n_kv_start = 0, max_rows = 0;
     float eps = 0, base = 0, base_swa = 0, softcap = 0;
@@ -153,7 +154,7 @@ struct lg_hip_model {
     int *pidx = nullptr;
     StepCtl *ctl = nullptr;
     int32_t *sched = nullptr, *out = nullptr, *adv = nullptr;
-    int sched_cap = 0, sched_steps = 0, sched_rows = 0;
+    int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1;
@@ -457,8 +458,9 @@ extern "C" void lg_hip_model_destroy(lg_hip_model *m) {
     if (m->target) {
         auto &v = m->target->drafts;
         for (size_t i = 0; i < v.size(); ++i) if (v[i] == m) { v.erase(v.begin() + i); break; }
-    } else if (m->stream) (void)hipStreamDestroy(m->stream);
-    for (lg_hip_model *d : m->drafts) d->target = nullptr;        // orphaned heads refuse to run
+    }
+    if (m->owns_stream && m->stream) (void)hipStreamDestroy(m->stream);
+    for (lg_hip_model *d : m->drafts) { d->target = nullptr; d->stream = nullptr; }        // orphaned heads refuse to run
     delete m;
 }
 
@@ -948,11 +950,14 @@ extern "C" int lg_hip_draft_create(lg_hip_model *target, const struct lg_hip_con
     if (target->target) return fail(-2, "draft_create: the target is itself a draft head");
     if (target->n_kv_start < 2) return fail(-2, "draft_create: the target needs a sliding and a global cache layer to read");
     if (c->n_embd_per_layer) return fail(-2, "draft_create: a draft head has no per-layer embedding");
+    // the rounds kept on the device copy the head's tokens straight into the target's blocks: same vocabulary or none
+    if (c->n_vocab != target->n_vocab) return fail(-2, "draft_create: the head's vocabulary (%d) is not the target's (%d)", c->n_vocab, target->n_vocab);
     lg_hip_model *m = nullptr;
     int rc = lg_hip_model_create(c, target->device, &m);
     if (rc) return rc;
     (void)hipStreamDestroy(m->stream);
     m->stream = target->stream;                    // same queue: a draft reads what the last verify step wrote
+    m->owns_stream = false;
     m->target = target;
     m->window = target->window;
     m->n_kv_start = 0;
@@ -1106,18 +1111,22 @@ extern "C" int lg_hip_get_logits(lg_hip_model *m, int row, float *dst) {
 extern "C" int lg_hip_schedule_load(lg_hip_model *m, const int32_t *toks, int n_steps, int rows, int pos0) {
     if (!m || !toks || !m->committed) return fail(-1, "schedule_load: bad argument");
     if (rows < 1 || rows > m->max_rows || n_steps < 1 || n_steps > m->sched_cap) return fail(-2, "schedule_load: %d steps of %d rows (limits %d, %d)", n_steps, rows, m->sched_cap, m->max_rows);
+    if (pos0 < 0) return fail(-2, "schedule_load: position %d", pos0);
     for (size_t i = 0; i < (size_t)n_steps * rows; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "schedule_load: token id %d outside the vocabulary", toks[i]);
     HIP_TRY(hipSetDevice(m->device));
     HIP_TRY(hipStreamSynchronize(m->stream));
     HIP_TRY(hipMemcpy(m->sched, toks, (size_t)n_steps * rows * 4, hipMemcpyHostToDevice));
     StepCtl c{ pos0, 0, 0, 0 };
     HIP_TRY(hipMemcpy(m->ctl, &c, sizeof c, hipMemcpyHostToDevice));
-    m->sched_steps = n_steps; m->sched_rows = rows;
+    m->sched_steps = n_steps; m->sched_rows = rows; m->sched_pos0 = pos0; m->sched_loaded = n_steps;
     return 0;
 }
 extern "C" int lg_hip_schedule_run(lg_hip_model *m, lg_hip_kv *kv, int n_steps) {
     if (!m || !kv || kv->m != m) return fail(-1, "schedule_run: bad argument");
     if (n_steps < 1 || n_steps > m->sched_steps) return fail(-2, "schedule_run: %d steps requested, %d loaded", n_steps, m->sched_steps);
+    // every step may accept its whole block: the last one of this call may start rows * (steps so far) positions on
+    const long long last = (long long)m->sched_pos0 + (long long)m->sched_rows * (m->sched_loaded - m->sched_steps + n_steps);
+    if (last > kv->max_seq) return fail(-2, "schedule_run: positions up to %lld do not fit a cache of %d", last - 1, kv->max_seq);
     HIP_TRY(hipSetDevice(m->device));
     for (int s = 0; s < n_steps; ++s) { int rc = launch_step(m, kv, m->sched_rows, true); if (rc) return rc; }
     m->sched_steps -= n_steps;       // steps left to run

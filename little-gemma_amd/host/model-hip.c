@@ -22,6 +22,8 @@ const int model_kv_host = 0;          /* cache rows live on the device */
  * (src/cuda/model-cuda.cuh:724-726) */
 static lg_hip_model *g_dev;
 static const struct model *g_owner;
+static const void *g_owner_ctx;       /* the file the weights came from: a new model at a reused address is a new model */
+static int g_live;                    /* caches and draft heads that hold pointers into g_dev */
 static int g_logits_on;
 
 static void die(const char *what) {
@@ -31,8 +33,14 @@ static void die(const char *what) {
 
 /* Weights go up on first use (the reference's ensure_weights, src/cuda/model-cuda.cuh:738-799). */
 static lg_hip_model *device_model(const struct model *m) {
-    if (g_dev && g_owner == m) return g_dev;
-    if (g_dev) { lg_hip_model_destroy(g_dev); g_dev = NULL; }
+    if (g_dev && g_owner == m && g_owner_ctx == (const void *)m->ctx) return g_dev;
+    if (g_dev) {
+        if (g_live > 0) {
+            fprintf(stderr, "run-hip: one model per process: %d cache(s) / draft head(s) of the previous model are still alive\n", g_live);
+            exit(1);
+        }
+        lg_hip_model_destroy(g_dev); g_dev = NULL;
+    }
     const struct config *c = &m->cfg;
     struct lg_hip_config hc = {
         .n_layer = c->n_layer, .n_embd = c->n_embd, .n_head = c->n_head, .n_vocab = c->n_vocab,
@@ -54,7 +62,7 @@ static lg_hip_model *device_model(const struct model *m) {
     if (rows > LG_HIP_MAX_ROWS) rows = LG_HIP_MAX_ROWS;
     if (LG_MTP_N > LG_HIP_MAX_ROWS) { fprintf(stderr, "run-hip: LG_MTP_N=%d exceeds the %d rows the kernels are built for\n", LG_MTP_N, LG_HIP_MAX_ROWS); exit(1); }
     if (lg_hip_model_commit(g_dev, rows) != 0) die("model_commit");
-    g_owner = m;
+    g_owner = m; g_owner_ctx = (const void *)m->ctx;
     g_logits_on = 0;
     return g_dev;
 }
@@ -77,6 +85,7 @@ int kvcache_init(struct kvcache *kv, const struct model *m, int max_seq) {
     if (!kv->kv_dim || !kv->seq || !kv->f16 || !kv->k || !kv->v) return -1;
     lg_hip_kv *h = NULL;
     if (lg_hip_kv_create(d, max_seq, &h) != 0) die("kv_create");
+    g_live++;
     for (int L = 0; L < nl; L++) {
         int rows = 0, width = 0;
         lg_hip_kv_layout(h, L, &rows, &width);
@@ -90,7 +99,7 @@ int kvcache_init(struct kvcache *kv, const struct model *m, int max_seq) {
 
 void kvcache_free(struct kvcache *kv) {
     if (!kv) return;
-    lg_hip_kv_destroy(device_kv(kv));
+    if (device_kv(kv)) { lg_hip_kv_destroy(device_kv(kv)); if (g_live > 0) g_live--; }
     free(kv->k); free(kv->v); free(kv->kv_dim); free(kv->seq); free(kv->f16);
     memset(kv, 0, sizeof *kv);
 }
@@ -170,7 +179,7 @@ void model_prefill_reserve(void) { }
 int lg_model_last_hidden(struct model *m, float *dst) { return lg_hip_get_hidden(device_model(m), dst); }
 lg_hip_model *lg_model_device(struct model *m) { return device_model(m); }
 lg_hip_kv    *lg_model_device_kv(struct kvcache *kv) { return device_kv(kv); }
-void lg_model_release(void) { if (g_dev) { lg_hip_model_destroy(g_dev); g_dev = NULL; g_owner = NULL; } }
+void lg_model_release(void) { if (g_dev) { lg_hip_model_destroy(g_dev); g_dev = NULL; g_owner = NULL; g_owner_ctx = NULL; g_live = 0; } }
 
 /* ---- draft head on the device (src/cuda/mtp-kernel.cuh:272-402) --------------------------------
  * First use uploads the head (mtp_cuda_init there); a failure disables drafting for the process
@@ -207,6 +216,7 @@ static lg_hip_model *draft_model(struct mtp *t, const struct model *m) {
         return NULL;
     }
     t->cuda = d;
+    g_live++;
     return d;
 }
 static int draft_on_device(struct mtp *t, const struct model *m, const struct kvcache *kv, int token, int pos, int chain) {
@@ -238,7 +248,7 @@ int lg_model_mtp_rounds(struct mtp *t, const struct model *m, struct kvcache *kv
     return 0;
 }
 void mtp_free_device(struct mtp *t) {
-    if (t->cuda && t->cuda != (void *)-1) lg_hip_model_destroy((lg_hip_model *)t->cuda);
+    if (t->cuda && t->cuda != (void *)-1) { lg_hip_model_destroy((lg_hip_model *)t->cuda); if (g_live > 0) g_live--; }
     t->cuda = NULL;
 }
 /* the head's device handle, for callers that read its hidden state or logits */

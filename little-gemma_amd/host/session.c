@@ -7,6 +7,7 @@
 
 int lg_model_forward_spec_n(struct model *m, struct kvcache *kv, const int *toks, int rows, int pos, int *out);
 lg_hip_model *lg_mtp_device(struct mtp *t, const struct model *m);
+void lg_model_release(void);
 int lg_model_mtp_rounds(struct mtp *t, const struct model *m, struct kvcache *kv, int token, int pos, int rows,
                         int n_rounds, int *blocks, int *out, int *adv);
 
@@ -22,6 +23,7 @@ struct lg_session *lg_session_open(const char *path) {
 void lg_session_close(struct lg_session *s) {
     if (!s) return;
     if (s->has_kv) kvcache_free(&s->kv);
+    lg_model_release();               /* the device copy of the weights goes with the model it was made from */
     model_free(&s->m);
     free_gguf(s->ctx);
     free(s);

@@ -111,3 +111,63 @@ def gpu_required(lg):
     if lg.hiplib.device_count() < 1:
         pytest.fail("a test marked gpu ran without a GPU: the HIP path has no CPU fallback")
     return True
+
+
+def gguf_tensor_span(path, name):
+    """(file offset, byte length, dims) of one tensor's data in a GGUF file: a minimal reader of the container
+    (header, metadata, tensor infos, alignment) for tests that edit a generated model in place."""
+    import struct
+    sizes = {0: 1, 1: 1, 2: 2, 3: 2, 4: 4, 5: 4, 6: 4, 7: 1, 10: 8, 11: 8, 12: 8}
+    type_bytes = {0: (1, 4), 1: (1, 2), 2: (32, 18), 8: (32, 34), 30: (1, 2)}       # ggml type -> (block elems, block bytes)
+    with open(path, "rb") as f:
+        data = f.read()
+    at = 0
+
+    def take(fmt):
+        nonlocal at
+        v = struct.unpack_from("<" + fmt, data, at)
+        at += struct.calcsize("<" + fmt)
+        return v[0] if len(v) == 1 else v
+
+    def string():
+        nonlocal at
+        n = take("Q")
+        s = data[at:at + n].decode()
+        at += n
+        return s
+
+    def skip_value(t):
+        nonlocal at
+        if t == 8:
+            string()
+        elif t == 9:
+            et, n = take("I"), take("Q")
+            for _ in range(n):
+                skip_value(et)
+        else:
+            at += sizes[t]
+
+    magic, version, n_tensors, n_meta = take("I"), take("I"), take("Q"), take("Q")
+    assert magic == 0x46554747 and version in (2, 3)
+    align = 32
+    for _ in range(n_meta):
+        key, t = string(), take("I")
+        if key == "general.alignment" and t == 4:
+            align = take("I")
+        else:
+            skip_value(t)
+    found = None
+    for _ in range(n_tensors):
+        tname, nd = string(), take("I")
+        dims = [take("Q") for _ in range(nd)]
+        ttype, off = take("I"), take("Q")
+        if tname == name:
+            found = (ttype, dims, off)
+    assert found, f"{name} not in {path}"
+    base = (at + align - 1) // align * align
+    ttype, dims, off = found
+    be, bb = type_bytes[ttype]
+    n = 1
+    for d in dims:
+        n *= d
+    return base + off, n // be * bb, dims

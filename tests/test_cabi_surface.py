@@ -96,6 +96,27 @@ def test_model_hip_compiles_against_the_reference_headers():
                         f"-I{ref}/include", f"-I{ref}/src", f"-I{ROOT}/include", src], check=True)
 
 
+def test_reference_core_links_against_the_hip_backend(lg, tmp_path):
+    """The drop-in claim as a link: the reference's unmodified CLI core (the CORE list of its CMakeLists.txt:42-45:
+    run.c gguf.c quant.c model.c tokenizer.c media.c mtp.c + the no-op media GPU seam) compiled from where it
+    lies, with this repository's model-hip.c as the backend translation unit and liblg_hip.so behind it, must
+    link with no undefined symbol (what `-fsyntax-only` cannot show) and start (it prints its usage)."""
+    ref = "/root/reference"
+    if not os.path.isdir(os.path.join(ref, "src")) or not shutil.which("gcc"):
+        pytest.skip("reference sources absent")
+    lg.hiplib.load_hip()                                   # the library must be built
+    csrc = os.path.join(ROOT, "little-gemma_amd", "csrc")
+    exe = str(tmp_path / "run-hip-from-reference-core")
+    core = [os.path.join(ref, "src", f) for f in ("run.c", "gguf.c", "quant.c", "model.c", "tokenizer.c", "media.c", "mtp.c")]
+    core.append(os.path.join(ref, "src", "cpu", "media-gpu-stub.c"))
+    cmd = ["gcc", "-std=gnu11", "-O1", "-DLG_MTP_N=4", f"-I{ref}/include", f"-I{ref}/src", f"-I{ROOT}/include", *core,
+           os.path.join(ROOT, "little-gemma_amd", "host", "model-hip.c"), f"-L{csrc}", "-llg_hip", f"-Wl,-rpath,{csrc}",
+           "-Wl,--no-undefined", "-lm", "-fopenmp", "-o", exe]
+    subprocess.run(cmd, check=True)
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert "Usage" in (r.stdout + r.stderr) and "-mtp" in (r.stdout + r.stderr)
+
+
 def test_product_sources_do_not_touch_the_oracle():
     """Nothing that ships may include, link or import anything under oracle/."""
     pkg = os.path.join(ROOT, "little-gemma_amd")

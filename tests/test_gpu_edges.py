@@ -1,0 +1,137 @@
+"""Two edge cases of the reference interface on the GPU: argmax ties (the lower index wins,
+src/cuda/model-cuda.cuh:703-720, src/cpu/model-cpu.c:477-478) and the sampling hook model_pick
+(include/model.h:105-111, src/cuda/mtp-kernel.cuh:103-118)."""
+import ctypes as C
+import os
+import shutil
+
+import numpy as np
+import pytest
+
+from conftest import gguf_tensor_span
+from test_gpu_draft import write_head
+
+pytestmark = pytest.mark.gpu
+
+
+def duplicate_upper_vocabulary(path):
+    """Rows V/2 .. V-1 of token_embd become copies of rows 0 .. V/2-1: with the tied head every logit
+    then appears twice, V/2 apart, so every argmax is a tie."""
+    off, nbytes, dims = gguf_tensor_span(path, "token_embd.weight")
+    with open(path, "r+b") as f:
+        f.seek(off)
+        lower = f.read(nbytes // 2)
+        f.seek(off + nbytes // 2)
+        f.write(lower)
+    return dims[1]
+
+
+def test_argmax_ties_resolve_to_the_lower_index(lg, ob, gpu_required, model_path, model_dir):
+    src, spec = model_path("tiny_full")
+    path = os.path.join(str(model_dir), "tiny_full_tied.gguf")
+    shutil.copyfile(src, path)
+    V = duplicate_upper_vocabulary(path)
+    head_src = write_head(lg, model_dir, "tiny_full", spec)
+    head = os.path.join(str(model_dir), "assistant_tied.gguf")
+    shutil.copyfile(head_src, head)
+    assert duplicate_upper_vocabulary(head) == V
+    half = V // 2
+    rng = np.random.default_rng(41)
+    prompt = rng.integers(0, half, 40).astype(np.int32)
+    o = ob.Oracle(path)
+    od = o.mtp_open(head)
+    gpu = lg.hiplib.HipBackend(path, 160, max_rows=5)
+    t = gpu.mtp_open(head)
+    try:
+        kv = o.kv_new(160, ob.I8)
+        o.prefill(kv, prompt[:-1], 0, ob.I8)
+        gpu.prefill(prompt[:-1], 0)
+        gpu.set_option("store_logits", 1)
+        print("ties: one-row decode", flush=True)
+        tok, pos = int(prompt[-1]), len(prompt) - 1
+        for _ in range(6):                                # model_forward_next: argmax on the device
+            want, row, hid = o.forward(kv, tok, pos, ob.I8, want_hidden=True)
+            got = gpu.forward_next(tok, pos)
+            dev = gpu.logits_row(0, V)
+            assert np.array_equal(dev[:half].view(np.uint32), dev[half:].view(np.uint32))      # every value is tied
+            assert int(np.argmax(dev)) < half and dev[got] == dev.max()
+            assert got == want and got < half
+            tok, pos = got, pos + 1
+        print("ties: draft head", flush=True)
+        d_want, d_hid, _ = od.draft(kv, tok, pos, hid, ob.I8, want_logits=True)
+        d_got = gpu.mtp_draft(t, tok, pos, chain=False)
+        assert d_got == d_want and d_got < half
+        print("ties: verify rows", flush=True)
+        for step in range(4):                             # verify rows: every row's successor is the lower twin
+            blk = np.array([tok] + [int(x) for x in rng.integers(0, half, 4)], np.int32)
+            adv, out, _ = o.forward_spec_all(kv, blk, pos, ob.I8, want_hidden=True)
+            gadv, gout = gpu.forward_spec(blk, pos)
+            assert gadv == adv and gout.tolist() == list(out)
+            assert all(int(x) < half for x in gout)
+            for j in range(5):
+                dev = gpu.logits_row(j, V)
+                assert dev[int(gout[j])] == dev.max() == dev[int(gout[j]) + half]
+            tok, pos = int(out[adv - 1]), pos + adv
+    finally:
+        gpu.mtp_close(t); gpu.close(); od.close(); o.close()
+
+
+PICK = C.CFUNCTYPE(C.c_int, C.POINTER(C.c_float), C.c_int)
+
+
+def second_best(row):
+    """A deterministic rule that is not the argmax: the index of the second largest value (lower index on ties)."""
+    order = np.lexsort((np.arange(row.size), -row))
+    return int(order[1])
+
+
+def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
+    """With model_pick set the backend reads every row's logits back, lets the hook choose, accepts while the
+    choice agrees with the next draft, and re-points the hidden state at the last accepted row."""
+    path, spec = model_path("tiny_full")
+    V, E, rows = spec["n_vocab"], spec["n_embd"], 4
+    rng = np.random.default_rng(43)
+    prompt = rng.integers(0, V, 50).astype(np.int32)
+    o = ob.Oracle(path)
+    gpu = lg.hiplib.HipBackend(path, 200, max_rows=rows)
+    calls = []
+
+    def pick(ptr, n):
+        row = np.ctypeslib.as_array(ptr, shape=(n,))
+        calls.append(n)
+        return second_best(row)
+
+    hook = PICK(pick)
+    slot = C.c_void_p.in_dll(gpu.B, "model_pick")
+    try:
+        kv = o.kv_new(200, ob.I8)
+        o.prefill(kv, prompt[:-1], 0, ob.I8)
+        gpu.prefill(prompt[:-1], 0)
+        slot.value = C.cast(hook, C.c_void_p).value
+        tok, pos = int(prompt[-1]), len(prompt) - 1
+        seen = set()
+        for step in range(10):
+            # the oracle's own chain under the same rule gives drafts that hold; plant the first wrong one
+            first_bad = int(rng.integers(1, rows + 1))
+            blk, picks, hiddens = [tok], [], []
+            for j in range(rows):
+                _, row, hid = o.forward(kv, blk[j], pos + j, ob.I8, want_hidden=True)
+                picks.append(second_best(row)); hiddens.append(hid)
+                if j + 1 < rows:
+                    nxt = picks[j] if j + 1 < first_bad else (picks[j] + 1 + int(rng.integers(0, V - 1))) % V
+                    blk.append(nxt)
+            want_adv = 1
+            while want_adv < rows and picks[want_adv - 1] == blk[want_adv]:
+                want_adv += 1
+            print(f"hook step {step} pos {pos} first_bad {first_bad} adv {want_adv}", flush=True)
+            calls.clear()
+            adv, out = gpu.forward_spec(np.array(blk, np.int32), pos)
+            assert len(calls) == rows and all(n == V for n in calls)
+            assert adv == want_adv and out.tolist() == picks
+            assert np.array_equal(gpu.last_hidden(E).view(np.uint32), hiddens[adv - 1].view(np.uint32))
+            seen.add(adv)
+            tok, pos = picks[adv - 1], pos + adv
+        assert len(seen) >= 2                              # both partial and full acceptance were exercised
+    finally:
+        slot.value = None
+        gpu.close(); o.close()

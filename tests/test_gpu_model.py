@@ -20,9 +20,9 @@ def greedy_oracle(ob, o, prompt, n_gen, max_seq):
 
 @pytest.mark.parametrize("name", ["tiny", "tiny_full"])
 def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, golden, name):
-    """BASELINE config 1: 128-token uniform-random prompt, then 64 greedy tokens.  The prompt is the
-    one of the committed reference fixture, so the same run is also compared with the reference `run`
-    path (f32 activations): that gap is the q8 noise and is reported, not asserted to be zero."""
+    """BASELINE config 1: 128-token uniform-random prompt, then 64 greedy tokens, against the int8-class oracle.
+    The prompt is the one of the committed reference fixture; the comparison with the reference's own f32 run
+    is test_gpu_against_the_reference_fixture_teacher_forced below."""
     path, spec = model_path(name)
     g = golden(f"ref_{name}.npz")
     prompt = g["prompt"]
@@ -53,8 +53,44 @@ def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, gol
             gk, gv = gpu.kv_read(L, 0), gpu.kv_read(L, 1)
             assert gk.shape == K.shape
             assert np.array_equal(gk, K) and np.array_equal(gv, V), f"cache of layer {L}"
-        agree = sum(int(a == b) for a, b in zip(toks, g["tokens"]))
-        print(f"{name}: tokens equal to the f32-activation reference run at {agree}/{N_GEN} steps (q8 noise, informational)")
+    finally:
+        gpu.close(); o.close()
+
+
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+def test_gpu_against_the_reference_fixture_teacher_forced(lg, ob, gpu_required, model_path, golden, name):
+    """The one check tied directly to reference-produced data: the device, teacher-forced on the 64 greedy tokens
+    the reference's CPU `run` path produced (tests/golden/ref_*.npz, f32 activations), stays inside the band that
+    q8 activations imply.  Bars: logits within 0.3 relative L2 of the recorded reference rows at every recorded
+    step (the band of the CPU test of the int8 class), and the device's argmax equal to the reference's token at
+    40 of 64 steps or more (the CPU figure is 57 and 45 of 64).  The same numbers from the CPU oracle of the int8
+    class must come out identical, since the device is bit-identical to it."""
+    path, spec = model_path(name)
+    g = golden(f"ref_{name}.npz")
+    prompt, ref_tokens = g["prompt"], g["tokens"]
+    steps = {int(s): i for i, s in enumerate(g["logit_steps"])}
+    o = ob.Oracle(path)
+    gpu = lg.hiplib.HipBackend(path, N_PROMPT + N_GEN + 16, max_rows=1)
+    try:
+        okv = o.kv_new(N_PROMPT + N_GEN + 16, ob.I8)
+        o.prefill(okv, prompt[:-1], 0, ob.I8)
+        print(f"{name}: teacher-forced on the reference tokens", flush=True)
+        gpu.prefill(prompt[:-1], 0)
+        tok, pos, gaps, ogaps, agree, oagree = int(prompt[-1]), N_PROMPT - 1, [], [], 0, 0
+        for step in range(N_GEN):
+            row = gpu.forward(tok, pos, spec["n_vocab"])
+            obest, orow, _ = o.forward(okv, tok, pos, ob.I8)
+            if step in steps:
+                want = g["logits"][steps[step]]
+                gaps.append(float(np.linalg.norm(row - want) / np.linalg.norm(want)))
+                ogaps.append(float(np.linalg.norm(orow - want) / np.linalg.norm(want)))
+            agree += int(np.argmax(row)) == int(ref_tokens[step])
+            oagree += obest == int(ref_tokens[step])
+            tok, pos = int(ref_tokens[step]), pos + 1
+        print(f"{name}: rel-L2 to the reference logits {[round(x, 4) for x in gaps]}, argmax equal at {agree}/{N_GEN} steps", flush=True)
+        assert len(gaps) == len(steps) and max(gaps) < 0.3
+        assert agree >= 40
+        assert gaps == ogaps and agree == oagree
     finally:
         gpu.close(); o.close()
 

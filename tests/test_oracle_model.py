@@ -142,3 +142,30 @@ def test_int8_class_sequential_spec_equals_plain_decode(ob, model_path):
             at += adv; pos += adv
     finally:
         o.close()
+
+
+def test_argmax_ties_resolve_to_the_lower_index(lg, ob, model_path, model_dir):
+    """A vocabulary whose upper half repeats its lower half makes every logit a tie with its twin V/2 above:
+    the greedy token is always the lower one (src/cpu/model-cpu.c:477-478), in REF and in the int8 class."""
+    import os
+    import shutil
+    from conftest import gguf_tensor_span
+    src, spec = model_path("tiny")
+    path = os.path.join(str(model_dir), "tiny_tied_cpu.gguf")
+    shutil.copyfile(src, path)
+    off, nbytes, dims = gguf_tensor_span(path, "token_embd.weight")
+    with open(path, "r+b") as f:
+        f.seek(off); lower = f.read(nbytes // 2); f.seek(off + nbytes // 2); f.write(lower)
+    half = dims[1] // 2
+    o = ob.Oracle(path)
+    try:
+        for mode in (ob.REF, ob.I8):
+            kv = o.kv_new(32, mode)
+            tok = 3
+            for pos in range(6):
+                best, row, _ = o.forward(kv, tok, pos, mode)
+                assert np.array_equal(row[:half].view(np.uint32), row[half:].view(np.uint32))
+                assert best < half and row[best] == row.max()
+                tok = best
+    finally:
+        o.close()
