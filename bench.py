@@ -180,7 +180,23 @@ def main():
     ap.add_argument("--seed", type=int, default=7)
     ap.add_argument("--prefill", type=int, default=1024, help="positions of the prompt-processing measurement; 0 skips it")
     ap.add_argument("--mtp-steps", type=int, default=24, help="steps of the draft-head loop measurement (4 chained device drafts + verify); 0 skips it")
+    ap.add_argument("--launch-floor", action="store_true",
+                    help="measure only what a captured chain of dependent kernels costs (empty, and with a 64-byte hand-over) and exit")
     a = ap.parse_args()
+    if a.launch_floor:
+        import ctypes as C
+        H = lg.hiplib.load_hip()
+        H.lg_hip_launch_floor.argtypes = [C.c_int] * 5 + [C.POINTER(C.c_float)]
+        rows = []
+        for n in (426, 300):
+            for mode, what in ((0, "empty"), (1, "64-byte load+store hand-over")):
+                for grid, block in ((1, 64), (256, 256)):
+                    us = C.c_float(0)
+                    lg.hiplib.hip_check(H.lg_hip_launch_floor(n, mode, grid, block, 30, C.byref(us)), "launch_floor")
+                    rows.append({"kernels_per_graph": n, "kernel": what, "grid": grid, "block": block,
+                                 "us_per_kernel": round(us.value, 4), "ms_per_graph": round(us.value * n / 1e3, 4)})
+        print(json.dumps({"metric": "launch floor of a captured chain of dependent kernels", "unit": "us per kernel", "rows": rows}), flush=True)
+        return
     if a.gpus != 1:
         print("bench.py: this build measures one GPU; the verify step is not sharded (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)

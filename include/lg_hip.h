@@ -151,6 +151,13 @@ int  lg_hip_profile_step(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, in
                          int repeats, const char **names, float *ms, int32_t *launches,
                          double *bytes, int cap);
 
+/* What a chain of dependent kernels costs on this machine before it does any work: a captured graph of
+ * n_kernels launches in a row, each of grid x block threads, replayed `replays` times; mode 0 = empty kernels,
+ * mode 1 = every kernel reads the 64 bytes its predecessor wrote and writes 64 for its successor.
+ * *us_per_kernel = elapsed / (replays * n_kernels).  No reference counterpart (the reference's own measure of
+ * the same thing is its graph-vs-launch comparison, src/cuda/mtp-kernel.cuh:63-80). */
+int  lg_hip_launch_floor(int n_kernels, int mode, int grid, int block, int replays, float *us_per_kernel);
+
 /* ---- isolated kernels, host pointers in and out (parity tests of the parts) ----------------
  * q4_0 x q8_0 matmul (matmul_q_spec, src/cuda/model-cuda-i8.cu:1592-1602): w = m rows of k/32
  * 18-byte q4_0 blocks; x = rows x k floats, quantized on the device per 32 (d_quant_group,

@@ -1460,3 +1460,53 @@ extern "C" int lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, 
     HIP_TRY(hipGetLastError());
     return 0;
 }
+
+// ---- launch floor -----------------------------------------------------------------------------------
+// What a chain of dependent kernels costs before it does any work: a captured graph of n kernels in a row, each
+// empty (mode 0) or reading the 64 bytes its predecessor wrote and writing 64 for its successor (mode 1).
+__global__ void lg_k_floor_empty() {}
+__global__ void lg_k_floor_chain(const int *src, int *dst) {
+    if (blockIdx.x == 0 && threadIdx.x < 16) dst[threadIdx.x] = src[threadIdx.x] + 1;
+}
+extern "C" int lg_hip_launch_floor(int n_kernels, int mode, int grid, int block, int replays, float *us_per_kernel) {
+    if (n_kernels < 1 || n_kernels > 4096 || mode < 0 || mode > 1 || grid < 1 || grid > 65536 || block < 1 || block > 1024 ||
+        replays < 1 || !us_per_kernel) return fail(-2, "launch_floor: bad argument");
+    if (lg_hip_device_count() < 1) return fail(-3, "launch_floor: no HIP device");
+    hipStream_t st = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int *a = nullptr, *b = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+        HIP_TRY(hipMalloc((void **)&a, 256)); HIP_TRY(hipMalloc((void **)&b, 256));
+        HIP_TRY(hipMemset(a, 0, 256)); HIP_TRY(hipMemset(b, 0, 256));
+        HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        for (int i = 0; i < n_kernels; ++i) {
+            if (mode == 0) hipLaunchKernelGGL(lg_k_floor_empty, dim3(grid), dim3(block), 0, st);
+            else hipLaunchKernelGGL(lg_k_floor_chain, dim3(grid), dim3(block), 0, st, (i & 1) ? b : a, (i & 1) ? a : b);
+        }
+        HIP_TRY(hipStreamEndCapture(st, &graph));
+        HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        HIP_TRY(hipGraphLaunch(exec, st));                   // warm-up
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipEventRecord(e0, st));
+        for (int r = 0; r < replays; ++r) HIP_TRY(hipGraphLaunch(exec, st));
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        float ms = 0;
+        HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+        *us_per_kernel = ms * 1e3f / ((float)replays * (float)n_kernels);
+        return 0;
+    };
+    const int rc = body();
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (a) (void)hipFree(a);
+    if (b) (void)hipFree(b);
+    if (st) (void)hipStreamDestroy(st);
+    return rc;
+}
