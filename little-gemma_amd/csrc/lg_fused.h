@@ -234,3 +234,272 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
     for (int j = 0; j < M; ++j) acc[j] = lg_sum_seg<8>(acc[j]);
     if (c < M) a.out[(size_t)c * a.m + gi * 8 + (lane >> 3)] = lg_pick<M>(acc, c);
 }
+
+// ---------------------------------------------------------------------------------------------
+// Attention tiles of a verify block for layers with many tiles (long global contexts, wide sliding windows):
+// one workgroup per (tile, kv head) serves ALL rows of the block against one staged K/V tile, where lg_k_attn
+// runs a workgroup per row and stages every tile once per row.  The queries arrive normed and rotated
+// (lg_k_qkv_post has run and has written the block's K/V rows to the cache).  Same arithmetic and order as
+// lg_k_attn: score = (a0+a1)+(a2+a3) over four fma chains, tile max / exp / 32-lane tree sum, value accumulation
+// over the slots ascending; the partials go to the same slots and lg_k_attn_merge finishes them.
+//
+// A unit is one (row, query head) pair, M*G of them; a wavefront takes the units wave, wave + 4, ... three at a
+// time, so that one LDS read of a K (V) row serves three units and 6 (12) independent fma chains are in flight.
+// K is staged in reader order (the lane of key slot sl and chain pair hf finds its hd/4 dwords as consecutive
+// 16-byte units); the queries are read 16 bytes at a time, the same address in all lanes of a half.  Every slot of
+// a tile goes through the value chains: slots outside a row's keys have exponential zero and zeroed or finite
+// values, and fma(0, v, acc) is acc for every acc that a chain started at +0 can hold.
+//
+// A workgroup takes `tp` consecutive tiles; the next tile's rows are requested into registers before the current
+// tile is computed, so the memory latency of all tiles but the first is covered.
+
+// fmaf(x, (float)h, acc) with h the low (high) f16 half of a packed pair: one instruction; the conversion is exact
+// and the sum rounds once, as the two-instruction form does.  The compiler picks this instruction by itself when a
+// converted value feeds one fma; written out here because each key/value element feeds one fma per unit.
+__device__ __forceinline__ float lg_fma_hlo(float x, uint32_t hp, float acc) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel_hi:[0,1,0]" : "+v"(acc) : "v"(x), "v"(hp));
+    return acc;
+}
+__device__ __forceinline__ float lg_fma_hhi(float x, uint32_t hp, float acc) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : "+v"(acc) : "v"(x), "v"(hp));
+    return acc;
+}
+
+template <int HD>
+struct AttnRowsGeo {
+    static constexpr int KSD = HD / 2 + 4;                    // dwords per staged K row (16-byte reads of 8 slots cover all banks)
+    static constexpr int VST = HD + 8;                        // halves per staged V row
+    static size_t bytes(int units) {
+        return (size_t)units * HD * 4 + (size_t)32 * KSD * 4 + (size_t)32 * VST * 2 + (size_t)units * 32 * 4;
+    }
+};
+template <int M, int HD>
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(AttnArgs a, const StepCtl *ctl, int tp) {
+    using Geo = AttnRowsGeo<HD>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int G = a.H / a.nkv, units = M * G;
+    float *qs = (float *)smem;                                // [unit][hf][HD/2]: element i at hf = (i%4)/2, 2*(i/4) + i%2
+    uint32_t *kt = (uint32_t *)(qs + (size_t)units * HD);     // [32][KSD]: row sl = [hf][HD/4 dwords]
+    uint16_t *vt = (uint16_t *)(kt + 32 * Geo::KSD);          // [32][VST]
+    float *es = (float *)(vt + 32 * Geo::VST);                // [unit][32]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kvh = blockIdx.y;
+    const int pos0 = ctl->pos + a.pos_off, plast = pos0 + M - 1;
+    const int start0 = lg_win_start(pos0, a.window), first = start0 >> 5, last = plast >> 5;
+    const int b0 = blockIdx.x * tp;                           // tiles first + b0 .. first + b0 + tp - 1
+    if (first + b0 > last) return;                            // no row of the block has keys here
+    constexpr int U4R = HD / 8;                               // 16-byte units per K/V row
+    constexpr int KL = (32 * U4R + LG_WG - 1) / LG_WG;        // 16-byte units of K (and of V) per thread
+    static_assert(32 * U4R % LG_WG == 0 || 32 * U4R < LG_WG, "tile staging assumes whole passes");
+    uint4 kq[KL], vq[KL];
+    auto fetch = [&](int bx) {
+        const int r0 = ((first + bx) << 5) % a.seq;
+        #pragma unroll
+        for (int u = 0; u < KL; ++u) {
+            const int idx = min((int)threadIdx.x + u * LG_WG, 32 * U4R - 1), row = idx / U4R, u4 = idx - row * U4R;
+            int rr = r0 + row; if (rr >= a.seq) rr -= a.seq;
+            const size_t go = (size_t)rr * a.kv_dim + (size_t)kvh * HD + u4 * 8;
+            kq[u] = a.kc4(go); vq[u] = a.vc4(go);
+        }
+    };
+    auto stash = [&](int bx) {
+        // slots outside the keys of every row of the block are zeroed (their exponentials are zero, and zero times
+        // a finite value leaves the sums as they are; stale bits that read as infinities would not)
+        const int t0 = (first + bx) << 5, slo = start0 - t0, shi = plast - t0;
+        #pragma unroll
+        for (int u = 0; u < KL; ++u) {
+            const int idx = (int)threadIdx.x + u * LG_WG, row = idx / U4R, u4 = idx - row * U4R;
+            if (32 * U4R < LG_WG && idx >= 32 * U4R) continue;
+            const uint32_t mk = (row >= slo && row <= shi) ? 0xFFFFFFFFu : 0u;
+            uint32_t *d = kt + row * Geo::KSD + 2 * u4;
+            *(uint2 *)d = make_uint2(kq[u].x & mk, kq[u].z & mk);             // chains 0,1 of two groups of four dims
+            *(uint2 *)(d + HD / 4) = make_uint2(kq[u].y & mk, kq[u].w & mk);  // chains 2,3
+            *(uint4 *)(vt + row * Geo::VST + u4 * 8) = make_uint4(vq[u].x & mk, vq[u].y & mk, vq[u].z & mk, vq[u].w & mk);
+        }
+    };
+    fetch(b0);
+    {   // the queries, once per workgroup (their loads follow the first tile's before any store)
+        constexpr int QB = 4;                                 // float4 of query per thread and pass
+        const int nq4 = units * (HD / 4);
+        for (int base = 0; base < nq4; base += QB * LG_WG) {
+            float4 qreg[QB];
+            #pragma unroll
+            for (int i = 0; i < QB; ++i) {
+                const int idx = min(base + (int)threadIdx.x + i * LG_WG, nq4 - 1);
+                const int u = idx / (HD / 4), g4 = idx - u * (HD / 4), j = u / G, g = u - j * G;
+                qreg[i] = *(const float4 *)(a.q + (size_t)j * a.H * HD + (size_t)(kvh * G + g) * HD + 4 * g4);
+            }
+            #pragma unroll
+            for (int i = 0; i < QB; ++i) {
+                const int idx = base + (int)threadIdx.x + i * LG_WG;
+                if (idx < nq4) {
+                    const int u = idx / (HD / 4), g4 = idx - u * (HD / 4);
+                    float *qd = qs + (size_t)u * HD + 2 * g4;
+                    *(float2 *)qd = make_float2(qreg[i].x, qreg[i].y);
+                    *(float2 *)(qd + HD / 2) = make_float2(qreg[i].z, qreg[i].w);
+                }
+            }
+        }
+    }
+    constexpr int NWV = LG_WG / 64, UB = 3;
+    for (int i = 0; i < tp; ++i) {
+        const int bx = b0 + i, n = first + bx, t0 = n << 5;
+        if (n > last) break;
+        if (i > 0) __syncthreads();                           // the previous tile has been read by every wavefront
+        stash(bx);
+        __syncthreads();
+        if (i + 1 < tp && n + 1 <= last) fetch(bx + 1);
+        {   // scores
+            const int sl = lane & 31, hf = lane >> 5, t = t0 + sl;
+            const uint32_t *ks = kt + sl * Geo::KSD + hf * (HD / 4);
+            for (int ub = wave; ub < units; ub += UB * NWV) {
+                int un[UB];
+                const float *qr[UB];
+                float ax[UB], ay[UB];
+                #pragma unroll
+                for (int b = 0; b < UB; ++b) {                // (a missing unit repeats the first one and stores nothing)
+                    un[b] = ub + b * NWV < units ? ub + b * NWV : ub;
+                    qr[b] = qs + (size_t)un[b] * HD + hf * (HD / 2);
+                    ax[b] = 0.0f; ay[b] = 0.0f;
+                }
+                #pragma unroll 2
+                for (int u = 0; u < HD / 16; ++u) {
+                    const uint4 k4 = *(const uint4 *)(ks + 4 * u);
+                    #pragma unroll
+                    for (int b = 0; b < UB; ++b) {
+                        const float4 p0 = *(const float4 *)(qr[b] + 8 * u), p1 = *(const float4 *)(qr[b] + 8 * u + 4);
+                        ax[b] = lg_fma_hlo(p0.x, k4.x, ax[b]); ay[b] = lg_fma_hhi(p0.y, k4.x, ay[b]);
+                        ax[b] = lg_fma_hlo(p0.z, k4.y, ax[b]); ay[b] = lg_fma_hhi(p0.w, k4.y, ay[b]);
+                        ax[b] = lg_fma_hlo(p1.x, k4.z, ax[b]); ay[b] = lg_fma_hhi(p1.y, k4.z, ay[b]);
+                        ax[b] = lg_fma_hlo(p1.z, k4.w, ax[b]); ay[b] = lg_fma_hhi(p1.w, k4.w, ay[b]);
+                    }
+                }
+                #pragma unroll
+                for (int b = 0; b < UB; ++b) {
+                    if (b > 0 && un[b] == ub) continue;
+                    const int unit = un[b], j = unit / G, pj = pos0 + j, startj = lg_win_start(pj, a.window);
+                    if (n < (startj >> 5) || n > (pj >> 5)) continue;         // tile outside this row's keys (wavefront-uniform)
+                    const bool valid = t >= startj && t <= pj;
+                    float s = lg_add_x32(ax[b] + ay[b]);      // (a0+a1) + (a2+a3): the two halves sit 32 lanes apart
+                    if (!valid) s = -INFINITY;
+                    const float mx = lg_max_n(s, 32);
+                    const float e = valid ? lg_expf(s - mx) : 0.0f;
+                    const float l = lg_sum32(e);
+                    if (hf == 0) es[unit * 32 + sl] = e;
+                    if (lane == 0) {
+                        const size_t pi = ((size_t)j * a.H + kvh * G + (unit - j * G)) * a.tiles_max + bx;
+                        a.pm[pi] = mx; a.pl[pi] = l;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        {   // values (lane = 4 dims)
+            const uint16_t *vl = vt + (4 * lane < HD ? 4 * lane : 0);
+            for (int ub = wave; ub < units; ub += UB * NWV) {
+                int un[UB];
+                bool on[UB];
+                const float *er[UB];
+                float4 acc[UB];
+                #pragma unroll
+                for (int b = 0; b < UB; ++b) {
+                    un[b] = ub + b * NWV < units ? ub + b * NWV : ub;
+                    const int j = un[b] / G, pj = pos0 + j, startj = lg_win_start(pj, a.window);
+                    on[b] = !(n < (startj >> 5) || n > (pj >> 5)) && !(b > 0 && un[b] == ub);
+                    er[b] = es + un[b] * 32;                  // (a unit that skipped the scores has stale rows here: never stored)
+                    acc[b] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                }
+                #pragma unroll 2
+                for (int u4 = 0; u4 < 8; ++u4) {
+                    float ev[UB][4];
+                    #pragma unroll
+                    for (int b = 0; b < UB; ++b) {
+                        const float4 e4 = *(const float4 *)(er[b] + 4 * u4);
+                        ev[b][0] = e4.x; ev[b][1] = e4.y; ev[b][2] = e4.z; ev[b][3] = e4.w;
+                    }
+                    #pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint2 v = *(const uint2 *)(vl + (4 * u4 + q) * Geo::VST);
+                        #pragma unroll
+                        for (int b = 0; b < UB; ++b) {
+                            acc[b].x = lg_fma_hlo(ev[b][q], v.x, acc[b].x); acc[b].y = lg_fma_hhi(ev[b][q], v.x, acc[b].y);
+                            acc[b].z = lg_fma_hlo(ev[b][q], v.y, acc[b].z); acc[b].w = lg_fma_hhi(ev[b][q], v.y, acc[b].w);
+                        }
+                    }
+                }
+                #pragma unroll
+                for (int b = 0; b < UB; ++b) {
+                    if (!on[b]) continue;
+                    const int unit = un[b], j = unit / G;
+                    const size_t pi = ((size_t)j * a.H + kvh * G + (unit - j * G)) * a.tiles_max + bx;
+                    if (4 * lane < HD) *(float4 *)(a.pacc + pi * HD + 4 * lane) = acc[b];
+                }
+            }
+        }
+    }
+}
+
+// lg_k_attn_merge for rows with very many tiles: one wavefront per (head, row, 64 dims) instead of one workgroup per
+// (head, row), so that four times as many CUs pull the partials (a (head, row) at 8192 keys has 257 KB of them).
+// Same order: weights exp(m_t - M), L and the output as fma chains over the tiles ascending, divide, q8.
+template <int M>
+__global__ __launch_bounds__(64) void lg_k_attn_merge_split(MergeArgs a, const StepCtl *ctl) {
+    __shared__ float wts[512];
+    const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd, lane = threadIdx.x;
+    const int d = blockIdx.z * 64 + lane;                     // hd is a multiple of 64
+    const int pos = ctl->pos + a.pos_off, pj = pos + j;
+    const int first = lg_win_start(pos, a.window) >> 5;
+    const int lo = (lg_win_start(pj, a.window) >> 5) - first, hi = (pj >> 5) - first;
+    const size_t base = ((size_t)j * a.H + head) * a.tiles_max;
+    // the partials do not depend on the weights: the first batch of them is requested before the maxima are read,
+    // and from then on batch n + 1 is in flight while batch n goes through the chains
+    constexpr int U = 32;
+    const int nt = hi - lo + 1;
+    float pl0[U], pa0[U], pl1[U], pa1[U];
+    auto fetch = [&](float (&pl)[U], float (&pa)[U], int n0) {
+        #pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int n = n0 + u < nt ? n0 + u : nt - 1;
+            pl[u] = a.pl[base + lo + n];
+            pa[u] = a.pacc[(base + lo + n) * hd + d];
+        }
+    };
+    fetch(pl0, pa0, 0);
+    float mx = -INFINITY;
+    for (int n = lo + lane; n <= hi; n += 64) mx = fmaxf(mx, a.pm[base + n]);
+    mx = lg_max_n(mx, 64);
+    float L = 0.0f, o = 0.0f;
+    auto chain = [&](const float (&pl)[U], const float (&pa)[U], int n0, int c0) {
+        #pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (n0 + u < nt) {
+                const float wn = wts[n0 + u - c0];
+                L = lg_fmaf(pl[u], wn, L);
+                o = lg_fmaf(pa[u], wn, o);
+            }
+        }
+    };
+    for (int c0 = 0; c0 < nt; c0 += 512) {                    // (512 is a multiple of 2 * U)
+        const int cn = nt - c0 < 512 ? nt - c0 : 512;
+        lg_wave_lds_sync();
+        for (int n = lane; n < cn; n += 64) wts[n] = lg_expf(a.pm[base + lo + c0 + n] - mx);
+        lg_wave_lds_sync();
+        for (int n0 = c0; n0 < c0 + cn; n0 += 2 * U) {
+            if (n0 + U < nt) fetch(pl1, pa1, n0 + U);
+            __builtin_amdgcn_sched_barrier(0);
+            chain(pl0, pa0, n0, c0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (n0 + 2 * U < nt) fetch(pl0, pa0, n0 + 2 * U);
+            __builtin_amdgcn_sched_barrier(0);
+            chain(pl1, pa1, n0 + U, c0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    const float r = o / L;
+    float dq; int sum;
+    const int q = lg_quant1_32lanes(r, &dq, &sum);
+    const int e = head * hd + d;
+    a.xq[lg_q8_off<M>(qd, j, e >> 4, e & 15)] = (int8_t)q;
+    if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));
+    if (a.xf) a.xf[(size_t)j * qd + e] = r;
+}

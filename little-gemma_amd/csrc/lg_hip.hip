@@ -157,7 +157,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -206,6 +206,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     m->n_head_kv.assign(c->n_head_kv, c->n_head_kv + c->n_layer);
     if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
     if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
+    if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
     *out = m;
@@ -678,6 +679,17 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
 }
 
 // one block of M rows through the decoder (and the head when with_head)
+static bool attention_rows_shared(int rows, int tiles, int nkv, int hd, int seq) {
+    return rows > 1 && rows <= LG_HIP_MAX_ROWS && hd <= 256 && seq >= 32 && tiles * nkv >= 256;
+}
+// tiles per workgroup of lg_k_attn_rows: one, until the grid would exceed the three workgroups per CU that the
+// staged tile's LDS lets a CU hold; then as many as bring it back under that (at most four), each tile's rows in
+// flight while the tile before it is computed
+static int attention_rows_tp(int tiles, int nkv) {
+    const int tp = (tiles * nkv + 3 * 256 - 1) / (3 * 256);
+    return tp < 1 ? 1 : tp > 4 ? 4 : tp;
+}
+
 template <int M>
 static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry) {
     Launcher lx{ m, dry };
@@ -760,6 +772,19 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                    1.0f / sqrtf((float)E), sqrtf((float)m->ple), 1.0f / sqrtf(2.0f), m->eps };
         LAUNCH(KC_PMP, lg_k_ipl, dim3(nl, M), dim3(64), 0, i, m->ctl);
     }
+    // tiles a block of layer L can touch (a sliding layer needs only its window's, not the cache's), and whether the
+    // layer takes the kernel that serves all rows of a block per (tile, kv head)
+    auto layer_tiles = [&](int L) {
+        const Layer &y = m->L[L];
+        const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
+        int tiles = kv->tiles_max;
+        if (window > 0 && M <= LG_HIP_MAX_ROWS) { const int t = (window + M - 1 + 31) / 32 + 1; if (t < tiles) tiles = t; }
+        return tiles;
+    };
+    auto rows_shared = [&](int L) {
+        const Layer &y = m->L[L];
+        return pos_off == 0 && m->attn_rows && attention_rows_shared(M, layer_tiles(L), y.nkv, y.hd, kv->seq[y.src]);
+    };
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
@@ -770,6 +795,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             else { rows(y.attn_norm, nullptr); launch_mm<M, false>(lx, KC_QKV, a); }
             // blocks of the model itself, up to LG_HIP_MAX_ROWS rows: the attention kernel does this part as well
             fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
+            // ... unless the layer has so many (tile, kv head) pairs that one workgroup per pair can serve all rows of
+            // the block against one staged tile (long global contexts, wide windows): the rows then arrive prepared
+            if (rows_shared(L)) fused_post = false;
             QkvPostArgs p{};
             p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
             p.H = H; p.nkv = y.nkv; p.hd = y.hd;
@@ -785,9 +813,18 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.q = m->q_rot; a.H = H; a.nkv = y.nkv; a.hd = y.hd;
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
-            // tiles a block of this layer can touch: a sliding layer needs only its window's, not the cache's
-            int tiles = kv->tiles_max;
-            if (window > 0 && M <= LG_HIP_MAX_ROWS) { const int t = (window + M - 1 + 31) / 32 + 1; if (t < tiles) tiles = t; }
+            const int tiles = layer_tiles(L);
+            const bool shared = rows_shared(L);
+            if (shared) {
+                if constexpr (M > 1 && M <= LG_HIP_MAX_ROWS) {
+                    const size_t lds = y.hd == 256 ? AttnRowsGeo<256>::bytes(M * G) : y.hd == 128 ? AttnRowsGeo<128>::bytes(M * G) : AttnRowsGeo<64>::bytes(M * G);
+                    const int tp = attention_rows_tp(tiles, y.nkv);
+                    const dim3 grid((tiles + tp - 1) / tp, y.nkv);
+                    if (y.hd == 256)      LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
+                    else if (y.hd == 128) LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
+                    else                  LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
+                }
+            } else
             if (fused_post) {
                 a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
                 a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
@@ -798,7 +835,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
-            LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
+            if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(64), 0, g, m->ctl);
+            else LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
         {   // attention output projection
             MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, nullptr };
@@ -879,7 +917,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -914,6 +952,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "use_graph")) m->use_graph = value != 0;
     else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
+    else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
 }
@@ -1028,7 +1067,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r");
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -1319,10 +1358,26 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
 }
 
 // the two launches of an isolated attention: tile partials, then the ordered merge
+// (the same choice of kernels as a verify step makes: many (tile, kv head) pairs -> one workgroup per pair serves all
+// rows; many tiles per row -> the merge is cut by dims)
 template <int M>
-static void enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs &g, StepCtl *ctl, int tiles, size_t lds) {
-    hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
-    hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
+static int enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs &g, StepCtl *ctl, int tiles, size_t lds) {
+    if (attention_rows_shared(M, tiles, a.nkv, a.hd, a.seq)) {
+        if constexpr (M > 1 && M <= LG_HIP_MAX_ROWS) {
+            const int units = M * (a.H / a.nkv);
+            const size_t l2 = a.hd == 256 ? AttnRowsGeo<256>::bytes(units) : a.hd == 128 ? AttnRowsGeo<128>::bytes(units) : AttnRowsGeo<64>::bytes(units);
+            int rc = a.hd == 256 ? set_lds(lg_k_attn_rows<M, 256>, l2) : a.hd == 128 ? set_lds(lg_k_attn_rows<M, 128>, l2) : set_lds(lg_k_attn_rows<M, 64>, l2);
+            if (rc) return rc;
+            const int tp = attention_rows_tp(tiles, a.nkv);
+            const dim3 grid((tiles + tp - 1) / tp, a.nkv);
+            if (a.hd == 256)      hipLaunchKernelGGL((lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
+            else if (a.hd == 128) hipLaunchKernelGGL((lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
+            else                  hipLaunchKernelGGL((lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
+        }
+    } else hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
+    if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && a.hd % 64 == 0) hipLaunchKernelGGL((lg_k_attn_merge_split<M>), dim3(a.H, M, a.hd / 64), dim3(64), 0, st, g, ctl);
+    else hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
+    return 0;
 }
 
 template <int M>
@@ -1335,7 +1390,8 @@ static int attention_rows(hipStream_t st, AttnArgs a, MergeArgs g, StepCtl *ctl,
         HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
         for (int r = 0; r < repeats + 1; ++r) {
             if (r == 1) HIP_TRY(hipEventRecord(e0, st));
-            enqueue_attention<M>(st, a, g, ctl, tiles, lds);
+            const int erc = enqueue_attention<M>(st, a, g, ctl, tiles, lds);
+            if (erc) return erc;
         }
         HIP_TRY(hipEventRecord(e1, st));
         HIP_TRY(hipStreamSynchronize(st));
@@ -1453,10 +1509,11 @@ extern "C" int lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, 
     // cleared; only the step state is set, by a kernel (a caller may be capturing this stream)
     hipLaunchKernelGGL(lg_k_set_ctl, dim3(1), dim3(1), 0, st, ctl, pos);
     switch (rows) {
-#define CASE(M) case M: enqueue_attention<M>(st, a, g, ctl, tiles, lds); break;
+#define CASE(M) case M: rc = enqueue_attention<M>(st, a, g, ctl, tiles, lds); break;
         CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
 #undef CASE
     }
+    if (rc) return rc;
     HIP_TRY(hipGetLastError());
     return 0;
 }
