@@ -236,6 +236,113 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// lm_head for verify blocks of 4..8 rows on the matrix cores: lg_k_geglu_m's tile loop (row-block tiles of the
+// vocabulary matrix, a wavefront = 64 vocabulary rows x one of the 8 K segments, two v_mfma_i32_32x32x32_i8 per
+// tile whatever M is, the activations in the same 80-dword block order) with lg_k_mm_head's epilogue: the 8
+// segment sums of a logit meet in the adjacent-pair tree, soft cap, optional store, running argmax per draft row
+// (first maximum: the lower index wins ties).  A workgroup walks `passes` consecutive blocks of 64 rows; the
+// first tiles of the next block are requested while the last of this one are multiplied, and the segment sums
+// go through one of two LDS buffers in turn, so a block costs one barrier.
+template <int M>
+__global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];     // [8 segments][nit][80 dwords]
+    __shared__ float red[2][8][LG_HIP_MAX_ROWS_DEV][64];
+    constexpr int CH = 2;
+    const int lane = threadIdx.x & 63, n = lane & 31, h = lane >> 5;
+    const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));      // K segment of this wavefront, and its draft row in the epilogue
+    const int nb = a.k >> 5, nit = nb >> 3, nblk = a.n_vocab >> 6;
+    const int t0 = blockIdx.x * a.passes, np = nblk - t0 < a.passes ? nblk - t0 : a.passes;
+    uint4 wq[CH], nwq[CH]; uint32_t wd[CH], nwd[CH];
+    auto fetch = [&](int p, int it0) {
+        const uint8_t *wt = a.w + ((size_t)(t0 + p) * nb + (size_t)s * nit) * LG_TILE;
+        #pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;
+            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
+            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+        }
+    };
+    if (np > 0) fetch(0, 0);
+    unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
+    {   // the wavefront's K segment of the activations, once (wave-private, no barrier)
+        const uint4 *src = (const uint4 *)(a.q_in + (size_t)s * nit * (LG_MU_DWORDS * 4));
+        const int nu = nit * (LG_MU_DWORDS / 4);
+        for (int i0 = lane; i0 < nu; i0 += 256) {
+            const int i1 = min(i0 + 64, nu - 1), i2 = min(i0 + 128, nu - 1), i3 = min(i0 + 192, nu - 1);
+            const uint4 t0v = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
+            __builtin_amdgcn_sched_barrier(0);
+            ((uint4 *)la)[i0] = t0v; ((uint4 *)la)[i1] = t1; ((uint4 *)la)[i2] = t2; ((uint4 *)la)[i3] = t3;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    lg_v16i magic;                                            // (float)(dot - 8*sum) in one subtraction: see lg_k_geglu_m
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;
+    const int arow = n < 8 ? n : 7;
+    float best = -INFINITY;                                   // wavefront s < M tracks draft row s, one vocabulary row per lane and block
+    int besti = 0x7fffffff;
+    for (int p = 0; p < np; ++p) {
+        float p0[4] = { 0.0f, 0.0f, 0.0f, 0.0f }, p1[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+        for (int it0 = 0; it0 < nit; it0 += CH) {
+            #pragma unroll
+            for (int u = 0; u < CH; ++u) { wq[u] = nwq[u]; wd[u] = nwd[u]; }
+            if (it0 + CH < nit) fetch(p, it0 + CH);
+            else if (p + 1 < np) fetch(p + 1, 0);
+            #pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                if (it0 + c < nit) {
+                    const unsigned char *lb = la + (size_t)(it0 + c) * (LG_MU_DWORDS * 4);
+                    const lg_v4i av = *(const lg_v4i *)(lb + arow * 32 + h * 16);
+                    const int4 sc0 = *(const int4 *)(lb + 256 + h * 32), sc1 = *(const int4 *)(lb + 256 + h * 32 + 16);
+                    const uint4 q = wq[c];
+                    const lg_v2u s0 = __builtin_amdgcn_permlane32_swap(q.x, q.z, false, false);
+                    const lg_v2u s1 = __builtin_amdgcn_permlane32_swap(q.y, q.w, false, false);
+                    const lg_v2u sd = __builtin_amdgcn_permlane32_swap(wd[c], wd[c], false, false);
+                    lg_v4i b0, b1;
+                    b0.x = s0.x & 0x0F0F0F0F; b0.y = s1.x & 0x0F0F0F0F; b0.z = (s0.x >> 4) & 0x0F0F0F0F; b0.w = (s1.x >> 4) & 0x0F0F0F0F;
+                    b1.x = s0.y & 0x0F0F0F0F; b1.y = s1.y & 0x0F0F0F0F; b1.z = (s0.y >> 4) & 0x0F0F0F0F; b1.w = (s1.y >> 4) & 0x0F0F0F0F;
+                    const float w0 = lg_h2f((uint16_t)sd.x), w1 = lg_h2f((uint16_t)sd.y);
+                    const lg_v16i d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b0, magic, 0, 0, 0);
+                    const lg_v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, b1, magic, 0, 0, 0);
+                    const float xd[4] = { __int_as_float(sc0.x), __int_as_float(sc0.z), __int_as_float(sc1.x), __int_as_float(sc1.z) };
+                    const float cf[4] = { __int_as_float(sc0.y), __int_as_float(sc0.w), __int_as_float(sc1.y), __int_as_float(sc1.w) };
+                    #pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        p0[i] = lg_fmaf(xd[i] * w0, __int_as_float(d0[i]) - cf[i], p0[i]);
+                        p1[i] = lg_fmaf(xd[i] * w1, __int_as_float(d1[i]) - cf[i], p1[i]);
+                    }
+                }
+            }
+        }
+        float (*rb)[LG_HIP_MAX_ROWS_DEV][64] = red[p & 1];
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) { rb[s][4 * h + i][n] = p0[i]; rb[s][4 * h + i][32 + n] = p1[i]; }
+        __syncthreads();                                      // (the buffer written two blocks ago was read before the barrier of the last block)
+        if (s < M) {
+            float g[8];
+            #pragma unroll
+            for (int c = 0; c < 8; ++c) g[c] = rb[c][s][lane];
+            float v = ((g[0] + g[1]) + (g[2] + g[3])) + ((g[4] + g[5]) + (g[6] + g[7]));
+            if (a.softcap > 0.0f) v = a.softcap * lg_tanhf(v / a.softcap);
+            const int row = (t0 + p) * 64 + lane;
+            if (a.logits) a.logits[(size_t)s * a.n_vocab + row] = v;
+            if (v > best) { best = v; besti = row; }          // (rows ascend with p: a later equal value never replaces)
+        }
+    }
+    if (s < M) {
+        #pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float ov = __shfl_xor(best, o);
+            const int oi = __shfl_xor(besti, o);
+            if (ov > best || (ov == best && oi < besti)) { best = ov; besti = oi; }
+        }
+        if (lane == 0) { a.pval[(size_t)blockIdx.x * M + s] = best; a.pidx[(size_t)blockIdx.x * M + s] = besti; }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Attention tiles of a verify block for layers with many tiles (long global contexts, wide sliding windows):
 // one workgroup per (tile, kv head) serves ALL rows of the block against one staged K/V tile, where lg_k_attn
 // runs a workgroup per row and stages every tile once per row.  The queries arrive normed and rotated

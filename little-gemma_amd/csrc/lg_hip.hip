@@ -143,6 +143,7 @@ struct lg_hip_model {
     // weights
     std::vector<Layer> L;
     uint8_t *emb = nullptr, *pmp = nullptr, *pte = nullptr;
+    uint8_t *emb_rb = nullptr;                     // token_embd again as row-block tiles: the lm_head of 4..8-row blocks (lg_k_head_m)
     float *output_norm = nullptr, *rope_freqs = nullptr, *proj_norm = nullptr;
     std::vector<void *> allocs;
     std::map<std::pair<int, int>, float *> rope_tabs;      // (is_local, hd) -> table
@@ -157,7 +158,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -308,6 +309,13 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         std::vector<const uint8_t *> rows;
         push_rows(rows, t, 0, m->n_vocab);
         if ((rc = upload_tiled(m, rows, E, &m->emb, stage))) return rc;
+        // a second copy in the order the matrix-core lm_head reads (the first also serves the embedding lookup);
+        // it is not counted into weight_bytes, which says what a step streams
+        if (max_rows >= 4 && m->n_vocab % 64 == 0 && lg_segments(E) == 8 && !getenv("LG_HIP_NO_HEAD_MFMA")) {
+            const size_t wb = m->weight_bytes;
+            if ((rc = upload_tiled(m, rows, E, &m->emb_rb, stage, true))) return rc;
+            m->weight_bytes = wb;
+        }
     }
     if ((rc = upload_vec(m, "output_norm.weight", E, true, &m->output_norm))) return rc;
     int hd_global = 0;
@@ -883,12 +891,17 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         return lx.rc;
     } else
     if (with_head && !lx.rc) {
-        rows(m->output_norm, m->hidden_rows);
+        const bool head_m = M >= 4 && m->emb_rb && m->head_mfma;
+        rows(m->output_norm, m->hidden_rows, head_m ? 2 : 0);
         int grid = 512;                                  // two workgroups per CU, each walks `passes` blocks of 64 rows
         int passes = (m->n_vocab / 64 + grid - 1) / grid;
         if (passes < 1) passes = 1;
         grid = (m->n_vocab / 64 + passes - 1) / passes;
-        HeadArgs h{ m->emb, E, m->n_vocab, passes, m->hq, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
+        HeadArgs h{ head_m ? m->emb_rb : m->emb, E, m->n_vocab, passes, m->hq, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
+        if (head_m) {
+            if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS)
+                LAUNCH(KC_HEAD, (lg_k_head_m<M>), dim3(grid), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, h);
+        } else
         LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(grid), dim3(LG_WG), lds_mm(M, E), h);
         AcceptArgs c{ m->pval, m->pidx, grid, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
         LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), dim3(LG_WG), 0, c, m->ctl);
@@ -917,7 +930,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -949,6 +962,7 @@ static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int 
 extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     if (!m || !name) return fail(-1, "set_option: null argument");
     if (!strcmp(name, "store_logits")) m->store_logits = value != 0;
+    else if (!strcmp(name, "head_mfma")) m->head_mfma = value != 0;
     else if (!strcmp(name, "use_graph")) m->use_graph = value != 0;
     else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
@@ -1067,7 +1081,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s");
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
