@@ -786,7 +786,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
         int tiles = kv->tiles_max;
-        if (window > 0 && M <= LG_HIP_MAX_ROWS) { const int t = (window + M - 1 + 31) / 32 + 1; if (t < tiles) tiles = t; }
+        if (window > 0) { const int t = (window + M - 1 + 31) / 32 + 1; if (t < tiles) tiles = t; }
         return tiles;
     };
     auto rows_shared = [&](int L) {
