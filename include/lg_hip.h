@@ -167,6 +167,10 @@ int  lg_hip_launch_floor(int n_kernels, int mode, int grid, int block, int repla
  * of the matmul kernel alone. */
 int  lg_hip_matmul_q4q8(const void *w, int k, int m, const float *x, int rows, float *out,
                         int32_t *dots, int8_t *xq, float *xd, int32_t *xsum, int repeats, float *kernel_ms);
+/* Matmul against a matrix kept in f32 (the per-layer-embedding matrices of QAT conversions; the reference's int8
+ * backend multiplies such weights by the f32 activations unquantized, src/cuda/model-cuda-i8.cu:645-653, :846-895):
+ * w = m rows of k floats, x = rows x k floats, out = rows x m floats.  Any number of rows (8 per workgroup row). */
+int  lg_hip_matmul_f32w(const float *w, int k, int m, const float *x, int rows, float *out);
 /* Decode attention over an f16 ring (split_attn_kernel + combine_attn_kernel,
  * src/cuda/model-cuda.cuh:527-608) for a block of `rows` queries at pos..pos+rows-1:
  * q = rows x n_head x hd floats, already normed and rotated; kc/vc = seq rows of n_head_kv*hd

@@ -236,6 +236,46 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Matmul against a weight matrix kept in f32 (the per-layer-embedding matrices of QAT conversions, which the
+// reference's int8 backend also multiplies unquantized: src/cuda/model-cuda-i8.cu:645-653, :846-895; f16 and bf16
+// files are widened to f32 at upload, which is exact).  Activations are the f32 rows themselves.  One wavefront per
+// weight row and MC block rows (blockIdx.y: which MC rows of a wider block); order: lane (e/4)%64 takes element e,
+// fma in ascending e, adjacent-pair tree over the 64 lanes.  Optional epilogue of the per-layer gate:
+// out = gelu(sum) * ipl[row][i].
+struct MmfArgs {
+    const float *w; int k, m;                                 // [m][k], k a multiple of 256
+    const float *x; int ldx, rows;                            // [rows][ldx]
+    float *out; int ldo;                                      // [rows][ldo]
+    const float *ipl; int ipl_ld;                             // nullptr, or [rows][ipl_ld] (already at the layer's slice)
+};
+template <int MC>
+__global__ __launch_bounds__(LG_WG) void lg_k_mmf(MmfArgs a) {
+    const int lane = threadIdx.x & 63, i = blockIdx.x * (LG_WG / 64) + (threadIdx.x >> 6), j0 = blockIdx.y * MC;
+    if (i >= a.m) return;
+    const float4 *wr = (const float4 *)(a.w + (size_t)i * a.k);
+    float acc[MC];
+    #pragma unroll
+    for (int j = 0; j < MC; ++j) acc[j] = 0.0f;
+    for (int q = lane; q < (a.k >> 2); q += 64) {             // (k/4 is a multiple of 64: whole wavefronts)
+        const float4 w4 = wr[q];
+        #pragma unroll
+        for (int j = 0; j < MC; ++j) {
+            const int jj = j0 + j < a.rows ? j0 + j : a.rows - 1;             // past the block: the last row again, never stored
+            const float4 x4 = ((const float4 *)(a.x + (size_t)jj * a.ldx))[q];
+            acc[j] = lg_fmaf(w4.x, x4.x, acc[j]); acc[j] = lg_fmaf(w4.y, x4.y, acc[j]);
+            acc[j] = lg_fmaf(w4.z, x4.z, acc[j]); acc[j] = lg_fmaf(w4.w, x4.w, acc[j]);
+        }
+    }
+    #pragma unroll
+    for (int j = 0; j < MC; ++j) acc[j] = lg_wave_sum64(acc[j]);
+    if (lane < MC && j0 + lane < a.rows) {
+        float v = lg_pick<MC>(acc, lane);
+        if (a.ipl) v = lg_gelu(v) * a.ipl[(size_t)(j0 + lane) * a.ipl_ld + i];
+        a.out[(size_t)(j0 + lane) * a.ldo + i] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // lm_head for verify blocks of 4..8 rows on the matrix cores: lg_k_geglu_m's tile loop (row-block tiles of the
 // vocabulary matrix, a wavefront = 64 vocabulary rows x one of the 8 K segments, two v_mfma_i32_32x32x32_i8 per
 // tile whatever M is, the activations in the same 80-dword block order) with lg_k_mm_head's epilogue: the 8

@@ -113,6 +113,7 @@ struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; }
 
 struct Layer {
     uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
+    float *winp_f = nullptr, *wproj_f = nullptr;   // inp_gate / proj when the file keeps them in a float type (then winp / wproj are null)
     float *attn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *post_attn = nullptr, *ffn_norm = nullptr,
           *post_ffw = nullptr, *post_norm = nullptr, *out_scale = nullptr;
     int is_local = 0, hd = 0, nkv = 0, nff = 0, qd = 0, kd = 0, qkv_m = 0, k_off = 0, v_off = 0, owns = 0, src = 0;
@@ -143,6 +144,8 @@ struct lg_hip_model {
     // weights
     std::vector<Layer> L;
     uint8_t *emb = nullptr, *pmp = nullptr, *pte = nullptr;
+    float *pmp_f = nullptr;                        // per_layer_model_proj kept in a float type (then pmp is null)
+    float *pgf = nullptr;                          // [rows][ple] f32 gate output, input of a float-typed proj
     uint8_t *emb_rb = nullptr;                     // token_embd again as row-block tiles: the lm_head of 4..8-row blocks (lg_k_head_m)
     float *output_norm = nullptr, *rope_freqs = nullptr, *proj_norm = nullptr;
     std::vector<void *> allocs;
@@ -259,6 +262,29 @@ static int check_mat(const HostTensor *t, const std::string &name, uint64_t k, u
     if (k % 256 || mrows % 8) return fail(-6, "model_commit: %s needs row length %% 256 == 0 and rows %% 8 == 0", name.c_str());
     return 0;
 }
+// f32 / f16 / bf16 (ggml types 0 / 1 / 30): matrices a QAT conversion keeps at full precision
+static bool float_typed(const HostTensor *t) { return t && (t->type == 0 || t->type == 1 || t->type == 30); }
+static int upload_float_mat(lg_hip_model *m, const HostTensor *t, const std::string &name, uint64_t k, uint64_t mrows, float **out) {
+    if (t->dims[0] != k || t->dims[1] != mrows) return fail(-6, "model_commit: %s is %llu x %llu, expected %llu x %llu", name.c_str(),
+        (unsigned long long)t->dims[0], (unsigned long long)t->dims[1], (unsigned long long)k, (unsigned long long)mrows);
+    if (k % 256) return fail(-6, "model_commit: %s needs row length %% 256 == 0", name.c_str());
+    const size_t n = (size_t)k * mrows;
+    std::vector<float> wide;
+    const float *src = (const float *)t->data;
+    if (t->type != 0) {                                       // widening f16 / bf16 to f32 is exact
+        wide.resize(n);
+        const uint16_t *h = (const uint16_t *)t->data;
+        for (size_t i = 0; i < n; ++i) {
+            if (t->type == 1) wide[i] = lg_f16_to_f32(h[i]);
+            else { const uint32_t u = (uint32_t)h[i] << 16; memcpy(&wide[i], &u, 4); }
+        }
+        src = wide.data();
+    }
+    if (dev_alloc(m, out, n)) return -7;
+    HIP_TRY(hipMemcpy(*out, src, n * 4, hipMemcpyHostToDevice));
+    m->weight_bytes += n * 4;
+    return 0;
+}
 // upload a tiled matrix whose virtual rows are given by `rows`
 static int upload_tiled(lg_hip_model *m, const std::vector<const uint8_t *> &rows, int k, uint8_t **out,
                         std::vector<uint8_t> &stage, bool rowblocks = false) {
@@ -332,10 +358,14 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (dev_alloc(m, &m->pte, bytes)) return -7;
         HIP_TRY(hipMemcpy(m->pte, t->data, bytes, hipMemcpyHostToDevice));
         const HostTensor *p = find(m, "per_layer_model_proj.weight");
-        if ((rc = check_mat(p, "per_layer_model_proj.weight", E, total))) return rc;
-        std::vector<const uint8_t *> rows;
-        push_rows(rows, p, 0, total);
-        if ((rc = upload_tiled(m, rows, E, &m->pmp, stage))) return rc;
+        if (float_typed(p)) {
+            if ((rc = upload_float_mat(m, p, "per_layer_model_proj.weight", E, total, &m->pmp_f))) return rc;
+        } else {
+            if ((rc = check_mat(p, "per_layer_model_proj.weight", E, total))) return rc;
+            std::vector<const uint8_t *> rows;
+            push_rows(rows, p, 0, total);
+            if ((rc = upload_tiled(m, rows, E, &m->pmp, stage))) return rc;
+        }
         if ((rc = upload_vec(m, "per_layer_proj_norm.weight", m->ple, true, &m->proj_norm))) return rc;
     } else m->ple = 0;
 
@@ -395,6 +425,12 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (m->ple) {
             if (m->ple != 256) return fail(-2, "model_commit: per-layer width %d (256 is built)", m->ple);
             const HostTensor *ig = find(m, lname(L, "inp_gate.weight")), *pj = find(m, lname(L, "proj.weight"));
+            if (float_typed(ig) != float_typed(pj))
+                return fail(-6, "model_commit: blk.%d inp_gate and proj must both be q4_0 or both f32/f16/bf16", L);
+            if (float_typed(ig)) {
+                if ((rc = upload_float_mat(m, ig, lname(L, "inp_gate.weight"), E, m->ple, &y.winp_f))) return rc;
+                if ((rc = upload_float_mat(m, pj, lname(L, "proj.weight"), m->ple, E, &y.wproj_f))) return rc;
+            } else {
             if ((rc = check_mat(ig, lname(L, "inp_gate.weight"), E, m->ple))) return rc;
             if ((rc = check_mat(pj, lname(L, "proj.weight"), m->ple, E))) return rc;
             push_rows(rows, ig, 0, m->ple);
@@ -402,6 +438,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
             rows.clear();
             push_rows(rows, pj, 0, E);
             if ((rc = upload_tiled(m, rows, m->ple, &y.wproj, stage))) return rc;
+            }
             if ((rc = upload_vec(m, lname(L, "post_norm.weight"), E, true, &y.post_norm))) return rc;
         }
         if ((rc = upload_vec(m, lname(L, "attn_norm.weight"), E, true, &y.attn_norm))) return rc;
@@ -442,7 +479,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
         dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
-    if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4)))
+    if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
         return -7;
     HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
     HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
@@ -687,6 +724,12 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
 }
 
 // one block of M rows through the decoder (and the head when with_head)
+// f32-weight matmul of a block of M rows: one wavefront per weight row, 8 block rows per workgroup row
+template <int M>
+static void launch_mmf(Launcher &lx, int cls, const MmfArgs &a) {
+    constexpr int MC = M < 8 ? M : 8;
+    LAUNCH(cls, (lg_k_mmf<MC>), dim3((a.m + LG_WG / 64 - 1) / (LG_WG / 64), (a.rows + MC - 1) / MC), dim3(LG_WG), 0, a);
+}
 static bool attention_rows_shared(int rows, int tiles, int nkv, int hd, int seq) {
     return rows > 1 && rows <= LG_HIP_MAX_ROWS && hd <= 256 && seq >= 32 && tiles * nkv >= 256;
 }
@@ -774,8 +817,13 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
 
     if (m->ple) {
         rows(nullptr, nullptr);
+        if (m->pmp_f) {                                       // kept in a float type: the f32 rows themselves are the input
+            MmfArgs f{ m->pmp_f, E, m->ple * nl, m->x[cur], E, M, m->pmp_raw, m->ple * nl, nullptr, 0 };
+            launch_mmf<M>(lx, KC_PMP, f);
+        } else {
         MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, nullptr };
         launch_mm<M, false>(lx, KC_PMP, a);
+        }
         IplArgs i{ m->pmp_raw, m->ple, nl, M, m->proj_norm, m->pte, m->sched,
                    1.0f / sqrtf((float)E), sqrtf((float)m->ple), 1.0f / sqrtf(2.0f), m->eps };
         LAUNCH(KC_PMP, lg_k_ipl, dim3(nl, M), dim3(64), 0, i, m->ctl);
@@ -868,6 +916,15 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
             pend_parts = (M > LG_HIP_MAX_ROWS && lg_segments(y.nff) == 32) ? 4 : 1;
         }
+        if (m->ple && y.winp_f) {   // per-layer embedding block, matrices kept in a float type: residual update, then the
+            // gate on the f32 rows (gelu(.) * ipl in its epilogue), then the projection of the f32 gate rows
+            rows(nullptr, nullptr);
+            MmfArgs g{ y.winp_f, E, m->ple, m->x[cur], E, M, m->pgf, m->ple, m->pmp_raw + (size_t)L * m->ple, m->ple * nl };
+            launch_mmf<M>(lx, KC_PLEGATE, g);
+            MmfArgs p{ y.wproj_f, m->ple, E, m->pgf, m->ple, M, m->dout, E, nullptr, 0 };
+            launch_mmf<M>(lx, KC_PLEPROJ, p);
+            pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
+        } else
         if (m->ple) {   // per-layer embedding block
             PleGateArgs a{ y.winp, E, m->ple, m->hq, m->pmp_raw, L, nl, m->pq };
             if constexpr (M > LG_HIP_MAX_ROWS) {
@@ -1219,14 +1276,14 @@ extern "C" int lg_hip_schedule_time(lg_hip_model *m, lg_hip_kv *kv, int n_steps,
 static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int rows, double *b) {
     const double q = 18.0 / 32.0;                         // bytes per q4_0 weight
     for (int i = 0; i < KC_COUNT; ++i) b[i] = 0;
-    if (m->ple) b[KC_PMP] = (double)m->E * m->ple * m->n_layer * q;
+    if (m->ple) b[KC_PMP] = (double)m->E * m->ple * m->n_layer * (m->pmp_f ? 4.0 : q);
     for (int L = 0; L < m->n_layer; ++L) {
         const Layer &y = m->L[L];
         b[KC_QKV] += (double)m->E * y.qkv_m * q;
         b[KC_O] += (double)y.qd * m->E * q;
         b[KC_GATEUP] += 2.0 * m->E * y.nff * q;
         b[KC_DOWN] += (double)y.nff * m->E * q;
-        if (m->ple) { b[KC_PLEGATE] += (double)m->E * m->ple * q; b[KC_PLEPROJ] += (double)m->ple * m->E * q; }
+        if (m->ple) { const double pq = y.winp_f ? 4.0 : q; b[KC_PLEGATE] += (double)m->E * m->ple * pq; b[KC_PLEPROJ] += (double)m->ple * m->E * pq; }
         const int window = (y.is_local && m->window > 0) ? m->window : 0;
         const int last = pos + rows - 1, start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
         b[KC_ATTN] += 2.0 * (last - start + 1) * y.kd * 2.0;          // K and V rows, f16
@@ -1309,6 +1366,23 @@ static int matmul_rows(hipStream_t st, const uint8_t *dw, int k, int mrows, cons
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     return rc;
+}
+
+extern "C" int lg_hip_matmul_f32w(const float *w, int k, int mrows, const float *x, int rows, float *out) {
+    if (!w || !x || !out) return fail(-1, "matmul_f32w: null argument");
+    if (k < 256 || k % 256 || mrows < 1 || rows < 1) return fail(-2, "matmul_f32w: k %d (a multiple of 256), m %d, rows %d", k, mrows, rows);
+    if (lg_hip_device_count() < 1) return fail(-3, "matmul_f32w: no HIP device");
+    Scratch sc;
+    float *dw, *dx, *dout;
+    if (sc.get(&dw, (size_t)mrows * k) || sc.get(&dx, (size_t)rows * k) || sc.get(&dout, (size_t)rows * mrows)) return -7;
+    HIP_TRY(hipMemcpy(dw, w, (size_t)mrows * k * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dx, x, (size_t)rows * k * 4, hipMemcpyHostToDevice));
+    MmfArgs a{ dw, k, mrows, dx, k, rows, dout, mrows, nullptr, 0 };
+    hipLaunchKernelGGL((lg_k_mmf<8>), dim3((mrows + LG_WG / 64 - 1) / (LG_WG / 64), (rows + 7) / 8), dim3(LG_WG), 0, nullptr, a);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(out, dout, (size_t)rows * mrows * 4, hipMemcpyDeviceToHost));
+    return 0;
 }
 
 extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *x, int rows, float *out, int32_t *dots,

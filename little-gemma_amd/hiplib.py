@@ -59,6 +59,7 @@ def load_hip():
     L.lg_hip_repack_q4_0.argtypes = [u8p, C.c_int, C.c_int, u8p]
     L.lg_hip_matmul_q4q8.argtypes = [u8p, C.c_int, C.c_int, f32p, C.c_int] + [C.c_void_p] * 5 + [C.c_int, C.c_void_p]
     L.lg_hip_attention.argtypes = [f32p, u16p, u16p] + [C.c_int] * 7 + [f32p, C.c_int, C.c_void_p]
+    L.lg_hip_matmul_f32w.argtypes = [f32p, C.c_int, C.c_int, f32p, C.c_int, f32p]
     L.lg_hip_kv_layout.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
     L.lg_hip_kv_write.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
     L.lg_hip_kv_read.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
@@ -338,6 +339,16 @@ def matmul_q4q8(w_q4_0, k, m, x, want_dots=False, repeats=0):
     hip_check(H.lg_hip_matmul_q4q8(w, k, m, x, rows, _opt(out), _opt(dots), _opt(xq), _opt(xd), _opt(xsum),
                                    repeats, C.cast(C.byref(ms), C.c_void_p)), "matmul_q4q8")
     return dict(out=out, dots=dots, xq=xq, xd=xd, xsum=xsum, ms=ms.value)
+
+
+def matmul_f32w(w, x):
+    """Isolated f32-weight matmul through the C ABI.  w: [m, k] f32, x: [rows, k] f32 -> [rows, m]."""
+    H = load_hip()
+    w = np.ascontiguousarray(w, np.float32)
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.zeros((x.shape[0], w.shape[0]), np.float32)
+    hip_check(H.lg_hip_matmul_f32w(w, w.shape[1], w.shape[0], x, x.shape[0], out), "matmul_f32w")
+    return out
 
 
 def attention(q, kc, vc, n_head, n_head_kv, hd, window, pos, repeats=0):

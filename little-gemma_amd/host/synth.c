@@ -7,6 +7,7 @@
 #include "gguf.h"
 #include "quant.h"
 #include "synth.h"
+#include "../../include/lg_math.h"
 
 static uint64_t mix64(uint64_t z) {
     z += 0x9E3779B97F4A7C15ull;
@@ -56,6 +57,20 @@ static int add_layer(struct plan *p, int L, const char *leaf, uint32_t type, uin
 }
 
 static void fill(const struct planned *t, void *dst, float norm_jitter, float w_std) {
+    if (t->type != GGML_TYPE_Q4_0 && t->centre == 0.0f) {    /* a matrix kept in a float type: N(0, w_std) like the q4_0 ones */
+        const uint64_t n = t->cols * t->rows;
+        for (uint64_t i = 0; i < n; i += 2) {
+            float a, b;
+            normal_pair(t->key, i / 2, &a, &b);
+            const float v[2] = { a * w_std, b * w_std };
+            for (int e = 0; e < 2 && i + e < n; e++) {
+                if (t->type == GGML_TYPE_F32) ((float *)dst)[i + e] = v[e];
+                else if (t->type == GGML_TYPE_F16) ((uint16_t *)dst)[i + e] = lg_f32_to_f16(v[e]);
+                else { uint32_t u; memcpy(&u, &v[e], 4); ((uint16_t *)dst)[i + e] = (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16); }
+            }
+        }
+        return;
+    }
     if (t->type == GGML_TYPE_F32) {
         float *o = dst;
         for (uint64_t i = 0; i < t->cols * t->rows; i++)
@@ -120,12 +135,13 @@ int lg_synth_write(const char *path, const struct lg_synth_spec *s) {
     struct plan p = { w, NULL, 0, 0, s->seed };
     const uint64_t E = (uint64_t)s->n_embd, F = (uint64_t)s->n_ff, P = (uint64_t)s->ple;
     const int n_kv_start = s->n_layer - s->shared_kv_layers;
+    const uint32_t ple_t = s->ple_float == 1 ? GGML_TYPE_F32 : s->ple_float == 2 ? GGML_TYPE_F16 : s->ple_float == 3 ? GGML_TYPE_BF16 : GGML_TYPE_Q4_0;
     rc |= plan_add(&p, "token_embd.weight", GGML_TYPE_Q4_0, E, (uint64_t)s->n_vocab, 0);
     rc |= plan_add(&p, "output_norm.weight", GGML_TYPE_F32, E, 1, 1.0f);
     if (s->has_rope_freqs) rc |= plan_add(&p, "rope_freqs.weight", GGML_TYPE_F32, (uint64_t)hd_g / 2, 1, 1.0f);
     if (P) {
         rc |= plan_add(&p, "per_layer_token_embd.weight", GGML_TYPE_Q4_0, P * (uint64_t)s->n_layer, (uint64_t)s->n_vocab, 0);
-        rc |= plan_add(&p, "per_layer_model_proj.weight", GGML_TYPE_Q4_0, E, P * (uint64_t)s->n_layer, 0);
+        rc |= plan_add(&p, "per_layer_model_proj.weight", ple_t, E, P * (uint64_t)s->n_layer, 0);
         rc |= plan_add(&p, "per_layer_proj_norm.weight", GGML_TYPE_F32, P, 1, 1.0f);
     }
     for (int L = 0; L < s->n_layer && !rc; L++) {
@@ -148,8 +164,8 @@ int lg_synth_write(const char *path, const struct lg_synth_spec *s) {
         rc |= add_layer(&p, L, "ffn_down.weight", GGML_TYPE_Q4_0, F, E, 0);
         rc |= add_layer(&p, L, "post_ffw_norm.weight", GGML_TYPE_F32, E, 1, 1.0f);
         if (P) {
-            rc |= add_layer(&p, L, "inp_gate.weight", GGML_TYPE_Q4_0, E, P, 0);
-            rc |= add_layer(&p, L, "proj.weight", GGML_TYPE_Q4_0, P, E, 0);
+            rc |= add_layer(&p, L, "inp_gate.weight", ple_t, E, P, 0);
+            rc |= add_layer(&p, L, "proj.weight", ple_t, P, E, 0);
             rc |= add_layer(&p, L, "post_norm.weight", GGML_TYPE_F32, E, 1, 1.0f);
         }
         if (s->out_scale > 0) rc |= add_layer(&p, L, "layer_output_scale.weight", GGML_TYPE_F32, 1, 1, s->out_scale);

@@ -21,6 +21,8 @@ struct lg_synth_spec {
     int32_t shared_kv_layers;  /* trailing layers that reuse an earlier layer's KV (their k/v tensors are omitted) */
     int32_t has_v;             /* 0: no attn_v tensors (V = un-normed K projection) */
     int32_t has_rope_freqs;
+    int32_t ple_float;         /* type of per_layer_model_proj / inp_gate / proj: 0 = q4_0, 1 = f32, 2 = f16, 3 = bf16 (what
+                                  QAT conversions keep at full precision, src/cuda/model-cuda-i8.cu:645-653) */
     float   w_std;             /* std of every matrix before q4_0 packing */
     float   qk_norm;           /* centre of attn_q_norm / attn_k_norm weights; 0 = sqrt(1.28/sqrt(head_dim)) */
     float   norm_jitter;       /* norm weights are centre * (1 + jitter*u), u uniform in [-1,1) */

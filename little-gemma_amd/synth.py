@@ -9,13 +9,13 @@ from . import hostlib
 class SynthSpec(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "n_layer", "n_embd", "n_head", "n_head_kv", "head_dim", "head_dim_full", "n_ff", "n_vocab",
-        "n_ctx", "sliding_window", "local_period", "ple", "shared_kv_layers", "has_v", "has_rope_freqs")] + [
+        "n_ctx", "sliding_window", "local_period", "ple", "shared_kv_layers", "has_v", "has_rope_freqs", "ple_float")] + [
         (n, C.c_float) for n in ("w_std", "qk_norm", "norm_jitter", "out_scale", "rms_eps", "rope_base",
                                  "rope_base_swa", "softcap")] + [("seed", C.c_uint64)]
 
 
 DEFAULTS = dict(head_dim_full=0, n_ctx=8192, sliding_window=512, local_period=6, ple=0, shared_kv_layers=0,
-                has_v=1, has_rope_freqs=1, w_std=0.02, qk_norm=0.0, norm_jitter=0.1, out_scale=0.0,
+                has_v=1, has_rope_freqs=1, ple_float=0, w_std=0.02, qk_norm=0.0, norm_jitter=0.1, out_scale=0.0,
                 rms_eps=1e-6, rope_base=1e6, rope_base_swa=1e4, softcap=30.0, seed=1234)
 
 # 4 layers, d 512, 8 x 64 heads, 2 KV heads, FFN 2048, vocab 8192, sliding-128 / global alternating
@@ -23,6 +23,10 @@ TINY = dict(DEFAULTS, n_layer=4, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
             sliding_window=128, local_period=2, qk_norm=0.7)
 # the same with every optional piece switched on: PLE, shared-KV tail, V-less layers, output scale
 TINY_FULL = dict(TINY, n_layer=6, ple=256, shared_kv_layers=2, has_v=0, out_scale=0.9, head_dim_full=128)
+# ... and with the per-layer-embedding matrices kept in a float type, as QAT conversions of E4B store them
+TINY_FULL_F32 = dict(TINY_FULL, ple_float=1)
+TINY_FULL_F16 = dict(TINY_FULL, ple_float=2)
+TINY_FULL_BF16 = dict(TINY_FULL, ple_float=3)
 # E4B shape: 42 layers, d 2560, 8/2 heads x 256, FFN 10240, PLE 256, vocab 262144; 5 sliding(512) : 1 global
 E4B = dict(DEFAULTS, n_layer=42, n_embd=2560, n_head=8, n_head_kv=2, head_dim=256, n_ff=10240, n_vocab=262144,
            ple=256, sliding_window=512, local_period=6, out_scale=1.0)

@@ -43,6 +43,7 @@ def lib():
     L.lgo_block_dot.restype = C.c_int32
     L.lgo_matmul_q4q8.argtypes = [c_u8p, C.c_int, C.c_int, c_i8p, c_f32p, C.c_int, c_f32p, C.c_void_p, C.c_int]
     L.lgo_matmul_f32.argtypes = [c_u8p, C.c_uint32, C.c_int, C.c_int, c_f32p, c_f32p]
+    L.lgo_matmul_fw.argtypes = [c_u8p, C.c_uint32, C.c_int, C.c_int, c_f32p, c_f32p]
     L.lgo_rmsnorm.argtypes = [c_f32p, c_f32p, C.c_void_p, C.c_int, C.c_float, C.c_int]
     L.lgo_rope.argtypes = [c_f32p, C.c_int, C.c_int, c_f32p, C.c_void_p, C.c_int]
     L.lgo_attention_f16.argtypes = [c_f32p, c_f32p, c_u16p, c_u16p] + [C.c_int] * 8

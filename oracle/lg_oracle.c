@@ -6,6 +6,10 @@
  *                                  fixture produced by the reference's dequantize_into (test_oracle_primitives)
  *   lgo_quant_q8                   numpy restatement with ties-to-even, zero group, saturating cases
  *   lgo_matmul_q4q8                float64 accumulation of d_w*d_x*dot within 1e-5; both orders agree
+ *   lgo_matmul_fw                  f32/f16/bf16 weight rows: float64 product within 1e-6 of the sum of magnitudes, unit
+ *                                  rows and small-integer operands exactly, the serial-order matmul within rounding
+ *                                  (test_oracle_primitives); models whose per-layer-embedding matrices are float-typed:
+ *                                  LGO_REF bit-identical to the reference build and its fixture, LGO_I8_F32 within 1e-3
  *   lgo_f32_to_f16 / f16_to_f32    numpy float16 over dense samples incl. subnormals, ties, overflow
  *   lgo_expf/tanhf/sincosf/gelu    double-precision libm within a few ulp (test_lg_math)
  *   lgo_rmsnorm, lgo_rope          float64 closed forms
@@ -156,6 +160,27 @@ void lgo_matmul_f32(const void *w, uint32_t type, int k, int m, const float *x, 
             float s = 0.0f;
             for (int j = 0; j < k; j++) s += buf[j] * x[j];
             out[i] = s;
+        }
+        free(buf);
+    }
+}
+
+/* ---- matmul against a weight matrix kept in a float type (f32 / f16 / bf16), f32 activations: what the int8
+ * backend does for the per-layer-embedding matrices of QAT conversions, which stay at full precision
+ * (src/cuda/model-cuda-i8.cu:645-653, :846-895: w * x summed per lane, then a lane tree; nothing is quantized).
+ * This build's order: 64 lane partials, element e belongs to lane (e/4)%64, fma in ascending e, adjacent-pair tree
+ * over the lanes. */
+void lgo_matmul_fw(const void *w, uint32_t type, int k, int m, const float *x, float *out) {
+    const size_t row_bytes = (size_t)(k / ggml_blck_size(type)) * ggml_type_size(type);
+    #pragma omp parallel
+    {
+        float *buf = malloc((size_t)k * sizeof(float));
+        #pragma omp for schedule(static)
+        for (int i = 0; i < m; i++) {
+            dequantize_into(type, (const unsigned char *)w + (size_t)i * row_bytes, buf, k);
+            float lane[64] = { 0 };
+            for (int e = 0; e < k; e++) lane[(e >> 2) & 63] = lg_fmaf(buf[e], x[e], lane[(e >> 2) & 63]);
+            out[i] = tree_sum(lane, 64);
         }
         free(buf);
     }
@@ -577,12 +602,14 @@ struct qact { int8_t *q; float *d; float *f; int noq; };
 /* noq: the quantization is switched off and the matmul takes the f32 vector itself (LGO_I8_F32): the same op
  * sequence, norm / attention orders and elementary functions, without the int8 rounding of the activations */
 static void quant_into(struct qact *a, const float *x, int n) {
-    if (a->noq) memcpy(a->f, x, (size_t)n * 4);
-    else lgo_quant_q8(x, n, a->q, a->d, NULL);
+    memcpy(a->f, x, (size_t)n * 4);                          /* (a float-typed weight takes the vector itself) */
+    if (!a->noq) lgo_quant_q8(x, n, a->q, a->d, NULL);
 }
+static int float_typed(uint32_t t) { return t == GGML_TYPE_F32 || t == GGML_TYPE_F16 || t == GGML_TYPE_BF16; }
 static void mm(const struct gguf_tensor *w, int k, int mrows, const struct qact *a, float *out) {
-    if (w->type != GGML_TYPE_Q4_0) { fprintf(stderr, "oracle: matmul weight %s is %s, only q4_0 is on the int8 path\n", w->name, ggml_type_name(w->type)); abort(); }
+    if (w->type != GGML_TYPE_Q4_0 && !float_typed(w->type)) { fprintf(stderr, "oracle: matmul weight %s is %s; the int8 path takes q4_0 and f32/f16/bf16\n", w->name, ggml_type_name(w->type)); abort(); }
     if (a->noq) lgo_matmul_f32(w->data, w->type, k, mrows, a->f, out);
+    else if (float_typed(w->type)) lgo_matmul_fw(w->data, w->type, k, mrows, a->f, out);
     else lgo_matmul_q4q8(w->data, k, mrows, a->q, a->d, 1, out, NULL, LGO_ORDER_SEG);
 }
 

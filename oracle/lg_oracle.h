@@ -39,6 +39,8 @@ int32_t lgo_block_dot(const unsigned char *block18, const int8_t *q32);
 void    lgo_matmul_q4q8(const void *w, int k, int m, const int8_t *xq, const float *xd, int rows,
                         float *out, int32_t *dots, int order);
 void    lgo_matmul_f32(const void *w, uint32_t ggml_type, int k, int m, const float *x, float *out);
+/* f32 / f16 / bf16 weights x f32 activations in this build's order: lane (e/4)%64 partials, fma ascending, pair tree */
+void    lgo_matmul_fw(const void *w, uint32_t ggml_type, int k, int m, const float *x, float *out);
 void    lgo_rmsnorm(float *out, const float *x, const float *w, int n, float eps, int tree);
 void    lgo_rope(float *v, int d, int pos, const float *freq_tab, const float *ff, int exact);
 /* one (query head) attention over an f16 ring: keys start..pos, row of position p = p % seq */

@@ -29,6 +29,8 @@ lg = importlib.import_module("little-gemma_amd")
 from oracle import binding as ob  # noqa: E402
 
 MODELS = {"tiny": lg.synth.TINY, "tiny_full": lg.synth.TINY_FULL}
+# the same with the per-layer-embedding matrices kept f32 (model fixtures only: a draft head never reads them)
+FLOAT_PLE_MODELS = {"tiny_full_f32": lg.synth.TINY_FULL_F32}
 N_PROMPT, N_GEN, LOGIT_STEPS = 128, 64, (0, 1, 31, 63)
 
 
@@ -51,7 +53,7 @@ def main():
     assert R.ref_dequantize(2, blocks.reshape(-1), out, 64 * 32) == 0
     np.savez_compressed(os.path.join(HERE, "q4_0_dequant.npz"), blocks=blocks, values=out.reshape(64, 32))
 
-    for name, spec in MODELS.items():
+    for name, spec in {**MODELS, **FLOAT_PLE_MODELS}.items():
         path = f"/tmp/lg_golden_{name}.gguf"
         lg.synth.write_model(path, **spec)
         ref = ob.Reference(path, 4)

@@ -60,6 +60,23 @@ def test_matmul_edge_shapes(lg, ob, gpu_required, m, k, rows):
     assert np.all(np.isfinite(r["out"]))
 
 
+@pytest.mark.parametrize("m,k,rows", [(256, 2560, 5), (2560, 256, 8), (10, 512, 1), (77, 1024, 21)])
+def test_matmul_float_weights_matches_oracle(lg, ob, gpu_required, m, k, rows):
+    """f32 weight matrix x f32 rows (what a float-typed per-layer-embedding matrix goes through): bit-identical to
+    the oracle's order for every row of the block, ragged row counts and row groups included."""
+    rng = np.random.default_rng(m * 7 + k + rows)
+    w = rng.normal(0, 0.02, (m, k)).astype(np.float32)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[0, :64] = 0.0
+    print(f"matmul_f32w m={m} k={k} rows={rows}", flush=True)
+    got = lg.hiplib.matmul_f32w(w, x)
+    L = ob.lib()
+    for j in range(rows):
+        want = np.zeros(m, np.float32)
+        L.lgo_matmul_fw(w.view(np.uint8).reshape(-1), 0, k, m, np.ascontiguousarray(x[j]), want)
+        assert np.array_equal(got[j].view(np.uint32), want.view(np.uint32)), f"row {j}"
+
+
 def test_matmul_is_linear_in_the_scales(lg, gpu_required):
     """Size-independent property: doubling every weight scale doubles every output exactly
     (powers of two commute with rounding), negating codes around 8 negates it."""

@@ -18,7 +18,7 @@ def greedy_oracle(ob, o, prompt, n_gen, max_seq):
     return toks, logits, kv
 
 
-@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+@pytest.mark.parametrize("name", ["tiny", "tiny_full", "tiny_full_f32"])
 def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, golden, name):
     """BASELINE config 1: 128-token uniform-random prompt, then 64 greedy tokens, against the int8-class oracle.
     The prompt is the one of the committed reference fixture; the comparison with the reference's own f32 run
@@ -95,7 +95,7 @@ def test_gpu_against_the_reference_fixture_teacher_forced(lg, ob, gpu_required, 
         gpu.close(); o.close()
 
 
-@pytest.mark.parametrize("name,rows,over", [("tiny", 2, {}), ("tiny", 4, {}), ("tiny", 5, {}), ("tiny_full", 3, {}), ("tiny_full", 4, {}),
+@pytest.mark.parametrize("name,rows,over", [("tiny", 2, {}), ("tiny", 4, {}), ("tiny", 5, {}), ("tiny_full", 3, {}), ("tiny_full", 4, {}), ("tiny_full_f32", 5, {}), ("tiny_full_f16", 2, {}), ("tiny_full_bf16", 8, {}),
                                             ("tiny_full", 6, {}), ("tiny_full", 7, {}), ("tiny_full", 8, {}),
                                             ("tiny", 5, {"head_dim_full": 512}), ("tiny_full", 8, {"head_dim_full": 256})])
 def test_verify_equals_decode_and_accept_counts(lg, ob, gpu_required, model_path, name, rows, over):

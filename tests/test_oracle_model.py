@@ -6,7 +6,7 @@ import pytest
 N_PROMPT, N_GEN = 128, 64
 
 
-@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+@pytest.mark.parametrize("name", ["tiny", "tiny_full", "tiny_full_f32"])
 def test_ref_mode_reproduces_reference_fixture(ob, model_path, golden, name):
     """Greedy tokens, logits rows and last_hidden recorded from the reference's `run` path
     (model_prefill + model_forward; tests/golden/make_fixtures.py) — bit for bit."""
@@ -39,7 +39,10 @@ def test_ref_mode_reproduces_reference_fixture(ob, model_path, golden, name):
         o.close()
 
 
-@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+FLOAT_PLE = ["tiny_full_f32", "tiny_full_f16", "tiny_full_bf16"]   # per-layer-embedding matrices kept in a float type
+
+
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"] + FLOAT_PLE)
 def test_ref_mode_against_live_reference(ob, model_path, name):
     if not ob.ref_available(4):
         pytest.skip("reference build absent (needs /root/reference; run make -C oracle ref)")
@@ -64,7 +67,7 @@ def test_ref_mode_against_live_reference(ob, model_path, name):
         o.close(); r.close()
 
 
-@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"] + FLOAT_PLE)
 def test_int8_class_stays_in_the_q8_noise_band_of_ref(ob, model_path, name):
     """The int8-class forward is the same network with q8 activations: teacher-forced on the REF
     tokens its logits stay within a few 1e-2 relative L2 of REF at every step.  A dropped residual,
@@ -95,7 +98,7 @@ def test_int8_class_stays_in_the_q8_noise_band_of_ref(ob, model_path, name):
         o.close()
 
 
-@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"] + FLOAT_PLE)
 def test_f32_variant_of_the_int8_sequence_matches_ref_to_reorder_noise(ob, model_path, name):
     """I8_F32 runs forward_i8's exact op sequence (quantization points, PLE build, residual and scale placement,
     tile attention, this build's norm orders and elementary functions) with the quantization switched off and

@@ -98,6 +98,37 @@ def test_matmul_q4q8_against_float64(ob, m, k, rows):
     assert np.abs(ref - outs[ob.ORDER_SEG][0]).max() <= 1e-4 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("gtype,k,m", [(0, 2560, 48), (1, 256, 40), (30, 512, 33), (0, 256, 8)])
+def test_matmul_float_weights_against_float64(ob, gtype, k, m):
+    """f32 / f16 / bf16 weight rows x one f32 vector: within reorder noise of float64, exact where the arithmetic
+    is exact (unit rows pick an element, small integers sum exactly in any order), and the same value as the
+    serial-order matmul up to rounding (a transposed or mis-strided operand fails all three)."""
+    rng = np.random.default_rng(gtype + k + m)
+    L = ob.lib()
+    wf = rng.normal(0, 0.02, (m, k)).astype(np.float32)
+    wf[0] = 0.0; wf[0, k - 3] = 1.0                                   # unit row: out = x[k-3] exactly
+    wf[1] = rng.integers(-4, 5, k).astype(np.float32)                 # small integers x small integers: exact
+    if gtype == 1:
+        raw = wf.astype(np.float16); wf = raw.astype(np.float32); raw = raw.view(np.uint16)
+    elif gtype == 30:
+        raw = (wf.view(np.uint32) >> 16).astype(np.uint16); wf = (raw.astype(np.uint32) << 16).view(np.float32)
+    else:
+        raw = wf
+    x = rng.normal(0, 1, k).astype(np.float32)
+    xi = rng.integers(-8, 9, k).astype(np.float32)
+    out = np.zeros(m, np.float32); outi = np.zeros(m, np.float32); ser = np.zeros(m, np.float32)
+    wb = np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
+    L.lgo_matmul_fw(wb, gtype, k, m, x, out)
+    L.lgo_matmul_fw(wb, gtype, k, m, xi, outi)
+    L.lgo_matmul_f32(wb, gtype, k, m, x, ser)
+    want = wf.astype(np.float64) @ x.astype(np.float64)
+    mag = np.abs(wf).astype(np.float64) @ np.abs(x).astype(np.float64)   # rounding scales with the sum of magnitudes
+    assert np.all(np.abs(out - want) <= 1e-6 * mag + 1e-12)
+    assert np.all(np.abs(out - ser) <= 2e-6 * mag + 1e-12)
+    assert out[0] == x[k - 3]
+    assert outi[1] == np.float32(wf[1].astype(np.float64) @ xi.astype(np.float64))
+
+
 def test_rmsnorm_both_orders(ob):
     rng = np.random.default_rng(6)
     L = ob.lib()
