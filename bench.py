@@ -365,7 +365,7 @@ def main():
         dt = time.time() - t0
         macs = sum(c["bytes"] for c in prof if c["name"] != "lm_head" and c["name"] != "attn_tiles") / (18.0 / 32.0)   # weights touched per position
         line["prefill"] = {"positions": int(a.prefill), "ms": 1e3 * dt, "tok_per_s": a.prefill / dt,
-                           "kernel": "v_mfma_i32_32x32x32_i8, 128-row blocks", "int8_TOPs": 2.0 * macs * a.prefill / dt / 1e12,
+                           "kernel": "v_mfma_i32_32x32x32_i8, 512-row blocks", "int8_TOPs": 2.0 * macs * a.prefill / dt / 1e12,
                            "mfma_peak_TOPs": 5000.0, "mfma_utilisation": 2.0 * macs * a.prefill / dt / 5.0e15}
     gpu.close()
     try:

@@ -80,9 +80,10 @@ int  lg_hip_kv_restore_prefix(lg_hip_kv *kv, int n);
 int  lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n_rows, int pos,
                          int32_t *out, int32_t *adv);
 /* model_prefill (include/model.h:121): positions pos0..pos0+n-1, cache writes only, no head.
- * Runs as blocks of 128 rows whose matmuls use the int8 matrix cores (the reference's chunked
- * prefill, src/cuda/prefill-kernel.cuh:631-675), then one 32-row block, then verify-width blocks
- * for the tail; every block leaves the cache rows that position-by-position decode would. */
+ * Runs as blocks of 512 rows (128 when the cache holds fewer than 1024 positions) whose matmuls use the int8
+ * matrix cores (the reference's chunked prefill, src/cuda/prefill-kernel.cuh:631-675), then 128- and 32-row
+ * blocks, then verify-width blocks for the tail; every block leaves the cache rows that position-by-position
+ * decode would. */
 int  lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int pos0);
 /* Post-output-norm hidden state of the last valid row of the latest verify step (n_embd
  * floats): what the reference keeps in g_hidden / model.last_hidden for the draft head

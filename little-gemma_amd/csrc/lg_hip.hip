@@ -39,8 +39,11 @@ extern "C" int lg_hip_device_count(void) {
     if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
     return n;
 }
+// The widest prompt block a cache of max_seq positions takes: LG_WIDE_ROWS for caches of 1024 positions and more,
+// LG_WIDE_MID below (a short cache does not pay 512 spare rows per sliding ring and 512 rows of attention partials)
+static int wide_rows_for(int max_seq) { return max_seq >= 1024 ? LG_WIDE_ROWS : LG_WIDE_MID; }
 extern "C" int lg_hip_ring_rows(int window, int max_seq) {
-    int r = (window + LG_WIDE_ROWS + 31) / 32 * 32;   // window + spare for the widest block written before its queries run, tile multiple
+    int r = (window + wide_rows_for(max_seq) + 31) / 32 * 32;   // window + spare for the widest block written before its queries run, tile multiple
     return r < max_seq ? r : max_seq;
 }
 
@@ -175,7 +178,7 @@ struct lg_hip_model {
 
 struct lg_hip_kv {
     lg_hip_model *m = nullptr;
-    int max_seq = 0, tiles_max = 0;
+    int max_seq = 0, tiles_max = 0, wide_rows = 0;      // wide_rows: the widest prompt block (sliding rings and partials are sized for it)
     std::vector<int> seq, kv_dim;
     std::vector<uint16_t *> k, v, px_k, px_v;
     float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
@@ -487,7 +490,8 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
     if (dev_alloc(m, &m->sched, (size_t)m->sched_cap * LG_HIP_MAX_ROWS + LG_WIDE_ROWS) || dev_alloc(m, &m->out, (size_t)m->sched_cap * LG_HIP_MAX_ROWS) ||
         dev_alloc(m, &m->adv, (size_t)m->sched_cap))
         return -7;
-    HIP_TRY(hipHostMalloc((void **)&m->pin, 256 * sizeof(int32_t), hipHostMallocDefault));
+    // pinned staging: step state at 0, a verify block's successors at 32 and accept count at 48, a block's tokens from 64
+    HIP_TRY(hipHostMalloc((void **)&m->pin, (64 + LG_WIDE_ROWS) * sizeof(int32_t), hipHostMallocDefault));
     HIP_TRY(hipDeviceSynchronize());
     m->committed = true;
     return 0;
@@ -516,7 +520,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
     if (max_seq < 1) return fail(-2, "kv_create: max_seq %d", max_seq);
     HIP_TRY(hipSetDevice(m->device));
     lg_hip_kv *kv = new lg_hip_kv();
-    kv->m = m; kv->max_seq = max_seq; kv->id = ++g_kv_ids;
+    kv->m = m; kv->max_seq = max_seq; kv->id = ++g_kv_ids; kv->wide_rows = wide_rows_for(max_seq);
     const int nl = m->n_layer;
     kv->seq.assign(nl, 0); kv->kv_dim.assign(nl, 0);
     kv->k.assign(nl, nullptr); kv->v.assign(nl, nullptr); kv->px_k.assign(nl, nullptr); kv->px_v.assign(nl, nullptr);
@@ -526,7 +530,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         kv->kv_dim[L] = y.kd;
         if (y.hd > max_hd) max_hd = y.hd;
         const bool ring = y.is_local && m->window > 0;
-        const int span = ring ? m->window + LG_WIDE_ROWS : max_seq;                 // keys any block can touch
+        const int span = ring ? m->window + kv->wide_rows : max_seq;                // keys any block can touch
         int t = (span < max_seq ? span : max_seq) / 32 + 2;
         if (t > tiles) tiles = t;
         if (!y.owns) continue;
@@ -537,7 +541,7 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
         (void)hipMemset(kv->k[L], 0, bytes); (void)hipMemset(kv->v[L], 0, bytes);
     }
     kv->tiles_max = tiles;
-    const size_t slots = (size_t)(m->max_rows > LG_WIDE_ROWS ? m->max_rows : LG_WIDE_ROWS) * m->H * tiles;
+    const size_t slots = (size_t)(m->max_rows > kv->wide_rows ? m->max_rows : kv->wide_rows) * m->H * tiles;
     if (hipMalloc((void **)&kv->pm, slots * 4) != hipSuccess || hipMalloc((void **)&kv->pl, slots * 4) != hipSuccess ||
         hipMalloc((void **)&kv->pacc, slots * max_hd * 4) != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory for attention partials"); }
     HIP_TRY(hipDeviceSynchronize());
@@ -979,6 +983,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
         case 7: return enqueue_step<7>(m, kv, with_head, dry);
         case 8: return enqueue_step<8>(m, kv, with_head, dry);
         case LG_WIDE: return enqueue_step<LG_WIDE>(m, kv, with_head, dry);
+        case LG_WIDE_MID: return enqueue_step<LG_WIDE_MID>(m, kv, with_head, dry);
         case LG_WIDE_ROWS: return enqueue_step<LG_WIDE_ROWS>(m, kv, with_head, dry);
     }
     return fail(-2, "rows %d outside 1..%d", rows, LG_HIP_MAX_ROWS);
@@ -1010,7 +1015,7 @@ static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head)
 
 static int check_block(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, int n, int rows, int pos, bool wide = false) {
     if (!m || !kv || !toks || kv->m != m) return fail(-1, "bad model / cache / token pointer");
-    if (rows < 1 || (rows > m->max_rows && !(wide && (rows == LG_WIDE || rows == LG_WIDE_ROWS)))) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
+    if (rows < 1 || (rows > m->max_rows && !(wide && (rows == LG_WIDE || rows == LG_WIDE_MID || rows == LG_WIDE_ROWS)))) return fail(-2, "block of %d rows; the model was committed for 1..%d", rows, m->max_rows);
     if (pos < 0 || pos + rows > kv->max_seq) return fail(-2, "positions %d..%d do not fit a cache of %d", pos, pos + rows - 1, kv->max_seq);
     for (int i = 0; i < n; ++i) if (toks[i] < 0 || toks[i] >= m->n_vocab) return fail(-2, "token id %d outside the vocabulary of %d", toks[i], m->n_vocab);
     return 0;
@@ -1031,9 +1036,9 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
 static int load_block(lg_hip_model *m, const int32_t *toks, int rows, int pos) {
     StepCtl c{ pos, 0, 0, 0 };
     memcpy(m->pin, &c, sizeof c);
-    memcpy(m->pin + 8, toks, (size_t)rows * 4);
+    memcpy(m->pin + 64, toks, (size_t)rows * 4);
     HIP_TRY(hipMemcpyAsync(m->ctl, m->pin, sizeof c, hipMemcpyHostToDevice, m->stream));
-    HIP_TRY(hipMemcpyAsync(m->sched, m->pin + 8, (size_t)rows * 4, hipMemcpyHostToDevice, m->stream));
+    HIP_TRY(hipMemcpyAsync(m->sched, m->pin + 64, (size_t)rows * 4, hipMemcpyHostToDevice, m->stream));
     return 0;
 }
 
@@ -1181,7 +1186,8 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
     }
     for (int done = 0; done < n;) {
         int rows = n - done < m->max_rows ? n - done : m->max_rows;
-        if (wide_ok && n - done >= LG_WIDE_ROWS) rows = LG_WIDE_ROWS;     // matrix-core blocks while the prompt lasts,
+        if (wide_ok && n - done >= LG_WIDE_ROWS && kv->wide_rows >= LG_WIDE_ROWS) rows = LG_WIDE_ROWS;     // matrix-core blocks while the prompt lasts,
+        else if (wide_ok && n - done >= LG_WIDE_MID) rows = LG_WIDE_MID;
         else if (wide_ok && n - done >= LG_WIDE) rows = LG_WIDE;        // a single row tile, then verify-width blocks for the tail
         int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done, true);
         if (rc) return rc;

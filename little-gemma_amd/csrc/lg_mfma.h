@@ -28,7 +28,8 @@ typedef int lg_v4i __attribute__((ext_vector_type(4)));
 typedef int lg_v16i __attribute__((ext_vector_type(16)));
 
 #define LG_WIDE 32                         // activation rows per row tile (one MFMA operand)
-#define LG_WIDE_ROWS 128                   // rows of a wide block: four row tiles share every launch
+#define LG_WIDE_ROWS 512                   // rows of the widest block: its 16 row tiles share every launch (and every weight tile's trip through L2)
+#define LG_WIDE_MID 128                    // the block between that and a single row tile, for prompts and remainders below 512
 
 #define LG_WIDE_WG 512                     // 8 wavefronts: two per SIMD, one K segment each
 

@@ -305,11 +305,12 @@ int lgo_accept(const int *toks, const int *out, int rows) {
     return adv;
 }
 
-/* sliding-window ring length of the int8 class: the window plus spare rows for the widest block
- * (128 prompt rows, or a few draft rows) written before any of its queries runs (src/cuda/model-cuda.cuh:1016-1035 uses
- * window + widest chunk), rounded to the 32-key attention tile */
+/* sliding-window ring length of the int8 class: the window plus spare rows for the widest block written before any
+ * of its queries runs (512 prompt rows for caches of 1024 positions and more, 128 below; src/cuda/model-cuda.cuh:1016-1035
+ * uses window + widest chunk), rounded to the 32-key attention tile.  A layout choice, not arithmetic: results do not
+ * depend on it; it is restated here so that cache rows can be compared ring row by ring row. */
 int lgo_ring_rows(int window, int max_seq) {
-    int r = (window + 128 + 31) / 32 * 32;
+    int r = (window + (max_seq >= 1024 ? 512 : 128) + 31) / 32 * 32;
     return r < max_seq ? r : max_seq;
 }
 

@@ -28,9 +28,11 @@ def test_wide_matmul_matches_oracle(lg, ob, gpu_required, m, k):
     assert np.array_equal(r["out"].view(np.uint32), out.view(np.uint32))
 
 
-@pytest.mark.parametrize("name,n_prompt", [("tiny", 97), ("tiny_full", 200), ("tiny", 32), ("tiny_full", 427), ("tiny", 128), ("tiny_full_f32", 200), ("tiny_full_f16", 171)])
+@pytest.mark.parametrize("name,n_prompt", [("tiny", 97), ("tiny_full", 200), ("tiny", 32), ("tiny_full", 427), ("tiny", 128), ("tiny_full_f32", 200), ("tiny_full_f16", 171),
+                                           ("tiny", 1100), ("tiny_full", 1061)])
 def test_wide_prefill_leaves_the_same_cache_and_logits(lg, ob, gpu_required, model_path, name, n_prompt):
-    """A prompt through 128-row blocks, 32-row blocks and a verify-width tail against one oracle forward per position:
+    """A prompt through 512-row blocks (caches of 1024 positions and more; the two long prompts also wrap the
+    640-row sliding rings), 128-row blocks, 32-row blocks and a verify-width tail against one oracle forward per position:
     every cache row identical, the logits of the next position identical; and identical to the same
     prompt pushed through 8-row blocks only."""
     path, spec = model_path(name)

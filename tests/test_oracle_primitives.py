@@ -220,7 +220,8 @@ def test_accept_rule_exhaustive(ob):
 
 def test_ring_rows(ob):
     L = ob.lib()
-    assert L.lgo_ring_rows(128, 4096) == 256 and L.lgo_ring_rows(512, 4096) == 640 and L.lgo_ring_rows(1024, 9000) == 1152
+    assert L.lgo_ring_rows(128, 4096) == 640 and L.lgo_ring_rows(512, 4096) == 1024 and L.lgo_ring_rows(1024, 9000) == 1536
+    assert L.lgo_ring_rows(128, 400) == 256 and L.lgo_ring_rows(512, 1000) == 640     # short caches: 128 spare rows
     assert L.lgo_ring_rows(512, 300) == 300                     # never more rows than positions
     for w in (100, 128, 511, 512, 1000):
         assert L.lgo_ring_rows(w, 1 << 20) % 32 == 0 and L.lgo_ring_rows(w, 1 << 20) >= w + 128 - 1
