@@ -586,6 +586,174 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(AttnArgs a, const StepCt
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Attention tiles of prompt blocks with the queries in registers: a workgroup is 8 (row, head) units (two rows x four
+// heads, four x two, ...), a wavefront IS a unit.
+// In the score phase lane (k, c) = key k of 16, chain c of the 4, holds the unit's query elements of its chain
+// (q[4g+c], g = 0..hd/4-1: hd/4 registers, loaded once per workgroup) and reads its key's elements of that chain from
+// a K tile staged chain-major, 16 bytes = 8 steps of the chain at a time: no LDS traffic for the queries at all, where
+// lg_k_attn and lg_k_attn_rows fetch a query element per fma from LDS and are bound by that.  The two 16-key
+// halves of a tile run as two independent chains.  The chains of a key meet as (a0+a1)+(a2+a3) by two quad swaps;
+// the tile sum of the exponentials is the same adjacent-pair tree as lg_sum32 (slot = 16 * half + k: lane bits 2..5
+// are slot bits 0..3, the halves are bit 4).  In the value phase (lane = 4 dims) the weight of slot s is read out of
+// the lane of its key into a scalar register.  Every slot goes through the value chains (masked slots weigh exactly
+// zero and their rows are zeroed at staging).  A workgroup walks `tp` tiles, the next one's rows in flight while the
+// current one is computed; the first four wavefronts stage.  Partials as lg_k_attn writes them.
+__device__ __forceinline__ float lg_fma_hlo_s(float x, uint32_t hp, float acc) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel_hi:[0,1,0]" : "+v"(acc) : "s"(x), "v"(hp));
+    return acc;
+}
+__device__ __forceinline__ float lg_fma_hhi_s(float x, uint32_t hp, float acc) {
+    asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : "+v"(acc) : "s"(x), "v"(hp));
+    return acc;
+}
+template <int HD>
+struct AttnUGeo {
+    static constexpr int CS = HD / 2 + 16;                    // bytes per (key, chain) run of the K tile: hd/4 halves + pad
+    static constexpr int KS = 4 * CS;                         // bytes per key (groups of 8 lanes = 2 keys x 4 chains cover all banks)
+    static constexpr int VS = HD * 2 + 16;                    // bytes per V row
+    static constexpr int QC = HD / 4 + 4;                     // floats per chain of a staged query
+    static size_t bytes(int units) { return (size_t)units * 4 * QC * 4 + (size_t)32 * KS + (size_t)32 * VS; }
+};
+template <int HD>                                             // (up to 256-wide heads: 128 registers a lane, two workgroups per CU)
+__global__ __launch_bounds__(512, HD > 256 ? 2 : 4) void lg_k_attn_u(AttnArgs a, const StepCtl *ctl, int rw, int tp) {
+    using Geo = AttnUGeo<HD>;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int G = a.H / a.nkv, units = 8;                     // rw * G == 8, blockDim.x == 512
+    float *qs = (float *)smem;                                // [unit][4 chains][QC]
+    unsigned char *kt = smem + (size_t)units * 4 * Geo::QC * 4;               // [32 keys][4 chains][CS]
+    unsigned char *vt = kt + 32 * Geo::KS;                    // [32][VS]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const int kvh = blockIdx.y, j0 = blockIdx.z * rw, posb = ctl->pos + a.pos_off;
+    // tiles are numbered from the first tile of the whole block, as lg_k_attn_merge reads them
+    const int first = lg_win_start(posb, a.window) >> 5;
+    const int glo = lg_win_start(posb + j0, a.window), ghi = posb + j0 + rw - 1;         // keys any row of the group sees
+    const int n0 = (glo >> 5) + blockIdx.x * tp;
+    int n1 = n0 + tp - 1; if (n1 > (ghi >> 5)) n1 = ghi >> 5;
+    if (n0 > n1) return;
+    constexpr int U4R = HD / 8;                               // 16-byte units per row
+    constexpr int STG = 32 * U4R >= 512 ? 512 : 256;          // staging threads
+    constexpr int KL = 32 * U4R / STG;                        // units per staging thread and matrix
+    static_assert(32 * U4R % STG == 0, "tile staging assumes whole passes");
+    const bool stager = threadIdx.x < STG;
+    uint4 kq[KL], vq[KL];
+    auto fetch = [&](int n) {
+        const int r0 = (n << 5) % a.seq;
+        #pragma unroll
+        for (int u = 0; u < KL; ++u) {
+            const int idx = (int)threadIdx.x + u * STG, row = idx / U4R, u4 = idx - row * U4R;
+            int rr = r0 + row; if (rr >= a.seq) rr -= a.seq;
+            const size_t go = (size_t)rr * a.kv_dim + (size_t)kvh * HD + u4 * 8;
+            kq[u] = a.kc4(go); vq[u] = a.vc4(go);
+        }
+    };
+    auto stash = [&](int n) {
+        const int t0 = n << 5;
+        #pragma unroll
+        for (int u = 0; u < KL; ++u) {
+            const int idx = (int)threadIdx.x + u * STG, row = idx / U4R, u4 = idx - row * U4R;
+            const uint32_t mk = (t0 + row >= glo && t0 + row <= ghi) ? 0xFFFFFFFFu : 0u;
+            const uint4 k = make_uint4(kq[u].x & mk, kq[u].y & mk, kq[u].z & mk, kq[u].w & mk);
+            unsigned char *d = kt + row * Geo::KS + u4 * 4;   // steps 2*u4, 2*u4+1 of every chain: elements c and 4+c of the 8
+            *(uint32_t *)(d) = (k.x & 0xFFFFu) | (k.z << 16);
+            *(uint32_t *)(d + Geo::CS) = (k.x >> 16) | (k.z & 0xFFFF0000u);
+            *(uint32_t *)(d + 2 * Geo::CS) = (k.y & 0xFFFFu) | (k.w << 16);
+            *(uint32_t *)(d + 3 * Geo::CS) = (k.y >> 16) | (k.w & 0xFFFF0000u);
+            *(uint4 *)(vt + row * Geo::VS + u4 * 16) = make_uint4(vq[u].x & mk, vq[u].y & mk, vq[u].z & mk, vq[u].w & mk);
+        }
+    };
+    if (stager) fetch(n0);
+    // this wavefront's unit and its query, chain-major through its own LDS rows into registers
+    const int j = j0 + wave / G, head = kvh * G + wave % G, pj = posb + j, startj = lg_win_start(pj, a.window);
+    const int kk = lane >> 2, c = lane & 3;
+    float qreg[HD / 4];
+    {
+        float *qw = qs + (size_t)wave * 4 * Geo::QC;
+        const float4 *qrow = (const float4 *)(a.q + (size_t)j * a.H * HD + (size_t)head * HD);
+        #pragma unroll
+        for (int i = 0; i < (HD / 4 + 63) / 64; ++i) {
+            const int g = lane + 64 * i;
+            if (g < HD / 4) {
+                const float4 f = qrow[g];
+                qw[g] = f.x; qw[Geo::QC + g] = f.y; qw[2 * Geo::QC + g] = f.z; qw[3 * Geo::QC + g] = f.w;
+            }
+        }
+        lg_wave_lds_sync();
+        #pragma unroll
+        for (int i = 0; i < HD / 16; ++i) {
+            const float4 f = *(const float4 *)(qw + c * Geo::QC + 4 * i);
+            qreg[4 * i] = f.x; qreg[4 * i + 1] = f.y; qreg[4 * i + 2] = f.z; qreg[4 * i + 3] = f.w;
+        }
+    }
+    for (int n = n0; n <= n1; ++n) {
+        if (n > n0) __syncthreads();                          // the previous tile has been read by every wavefront
+        if (stager) stash(n);
+        __syncthreads();
+        if (stager && n < n1) fetch(n + 1);
+        if (n < (startj >> 5) || n > (pj >> 5)) continue;     // tile outside this unit's keys (wavefront-uniform; barriers are above)
+        const int t0 = n << 5, bx = n - first;
+        float e0, e1;
+        {   // scores of keys kk and 16 + kk, chain c
+            const unsigned char *k0 = kt + kk * Geo::KS + c * Geo::CS, *k1 = k0 + 16 * Geo::KS;
+            float a0 = 0.0f, a1 = 0.0f;
+            #pragma unroll
+            for (int i = 0; i < HD / 32; ++i) {
+                const uint4 x = *(const uint4 *)(k0 + 16 * i), y = *(const uint4 *)(k1 + 16 * i);
+                a0 = lg_fma_hlo(qreg[8 * i], x.x, a0);     a1 = lg_fma_hlo(qreg[8 * i], y.x, a1);
+                a0 = lg_fma_hhi(qreg[8 * i + 1], x.x, a0); a1 = lg_fma_hhi(qreg[8 * i + 1], y.x, a1);
+                a0 = lg_fma_hlo(qreg[8 * i + 2], x.y, a0); a1 = lg_fma_hlo(qreg[8 * i + 2], y.y, a1);
+                a0 = lg_fma_hhi(qreg[8 * i + 3], x.y, a0); a1 = lg_fma_hhi(qreg[8 * i + 3], y.y, a1);
+                a0 = lg_fma_hlo(qreg[8 * i + 4], x.z, a0); a1 = lg_fma_hlo(qreg[8 * i + 4], y.z, a1);
+                a0 = lg_fma_hhi(qreg[8 * i + 5], x.z, a0); a1 = lg_fma_hhi(qreg[8 * i + 5], y.z, a1);
+                a0 = lg_fma_hlo(qreg[8 * i + 6], x.w, a0); a1 = lg_fma_hlo(qreg[8 * i + 6], y.w, a1);
+                a0 = lg_fma_hhi(qreg[8 * i + 7], x.w, a0); a1 = lg_fma_hhi(qreg[8 * i + 7], y.w, a1);
+            }
+            // (a0+a1)+(a2+a3) over the four chain lanes of a key
+            a0 = a0 + lg_dpp_f<LG_DPP_SWAP1>(a0); a0 = a0 + lg_dpp_f<LG_DPP_SWAP2>(a0);
+            a1 = a1 + lg_dpp_f<LG_DPP_SWAP1>(a1); a1 = a1 + lg_dpp_f<LG_DPP_SWAP2>(a1);
+            const int ta = t0 + kk, tb = ta + 16;
+            const bool va = ta >= startj && ta <= pj, vb = tb >= startj && tb <= pj;
+            const float s0 = va ? a0 : -INFINITY, s1 = vb ? a1 : -INFINITY;
+            const float mx = lg_max_n(fmaxf(s0, s1), 64);
+            e0 = va ? lg_expf(s0 - mx) : 0.0f;
+            e1 = vb ? lg_expf(s1 - mx) : 0.0f;
+            // lg_sum32 over slot = 16 * half + kk: slot bits 0..3 are lane bits 2..5 (values repeat over the chain lanes,
+            // so the mirrors that also flip lower lane bits pair the same values), bit 4 is the half
+            float l0 = e0, l1 = e1;
+            l0 = l0 + lg_dpp_f<LG_DPP_MIRROR8>(l0);  l1 = l1 + lg_dpp_f<LG_DPP_MIRROR8>(l1);
+            l0 = l0 + lg_dpp_f<LG_DPP_MIRROR16>(l0); l1 = l1 + lg_dpp_f<LG_DPP_MIRROR16>(l1);
+            l0 = lg_add_x16(l0); l1 = lg_add_x16(l1);
+            l0 = lg_add_x32(l0); l1 = lg_add_x32(l1);
+            if (lane == 0) {
+                const size_t pi = ((size_t)j * a.H + head) * a.tiles_max + bx;
+                a.pm[pi] = mx; a.pl[pi] = l0 + l1;
+            }
+        }
+        // values: lane = 4 dims of each 256
+        #pragma unroll
+        for (int dh = 0; dh < HD; dh += 256) {
+            const bool live = dh + 4 * lane < HD;
+            const unsigned char *vl = vt + (live ? (dh + 4 * lane) * 2 : 0);
+            float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            #pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int eb = __float_as_int(half ? e1 : e0);
+                #pragma unroll 8
+                for (int k = 0; k < 16; ++k) {
+                    const uint2 v = *(const uint2 *)(vl + (16 * half + k) * Geo::VS);
+                    const float es = __int_as_float(__builtin_amdgcn_readlane(eb, 4 * k));
+                    acc.x = lg_fma_hlo_s(es, v.x, acc.x); acc.y = lg_fma_hhi_s(es, v.x, acc.y);
+                    acc.z = lg_fma_hlo_s(es, v.y, acc.z); acc.w = lg_fma_hhi_s(es, v.y, acc.w);
+                }
+            }
+            if (live) {
+                const size_t pi = ((size_t)j * a.H + head) * a.tiles_max + bx;
+                *(float4 *)(a.pacc + pi * HD + dh + 4 * lane) = acc;
+            }
+        }
+    }
+}
+
 // lg_k_attn_merge for rows with very many tiles: one wavefront per (head, row, 64 dims) instead of one workgroup per
 // (head, row), so that four times as many CUs pull the partials (a (head, row) at 8192 keys has 257 KB of them).
 // Same order: weights exp(m_t - M), L and the output as fma chains over the tiles ascending, divide, q8.

@@ -745,6 +745,32 @@ static int attention_rows_tp(int tiles, int nkv) {
     return tp < 1 ? 1 : tp > 4 ? 4 : tp;
 }
 
+// lg_k_attn_u (prompt blocks, queries in registers, a wavefront per (row, head) unit, 8 units per workgroup): rows of
+// the block per workgroup, 0 when the shape does not fit
+static int attention_u_rows(int rows, int G, int hd, int seq) {
+    if (rows <= LG_HIP_MAX_ROWS || seq < 32 || (hd != 64 && hd != 128 && hd != 256 && hd != 512)) return 0;
+    if (G < 1 || G > 8 || 8 % G) return 0;
+    const int rw = 8 / G;
+    return rows % rw == 0 ? rw : 0;
+}
+// launch geometry: tiles a row group can touch, tiles per workgroup (so that the grid has about two workgroups per CU)
+template <typename L>
+static int attention_u_launch(L &&launch, int rows, int rw, int nkv, int hd, int window, int block_tiles) {
+    int nt = block_tiles;
+    if (window > 0) { const int t = (window + rw - 1 + 31) / 32 + 1; if (t < nt) nt = t; }
+    const int groups = rows / rw;
+    int tp = (int)(((long long)nt * nkv * groups + 511) / 512);
+    if (tp < 1) tp = 1;
+    if (tp > nt) tp = nt;
+    const dim3 grid((nt + tp - 1) / tp, nkv, groups);
+    switch (hd) {
+        case 512: return launch(lg_k_attn_u<512>, grid, AttnUGeo<512>::bytes(8), tp);
+        case 256: return launch(lg_k_attn_u<256>, grid, AttnUGeo<256>::bytes(8), tp);
+        case 128: return launch(lg_k_attn_u<128>, grid, AttnUGeo<128>::bytes(8), tp);
+        default:  return launch(lg_k_attn_u<64>, grid, AttnUGeo<64>::bytes(8), tp);
+    }
+}
+
 template <int M>
 static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry) {
     Launcher lx{ m, dry };
@@ -875,6 +901,15 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
             const int tiles = layer_tiles(L);
             const bool shared = rows_shared(L);
+            // prompt blocks (the queries arrive prepared: lg_k_qkv_post ran): eight (row, head) units per workgroup with the
+            // queries in registers
+            const int urows = (!fused_post && pos_off == 0 && m->attn_rows) ? attention_u_rows(M, G, y.hd, kv->seq[y.src]) : 0;
+            if (urows) {
+                attention_u_launch([&](auto kernel, dim3 grid, size_t lds, int tp) {
+                    LAUNCH(KC_ATTN, kernel, grid, dim3(512), lds, a, m->ctl, urows, tp);
+                    return 0;
+                }, M, urows, y.nkv, y.hd, window, tiles);
+            } else
             if (shared) {
                 if constexpr (M > 1 && M <= LG_HIP_MAX_ROWS) {
                     const size_t lds = y.hd == 256 ? AttnRowsGeo<256>::bytes(M * G) : y.hd == 128 ? AttnRowsGeo<128>::bytes(M * G) : AttnRowsGeo<64>::bytes(M * G);
