@@ -266,13 +266,16 @@ __global__ __launch_bounds__(LG_WG) void lg_k_draft_input(DraftInArgs a, const S
 // activations are staged (weights depend on nothing), each later chunk while the previous one is
 // being consumed.
 #define LG_U 2
-template <int G>
-struct WChunk { uint4 q[G][LG_U]; uint32_t s[G][LG_U]; };
+#ifndef LG_U32
+#define LG_U32 4                            // tiles per chunk of the long-row (32-segment) matmul
+#endif
+template <int G, int U = LG_U>
+struct WChunk { uint4 q[G][U]; uint32_t s[G][U]; };
 
-template <int G>
-__device__ __forceinline__ void lg_mm_fetch(WChunk<G> &w, const uint8_t *const (&wg)[G], int it0, int nit, int lane) {
+template <int G, int U = LG_U>
+__device__ __forceinline__ void lg_mm_fetch(WChunk<G, U> &w, const uint8_t *const (&wg)[G], int it0, int nit, int lane) {
     #pragma unroll
-    for (int u = 0; u < LG_U; ++u)
+    for (int u = 0; u < U; ++u)
         #pragma unroll
         for (int g = 0; g < G; ++g) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;                 // clamp: never read past the group
@@ -283,8 +286,8 @@ __device__ __forceinline__ void lg_mm_fetch(WChunk<G> &w, const uint8_t *const (
 
 // On return every lane of a row holds that row's M results (adjacent-pair tree over the S lanes done).
 // `first` must hold the chunk of tiles 0..LG_U-1.
-template <int M, int S, int G, bool DUMP>
-__device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChunk<G> &first, int nit, const int8_t *act,
+template <int M, int S, int G, bool DUMP, int U = LG_U>
+__device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChunk<G, U> &first, int nit, const int8_t *act,
                                              const float2 *actds, int k, float (&acc)[G][M], int lane,
                                              int32_t *dots, int m, const int (&row)[G]) {
     const int c = lane & (S - 1), nb = k >> 5;
@@ -292,12 +295,12 @@ __device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChu
     for (int g = 0; g < G; ++g)
         #pragma unroll
         for (int j = 0; j < M; ++j) acc[g][j] = 0.0f;
-    WChunk<G> cur = first;
-    for (int it0 = 0; it0 < nit; it0 += LG_U) {
-        WChunk<G> nxt;
-        if (it0 + LG_U < nit) lg_mm_fetch<G>(nxt, wg, it0 + LG_U, nit, lane);
+    WChunk<G, U> cur = first;
+    for (int it0 = 0; it0 < nit; it0 += U) {
+        WChunk<G, U> nxt;
+        if (it0 + U < nit) lg_mm_fetch<G, U>(nxt, wg, it0 + U, nit, lane);
         #pragma unroll
-        for (int u = 0; u < LG_U; ++u) {
+        for (int u = 0; u < U; ++u) {
             if (it0 + u >= nit) break;
             const int it = it0 + u, b = c * nit + it;        // b: block of the natural order (for DUMP)
             // the LDS reads of all M rows go out together, ahead of the first dot: left to itself the compiler
@@ -320,7 +323,7 @@ __device__ __forceinline__ void lg_mm_groups(const uint8_t *const (&wg)[G], WChu
                 }
             }
         }
-        if (it0 + LG_U < nit) cur = nxt;
+        if (it0 + U < nit) cur = nxt;
     }
     #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -365,13 +368,14 @@ __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
         wg[g] = a.w + (size_t)gi * nit * LG_TILE;
         row[g] = gi * RW + lane / S;
     }
-    WChunk<G> first;
-    lg_mm_fetch<G>(first, wg, 0, nit, lane);
+    constexpr int U = S == 32 ? LG_U32 : LG_U;
+    WChunk<G, U> first;
+    lg_mm_fetch<G, U>(first, wg, 0, nit, lane);
     lg_load_q8<M>(a.q_in, a.k, lq);
     __syncthreads();
     if (g0 >= ngroups) return;
     float acc[G][M];
-    lg_mm_groups<M, S, G, DUMP>(wg, first, nit, lq, lds, a.k, acc, lane, a.dots, a.m, row);
+    lg_mm_groups<M, S, G, DUMP, U>(wg, first, nit, lq, lds, a.k, acc, lane, a.dots, a.m, row);
     const int c = lane & (S - 1);
     if (c < M) {
         #pragma unroll
