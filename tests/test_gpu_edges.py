@@ -135,3 +135,38 @@ def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
     finally:
         slot.value = None
         gpu.close(); o.close()
+
+
+@pytest.mark.parametrize("rows", [2, 5])
+def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, rows):
+    """The options that pick between kernels for the same arithmetic (row work inside the q/k/v matmul, the
+    attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay) change
+    timing only: every combination leaves the same cache rows and the same logits rows of a verify block."""
+    path, spec = model_path("tiny_full")
+    V = spec["n_vocab"]
+    rng = np.random.default_rng(rows)
+    prompt = rng.integers(0, V, 300).astype(np.int32)
+    blk = rng.integers(0, V, rows).astype(np.int32)
+
+    def run(**opts):
+        gpu = lg.hiplib.HipBackend(path, 400, max_rows=8)
+        try:
+            for k, v in opts.items():
+                gpu.set_option(k, v)
+            gpu.set_option("store_logits", 1)
+            gpu.prefill(prompt, 0)
+            adv, out = gpu.forward_spec(blk, 300)
+            logits = np.stack([gpu.logits_row(j, V) for j in range(rows)])
+            cache = [gpu.kv_read(L, w).copy() for L in range(spec["n_layer"] - spec["shared_kv_layers"]) for w in (0, 1)]
+            return adv, out.copy(), logits, cache
+        finally:
+            gpu.close()
+
+    base = run()
+    for name in ("fuse_rows", "attn_rows", "head_mfma", "wide_prefill", "use_graph"):
+        print(f"rows={rows} option {name}=0", flush=True)
+        got = run(**{name: 0})
+        assert got[0] == base[0] and np.array_equal(got[1], base[1]), name
+        assert np.array_equal(got[2].view(np.uint32), base[2].view(np.uint32)), name
+        for a, b in zip(got[3], base[3]):
+            assert np.array_equal(a, b), name
