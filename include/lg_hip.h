@@ -168,6 +168,14 @@ int  lg_hip_launch_floor(int n_kernels, int mode, int grid, int block, int repla
  * of the matmul kernel alone. */
 int  lg_hip_matmul_q4q8(const void *w, int k, int m, const float *x, int rows, float *out,
                         int32_t *dots, int8_t *xq, float *xd, int32_t *xsum, int repeats, float *kernel_ms);
+/* The row work between two matmuls of a verify block (add-norm + norm + q8: add_rmsnorm_kernel, rmsnorm_kernel and
+ * d_quant_group, src/cuda/model-cuda.cuh:119-175, :84-110, one kernel here): x_out = (x + rmsnorm(dout) * w_post) *
+ * out_scale (dout, out_scale may be NULL), h = rmsnorm(x_out) * w_pre (w_pre NULL: h = x_out), q8 of h per 32.
+ * rows 1..8, E a multiple of 256 up to 4096.  Outputs (each may be NULL): x_out, h_out [rows][E] f32, xq [rows][E]
+ * int8, xd / xsum [rows][E/32]. */
+int  lg_hip_rows_norm_q8(const float *x, const float *dout, const float *w_post, const float *out_scale,
+                         const float *w_pre, int rows, int E, float eps, float *x_out, float *h_out,
+                         int8_t *xq, float *xd, int32_t *xsum);
 /* Matmul against a matrix kept in f32 (the per-layer-embedding matrices of QAT conversions; the reference's int8
  * backend multiplies such weights by the f32 activations unquantized, src/cuda/model-cuda-i8.cu:645-653, :846-895):
  * w = m rows of k floats, x = rows x k floats, out = rows x m floats.  Any number of rows (8 per workgroup row). */

@@ -1486,6 +1486,66 @@ extern "C" int lg_hip_matmul_q4q8(const void *w, int k, int mrows, const float *
     return 0;
 }
 
+// q8 rows of a verify-width block from the device's activation order back to natural order
+static int read_back_q8(const int8_t *dq, int rows, int k, int8_t *xq, float *xd, int32_t *xsum) {
+    const ActLayout lay = lg_act_layout(k);
+    const int nb = k / 32;
+    if (xq) {
+        std::vector<int8_t> dev((size_t)rows * k);
+        HIP_TRY(hipMemcpy(dev.data(), dq, dev.size(), hipMemcpyDeviceToHost));
+        for (int j = 0; j < rows; ++j)
+            for (int w = 0; w < k / 16; ++w)
+                memcpy(xq + (size_t)j * k + (size_t)w * 16, dev.data() + (size_t)j * k + (size_t)lg_act_unit(lay, w) * 16, 16);
+    }
+    if (xd || xsum) {
+        std::vector<float2> ds((size_t)rows * nb);
+        HIP_TRY(hipMemcpy(ds.data(), dq + (size_t)rows * k, ds.size() * 8, hipMemcpyDeviceToHost));
+        for (int j = 0; j < rows; ++j)
+            for (int b = 0; b < nb; ++b) {
+                const float2 v = ds[(size_t)j * nb + lg_act_block(lay, b)];
+                if (xd) xd[(size_t)j * nb + b] = v.x;
+                if (xsum) memcpy(&xsum[(size_t)j * nb + b], &v.y, 4);
+            }
+    }
+    return 0;
+}
+
+template <int M>
+static void rows_isolated(hipStream_t st, const RowArgs &s, StepCtl *ctl) {
+    const int slices = (s.E + 1023) / 1024;                   // as a verify step launches it: the tail sliced over workgroups
+    hipLaunchKernelGGL((lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, st, s, ctl);
+}
+extern "C" int lg_hip_rows_norm_q8(const float *x, const float *dout, const float *w_post, const float *out_scale,
+                                   const float *w_pre, int rows, int E, float eps, float *x_out, float *h_out,
+                                   int8_t *xq, float *xd, int32_t *xsum) {
+    if (!x) return fail(-1, "rows_norm_q8: null input");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || E < 256 || E % 256 || E > 4096) return fail(-2, "rows_norm_q8: rows %d (1..%d), E %d (a multiple of 256 up to 4096)", rows, LG_HIP_MAX_ROWS, E);
+    if (dout && !w_post) return fail(-1, "rows_norm_q8: a sub-layer output needs its norm weight");
+    if (lg_hip_device_count() < 1) return fail(-3, "rows_norm_q8: no HIP device");
+    Scratch sc;
+    float *dx, *dd = nullptr, *dwp = nullptr, *dos = nullptr, *dwr = nullptr, *dxo, *dho; int8_t *dq; StepCtl *ctl;
+    const size_t n = (size_t)rows * E;
+    if (sc.get(&dx, n) || sc.get(&dxo, n) || sc.get(&dho, n) || sc.get(&dq, n * 5 / 4) || sc.get(&ctl, 1)) return -7;
+    HIP_TRY(hipMemcpy(dx, x, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    if (dout) { if (sc.get(&dd, n) || sc.get(&dwp, (size_t)E)) return -7; HIP_TRY(hipMemcpy(dd, dout, n * 4, hipMemcpyHostToDevice)); HIP_TRY(hipMemcpy(dwp, w_post, (size_t)E * 4, hipMemcpyHostToDevice)); }
+    if (out_scale) { if (sc.get(&dos, 1)) return -7; HIP_TRY(hipMemcpy(dos, out_scale, 4, hipMemcpyHostToDevice)); }
+    if (w_pre) { if (sc.get(&dwr, (size_t)E)) return -7; HIP_TRY(hipMemcpy(dwr, w_pre, (size_t)E * 4, hipMemcpyHostToDevice)); }
+    RowArgs s{};
+    s.x = dx; s.dout = dd; s.dparts = 1; s.w_post = dwp; s.os = dos; s.x_out = dxo; s.w_pre = dwr; s.h_out = dho;
+    s.q = dq; s.E = E; s.eps = eps;
+    switch (rows) {
+#define CASE(M) case M: rows_isolated<M>(nullptr, s, ctl); break;
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+    }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    if (x_out) HIP_TRY(hipMemcpy(x_out, dxo, n * 4, hipMemcpyDeviceToHost));
+    if (h_out) HIP_TRY(hipMemcpy(h_out, dho, n * 4, hipMemcpyDeviceToHost));
+    return read_back_q8(dq, rows, E, xq, xd, xsum);
+}
+
 // the two launches of an isolated attention: tile partials, then the ordered merge
 // (the same choice of kernels as a verify step makes: many (tile, kv head) pairs -> one workgroup per pair serves all
 // rows; many tiles per row -> the merge is cut by dims)

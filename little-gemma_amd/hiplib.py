@@ -60,6 +60,7 @@ def load_hip():
     L.lg_hip_matmul_q4q8.argtypes = [u8p, C.c_int, C.c_int, f32p, C.c_int] + [C.c_void_p] * 5 + [C.c_int, C.c_void_p]
     L.lg_hip_attention.argtypes = [f32p, u16p, u16p] + [C.c_int] * 7 + [f32p, C.c_int, C.c_void_p]
     L.lg_hip_matmul_f32w.argtypes = [f32p, C.c_int, C.c_int, f32p, C.c_int, f32p]
+    L.lg_hip_rows_norm_q8.argtypes = [f32p] + [C.c_void_p] * 4 + [C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 5
     L.lg_hip_kv_layout.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
     L.lg_hip_kv_write.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
     L.lg_hip_kv_read.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
@@ -339,6 +340,20 @@ def matmul_q4q8(w_q4_0, k, m, x, want_dots=False, repeats=0):
     hip_check(H.lg_hip_matmul_q4q8(w, k, m, x, rows, _opt(out), _opt(dots), _opt(xq), _opt(xd), _opt(xsum),
                                    repeats, C.cast(C.byref(ms), C.c_void_p)), "matmul_q4q8")
     return dict(out=out, dots=dots, xq=xq, xd=xd, xsum=xsum, ms=ms.value)
+
+
+def rows_norm_q8(x, dout=None, w_post=None, out_scale=None, w_pre=None, eps=1e-6):
+    """Isolated row kernel through the C ABI.  x, dout: [rows, E] f32; returns dict(x_out, h, xq, xd, xsum)."""
+    H = load_hip()
+    x = np.ascontiguousarray(x, np.float32)
+    rows, E = x.shape
+    keep = [np.ascontiguousarray(a, np.float32) if a is not None else None
+            for a in (dout, w_post, None if out_scale is None else np.array([out_scale], np.float32), w_pre)]
+    x_out = np.zeros_like(x); h = np.zeros_like(x)
+    xq = np.zeros((rows, E), np.int8); xd = np.zeros((rows, E // 32), np.float32); xsum = np.zeros((rows, E // 32), np.int32)
+    hip_check(H.lg_hip_rows_norm_q8(x, *[_opt(a) for a in keep], rows, E, eps, _opt(x_out), _opt(h), _opt(xq), _opt(xd), _opt(xsum)),
+              "rows_norm_q8")
+    return dict(x_out=x_out, h=h, xq=xq, xd=xd, xsum=xsum)
 
 
 def matmul_f32w(w, x):

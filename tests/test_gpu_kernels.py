@@ -77,6 +77,43 @@ def test_matmul_float_weights_matches_oracle(lg, ob, gpu_required, m, k, rows):
         assert np.array_equal(got[j].view(np.uint32), want.view(np.uint32)), f"row {j}"
 
 
+@pytest.mark.parametrize("rows,E,with_dout,with_os,with_pre", [(5, 2560, True, True, True), (1, 512, True, False, True),
+                                                            (8, 3840, True, True, False), (3, 256, False, False, True),
+                                                            (4, 4096, False, False, False)])
+def test_rows_kernel_matches_oracle(lg, ob, gpu_required, rows, E, with_dout, with_os, with_pre):
+    """The row work between two matmuls in isolation (add-norm, output scale, norm, q8): the updated residual, the
+    normed row and its q8 are the oracle's, bit for bit, with and without each optional part."""
+    rng = np.random.default_rng(rows * 1000 + E)
+    L = ob.lib()
+    x = rng.normal(0, 1, (rows, E)).astype(np.float32)
+    dout = rng.normal(0, 3, (rows, E)).astype(np.float32) if with_dout else None
+    w_post = (1 + 0.1 * rng.normal(0, 1, E)).astype(np.float32) if with_dout else None
+    w_pre = (1 + 0.1 * rng.normal(0, 1, E)).astype(np.float32) if with_pre else None
+    os_ = 0.9 if with_os else None
+    x[0, :64] = 0.0
+    print(f"rows kernel rows={rows} E={E} dout={with_dout} os={with_os} pre={with_pre}", flush=True)
+    r = lg.hiplib.rows_norm_q8(x, dout, w_post, os_, w_pre, eps=1e-6)
+    for j in range(rows):
+        xn = x[j].copy()
+        if with_dout:
+            ob_ = np.zeros(E, np.float32)
+            L.lgo_rmsnorm(ob_, np.ascontiguousarray(dout[j]), w_post.ctypes.data, E, 1e-6, 1)
+            xn = xn + ob_
+            if with_os:
+                xn = xn * np.float32(os_)
+        h = np.zeros(E, np.float32)
+        if with_pre:
+            L.lgo_rmsnorm(h, np.ascontiguousarray(xn), w_pre.ctypes.data, E, 1e-6, 1)
+        else:
+            h = xn
+        q = np.zeros(E, np.int8); d = np.zeros(E // 32, np.float32); sm = np.zeros(E // 32, np.int32)
+        L.lgo_quant_q8(np.ascontiguousarray(h), E, q, d, sm)
+        assert np.array_equal(r["x_out"][j].view(np.uint32), xn.view(np.uint32)), f"row {j}: residual"
+        assert np.array_equal(r["h"][j].view(np.uint32), h.view(np.uint32)), f"row {j}: normed row"
+        assert np.array_equal(r["xq"][j], q) and np.array_equal(r["xsum"][j], sm), f"row {j}: q8"
+        assert np.array_equal(r["xd"][j].view(np.uint32), d.view(np.uint32)), f"row {j}: scales"
+
+
 def test_matmul_is_linear_in_the_scales(lg, gpu_required):
     """Size-independent property: doubling every weight scale doubles every output exactly
     (powers of two commute with rounding), negating codes around 8 negates it."""
