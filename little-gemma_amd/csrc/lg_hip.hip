@@ -709,12 +709,11 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
         const int W = 4;
         LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
     } else if (M >= 4 && a.k >= 2048 && !DUMP) {
-        // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over four wavefronts
+        // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over two wavefronts
+        // (over four was no faster)
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
-            static const int kp = getenv("LG_KP") ? atoi(getenv("LG_KP")) : 2;
             const size_t l2 = ((lds + 15) & ~(size_t)15) + (size_t)2 * M * 64 * 4;
-            if (kp == 4) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, a);
-            else         LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
+            LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
         }
     } else {
         // Two row groups per workgroup when there are very many groups, and for blocks of 4+ rows when one group per
