@@ -754,62 +754,66 @@ __global__ __launch_bounds__(512, HD > 256 ? 2 : 4) void lg_k_attn_u(AttnArgs a,
     }
 }
 
-// lg_k_attn_merge for rows with very many tiles: one wavefront per (head, row, 64 dims) instead of one workgroup per
-// (head, row), so that four times as many CUs pull the partials (a (head, row) at 8192 keys has 257 KB of them).
-// Same order: weights exp(m_t - M), L and the output as fma chains over the tiles ascending, divide, q8.
+// lg_k_attn_merge for rows with very many tiles: one workgroup of four wavefronts per (head, row, 64 dims).  The
+// merge is one fma chain over the tiles ascending, and walked by a single wavefront its time is the instruction issue
+// of 2 loads + 2 fma per tile, tile after tile.  Here the tiles go in rounds of 256: wavefront w requests the 64
+// partials of tiles 64w..64w+63 of the round at once (all four wavefronts' loads in flight together) while the
+// workgroup computes the round's weights exp(m_t - M) into LDS; then the chain passes through the wavefronts in
+// order, each running its 64 fma back to back from registers and handing (L, o) to the next through LDS.  Same
+// order, same bits: weights exp(m_t - M), L and the output as fma chains over the tiles ascending, divide, q8.
 template <int M>
-__global__ __launch_bounds__(64) void lg_k_attn_merge_split(MergeArgs a, const StepCtl *ctl) {
-    __shared__ float wts[512];
-    const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd, lane = threadIdx.x;
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge_split(MergeArgs a, const StepCtl *ctl) {
+    __shared__ float wts[256], pls[256], hand[2][64], wmx[4];
+    const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int d = blockIdx.z * 64 + lane;                     // hd is a multiple of 64
     const int pos = ctl->pos + a.pos_off, pj = pos + j;
     const int first = lg_win_start(pos, a.window) >> 5;
     const int lo = (lg_win_start(pj, a.window) >> 5) - first, hi = (pj >> 5) - first;
-    const size_t base = ((size_t)j * a.H + head) * a.tiles_max;
-    // the partials do not depend on the weights: the first batch of them is requested before the maxima are read,
-    // and from then on batch n + 1 is in flight while batch n goes through the chains
-    constexpr int U = 32;
+    const size_t base = ((size_t)j * a.H + head) * a.tiles_max + lo;
     const int nt = hi - lo + 1;
-    float pl0[U], pa0[U], pl1[U], pa1[U];
-    auto fetch = [&](float (&pl)[U], float (&pa)[U], int n0) {
+    constexpr int U = 64;
+    float pa[U];
+    auto fetch = [&](int t0) {                                // tiles t0 .. t0+63 of this row (past the end: the last one again)
         #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int n = n0 + u < nt ? n0 + u : nt - 1;
-            pl[u] = a.pl[base + lo + n];
-            pa[u] = a.pacc[(base + lo + n) * hd + d];
+            const int n = t0 + u < nt ? t0 + u : nt - 1;
+            pa[u] = a.pacc[(base + n) * hd + d];
         }
     };
-    fetch(pl0, pa0, 0);
+    fetch(wave * U);                                          // the partials do not depend on the weights
     float mx = -INFINITY;
-    for (int n = lo + lane; n <= hi; n += 64) mx = fmaxf(mx, a.pm[base + n]);
+    for (int n = threadIdx.x; n < nt; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
     mx = lg_max_n(mx, 64);
+    if (lane == 0) wmx[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
     float L = 0.0f, o = 0.0f;
-    auto chain = [&](const float (&pl)[U], const float (&pa)[U], int n0, int c0) {
-        #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (n0 + u < nt) {
-                const float wn = wts[n0 + u - c0];
-                L = lg_fmaf(pl[u], wn, L);
-                o = lg_fmaf(pa[u], wn, o);
-            }
+    for (int r0 = 0; r0 < nt; r0 += 4 * U) {
+        if (r0 > 0) fetch(r0 + wave * U);
+        {   // the round's weights and sums (one tile per thread)
+            const int n = r0 + (int)threadIdx.x;
+            if (n < nt) { wts[threadIdx.x] = lg_expf(a.pm[base + n] - mx); pls[threadIdx.x] = a.pl[base + n]; }
         }
-    };
-    for (int c0 = 0; c0 < nt; c0 += 512) {                    // (512 is a multiple of 2 * U)
-        const int cn = nt - c0 < 512 ? nt - c0 : 512;
-        lg_wave_lds_sync();
-        for (int n = lane; n < cn; n += 64) wts[n] = lg_expf(a.pm[base + lo + c0 + n] - mx);
-        lg_wave_lds_sync();
-        for (int n0 = c0; n0 < c0 + cn; n0 += 2 * U) {
-            if (n0 + U < nt) fetch(pl1, pa1, n0 + U);
-            __builtin_amdgcn_sched_barrier(0);
-            chain(pl0, pa0, n0, c0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (n0 + 2 * U < nt) fetch(pl0, pa0, n0 + 2 * U);
-            __builtin_amdgcn_sched_barrier(0);
-            chain(pl1, pa1, n0 + U, c0);
-            __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        #pragma unroll
+        for (int turn = 0; turn < 4; ++turn) {
+            if (wave == turn && r0 + turn * U < nt) {
+                if (r0 + turn > 0) { L = hand[0][lane]; o = hand[1][lane]; }
+                #pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (r0 + turn * U + u < nt) {             // (a guard, not a break: the partials stay in registers)
+                        const float wn = wts[turn * U + u];
+                        L = lg_fmaf(pls[turn * U + u], wn, L);
+                        o = lg_fmaf(pa[u], wn, o);
+                    }
+                }
+                hand[0][lane] = L; hand[1][lane] = o;
+            }
+            __syncthreads();
         }
     }
+    if (wave != 0) return;
+    L = hand[0][lane]; o = hand[1][lane];
     const float r = o / L;
     float dq; int sum;
     const int q = lg_quant1_32lanes(r, &dq, &sum);

@@ -929,7 +929,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
-            if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(64), 0, g, m->ctl);
+            if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(LG_WG), 0, g, m->ctl);
             else LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
         }
         {   // attention output projection
@@ -1563,7 +1563,7 @@ static int enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs 
             else                  hipLaunchKernelGGL((lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
         }
     } else hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
-    if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && a.hd % 64 == 0) hipLaunchKernelGGL((lg_k_attn_merge_split<M>), dim3(a.H, M, a.hd / 64), dim3(64), 0, st, g, ctl);
+    if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && a.hd % 64 == 0) hipLaunchKernelGGL((lg_k_attn_merge_split<M>), dim3(a.H, M, a.hd / 64), dim3(LG_WG), 0, st, g, ctl);
     else hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
     return 0;
 }
