@@ -266,9 +266,6 @@ __global__ __launch_bounds__(LG_WG) void lg_k_draft_input(DraftInArgs a, const S
 // activations are staged (weights depend on nothing), each later chunk while the previous one is
 // being consumed.
 #define LG_U 2
-#ifndef LG_U32
-#define LG_U32 4                            // tiles per chunk of the long-row (32-segment) matmul
-#endif
 template <int G, int U = LG_U>
 struct WChunk { uint4 q[G][U]; uint32_t s[G][U]; };
 
@@ -351,7 +348,8 @@ struct MmArgs {
 
 // Plain matmul: out[j][i] f32.  blockDim = 64*W wavefronts, each wavefront takes G neighbouring
 // row groups (G*64/S rows); grid covers ceil(groups / (W*G)) workgroups.
-template <int M, int S, int G, bool DUMP>
+// U: weight tiles per chunk (requested together, the next chunk while the current one is consumed)
+template <int M, int S, int G, bool DUMP, int U = LG_U>
 __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
@@ -368,7 +366,6 @@ __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
         wg[g] = a.w + (size_t)gi * nit * LG_TILE;
         row[g] = gi * RW + lane / S;
     }
-    constexpr int U = S == 32 ? LG_U32 : LG_U;
     WChunk<G, U> first;
     lg_mm_fetch<G, U>(first, wg, 0, nit, lane);
     lg_load_q8<M>(a.q_in, a.k, lq);
