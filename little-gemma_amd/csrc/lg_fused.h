@@ -179,8 +179,8 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
     #pragma unroll
     for (int u = 0; u < TMAX; ++u) {
         const int it = it_lo + u < nit ? it_lo + u : nit - 1;
-        wq[u] = *(const uint4 *)(wg + (size_t)it * LG_TILE + lane * 16);
-        ws[u] = *(const uint16_t *)(wg + (size_t)it * LG_TILE + 1024 + lane * 2);
+        wq[u] = lg_ldt16(wg, it, lane);
+        ws[u] = lg_ldt2(wg, it, lane);
     }
     lg_load_q8<M>(a.q_in, k, lq);
     __syncthreads();
@@ -298,8 +298,8 @@ __global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
         #pragma unroll
         for (int u = 0; u < CH; ++u) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;
-            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
-            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+            nwq[u] = lg_ldt16(wt, it, lane);
+            nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
     if (np > 0) fetch(0, 0);
@@ -446,7 +446,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(AttnArgs a, const StepCt
             const int idx = min((int)threadIdx.x + u * LG_WG, 32 * U4R - 1), row = idx / U4R, u4 = idx - row * U4R;
             int rr = r0 + row; if (rr >= a.seq) rr -= a.seq;
             const size_t go = (size_t)rr * a.kv_dim + (size_t)kvh * HD + u4 * 8;
-            kq[u] = a.kc4(go); vq[u] = a.vc4(go);
+            kq[u] = a.kc4s(go); vq[u] = a.vc4s(go);
         }
     };
     auto stash = [&](int bx) {
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(512, HD > 256 ? 2 : 4) void lg_k_attn_u(AttnArgs a,
             const int idx = (int)threadIdx.x + u * STG, row = idx / U4R, u4 = idx - row * U4R;
             int rr = r0 + row; if (rr >= a.seq) rr -= a.seq;
             const size_t go = (size_t)rr * a.kv_dim + (size_t)kvh * HD + u4 * 8;
-            kq[u] = a.kc4(go); vq[u] = a.vc4(go);
+            kq[u] = a.kc4s(go); vq[u] = a.vc4s(go);
         }
     };
     auto stash = [&](int n) {

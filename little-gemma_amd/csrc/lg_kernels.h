@@ -276,8 +276,8 @@ __device__ __forceinline__ void lg_mm_fetch(WChunk<G, U> &w, const uint8_t *cons
         #pragma unroll
         for (int g = 0; g < G; ++g) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;                 // clamp: never read past the group
-            w.q[g][u] = *(const uint4 *)(wg[g] + (size_t)it * LG_TILE + lane * 16);
-            w.s[g][u] = *(const uint16_t *)(wg[g] + (size_t)it * LG_TILE + 1024 + lane * 2);
+            w.q[g][u] = lg_ldt16(wg[g], it, lane);
+            w.s[g][u] = lg_ldt2(wg[g], it, lane);
         }
 }
 
@@ -414,8 +414,8 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
         #pragma unroll
         for (int u = 0; u < CH; ++u) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;
-            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
-            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+            nwq[u] = lg_ldt16(wt, it, lane);
+            nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
     fetch(0);
@@ -519,8 +519,8 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
         #pragma unroll
         for (int u = 0; u < CH; ++u) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;
-            nwq[u] = *(const uint4 *)(wt + (size_t)it * LG_TILE + lane * 16);
-            nwd[u] = *(const uint16_t *)(wt + (size_t)it * LG_TILE + 1024 + lane * 2);
+            nwq[u] = lg_ldt16(wt, it, lane);
+            nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
     fetch(0);
@@ -664,8 +664,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     #pragma unroll
     for (int u = 0; u < LG_MAXV; ++u) {
         const int it = u < nit ? u : nit - 1;
-        wq[u] = *(const uint4 *)(wg[0] + (size_t)it * LG_TILE + lane * 16);
-        wsc[u] = *(const uint16_t *)(wg[0] + (size_t)it * LG_TILE + 1024 + lane * 2);
+        wq[u] = lg_ldt16(wg[0], it, lane);
+        wsc[u] = lg_ldt2(wg[0], it, lane);
     }
     if (threadIdx.x < 32) ipl[threadIdx.x] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + threadIdx.x];
     {
@@ -1024,6 +1024,9 @@ struct AttnArgs {
     float eps;
     __device__ __forceinline__ uint4 kc4(size_t off) const { return *(const uint4 *)(kc + off); }
     __device__ __forceinline__ uint4 vc4(size_t off) const { return *(const uint4 *)(vc + off); }
+    // for the kernels that stage a tile once for all the rows of a block: no second reader, so non-temporal
+    __device__ __forceinline__ uint4 kc4s(size_t off) const { return lg_ldw16(kc + off); }
+    __device__ __forceinline__ uint4 vc4s(size_t off) const { return lg_ldw16(vc + off); }
 };
 
 __device__ __forceinline__ int lg_win_start(int pos, int window) {
