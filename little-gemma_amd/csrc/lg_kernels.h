@@ -664,8 +664,9 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     #pragma unroll
     for (int u = 0; u < LG_MAXV; ++u) {
         const int it = u < nit ? u : nit - 1;
-        wq[u] = lg_ldt16(wg[0], it, lane);
-        wsc[u] = lg_ldt2(wg[0], it, lane);
+        // (plain loads: the M workgroups of a gate block read the same tiles)
+        wq[u] = *(const uint4 *)(wg[0] + (size_t)it * LG_TILE + lane * 16);
+        wsc[u] = *(const uint16_t *)(wg[0] + (size_t)it * LG_TILE + 1024 + lane * 2);
     }
     if (threadIdx.x < 32) ipl[threadIdx.x] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + threadIdx.x];
     {
