@@ -383,6 +383,90 @@ __global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Matmul of a verify block (4..8 rows) against a long-row matrix (S = 32 K segments per row, ffn_down), cut by K
+// quarter: workgroup (x, q) takes 8 rows per wavefront and the segments 8q .. 8q+7 of them, so it stages a quarter
+// of the activations (24 KB at 5 x 15360, where a workgroup that owns whole rows stages all 96 KB and a CU then
+// holds a single workgroup of four wavefronts).  A lane is (row r8, segment sg) and walks the segment's tiles with
+// the same serial fma chain as lg_k_mm; the 8 segment sums of a row meet in the same adjacent-pair tree (lg_sum8),
+// which is the bottom of the 32-segment tree.  The quarter's partial sums go to slab q of `out` ([4][M][m]); the
+// consumer adds the top of the tree, (p0+p1)+(p2+p3).
+template <int M>
+__global__ __launch_bounds__(320, 2) void lg_k_mm_kq(MmArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int q = blockIdx.y, nb = a.k >> 5, nit = nb >> 5;
+    uint4 *lq = (uint4 *)smem;                                // [M][nit][2 halves][8 segments] 16-byte units
+    float2 *lds = (float2 *)(smem + (size_t)M * nit * 256);   // [M][nit][8 segments] {scale, sum}
+    const int r8 = lane >> 3, sg = lane & 7, c = 8 * q + sg;
+    const int row0 = (blockIdx.x * nw + wave) * 8;
+    const int row = row0 + r8 < a.m ? row0 + r8 : a.m - 1;    // ragged tail: recompute the last row
+    // tiles hold two rows x 32 segments: this lane's 16 nibble bytes sit at (row & 1) * 32 + c
+    const uint8_t *wt = a.w + (size_t)(row >> 1) * nit * LG_TILE + ((row & 1) * 32 + c) * 16;
+    const uint8_t *ws = a.w + (size_t)(row >> 1) * nit * LG_TILE + 1024 + ((row & 1) * 32 + c) * 2;
+    constexpr int U = 4;
+    struct Chunk { uint4 q[U]; uint32_t s[U]; } cur, nxt;
+    auto fetch = [&](Chunk &w, int it0) {
+        #pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int it = it0 + u < nit ? it0 + u : nit - 1;
+            w.q[u] = lg_ldw16(wt + (size_t)it * LG_TILE);
+            w.s[u] = lg_ldw2(ws + (size_t)it * LG_TILE);
+        }
+    };
+    fetch(nxt, 0);                                            // (weights depend on nothing)
+    {   // the quarter of the activations: per (row, tile) two runs of 8 units and one run of 8 {scale, sum} = 20 x 16 bytes
+        const int n = M * nit * 20, T = blockDim.x;
+        const uint4 *gq = (const uint4 *)a.q_in, *gd = (const uint4 *)(a.q_in + (size_t)M * a.k);
+        auto where = [&](int i, int &dst) -> const uint4 * {
+            const int jt = i / 20, r = i - jt * 20, j = jt / nit, it = jt - j * nit;
+            dst = r < 16 ? jt * 16 + r : M * nit * 16 + jt * 4 + (r - 16);
+            return r < 16 ? gq + ((size_t)j * (a.k >> 4) + it * 64 + (r >> 3) * 32 + 8 * q + (r & 7))
+                          : gd + ((((size_t)j * nb + it * 32 + 8 * q) >> 1) + (r - 16));
+        };
+        for (int i0 = threadIdx.x; i0 < n; i0 += 4 * T) {    // four loads in flight per thread (past the end: the last unit again)
+            int d0, d1, d2, d3;
+            const uint4 *s0 = where(min(i0, n - 1), d0), *s1 = where(min(i0 + T, n - 1), d1);
+            const uint4 *s2 = where(min(i0 + 2 * T, n - 1), d2), *s3 = where(min(i0 + 3 * T, n - 1), d3);
+            const uint4 v0 = *s0, v1 = *s1, v2 = *s2, v3 = *s3;
+            __builtin_amdgcn_sched_barrier(0);
+            lq[d0] = v0; lq[d1] = v1; lq[d2] = v2; lq[d3] = v3;
+        }
+    }
+    __syncthreads();
+    if (row0 >= a.m) return;
+    float acc[M];
+    #pragma unroll
+    for (int j = 0; j < M; ++j) acc[j] = 0.0f;
+    for (int it0 = 0; it0 < nit; it0 += U) {
+        cur = nxt;
+        if (it0 + U < nit) fetch(nxt, it0 + U);
+        #pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (it0 + u < nit) {
+                const int it = it0 + u;
+                float2 ds[M]; int4 a0[M], a1[M];
+                #pragma unroll
+                for (int j = 0; j < M; ++j) {
+                    const int jt = j * nit + it;
+                    ds[j] = lds[jt * 8 + sg];
+                    a0[j] = *(const int4 *)(lq + jt * 16 + sg); a1[j] = *(const int4 *)(lq + jt * 16 + 8 + sg);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const float dw = lg_h2f((uint16_t)cur.s[u]);
+                #pragma unroll
+                for (int j = 0; j < M; ++j) {
+                    const int dot = lg_block_dot(cur.q[u], a0[j], a1[j], __float_as_int(ds[j].y));
+                    acc[j] = lg_fmaf(ds[j].x * dw, (float)dot, acc[j]);
+                }
+            }
+        }
+    }
+    #pragma unroll
+    for (int j = 0; j < M; ++j) acc[j] = lg_sum8(acc[j]);
+    if (sg < M && row0 + r8 < a.m) a.out[((size_t)q * M + sg) * a.m + row] = lg_pick<M>(acc, sg);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Attention tiles of a verify block for layers with many tiles (long global contexts, wide sliding windows):
 // one workgroup per (tile, kv head) serves ALL rows of the block against one staged K/V tile, where lg_k_attn
 // runs a workgroup per row and stages every tile once per row.  The queries arrive normed and rotated

@@ -164,7 +164,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -214,6 +214,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
     if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
+    if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
     *out = m;
@@ -689,17 +690,27 @@ static int cu_count() {
 // Plain matmul launch: picks the segment count from k and the workgroup shape from the row count
 // (small matrices get one wavefront per workgroup so that every CU has work).
 template <int M, bool DUMP>
-static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
+static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = false) {
     const int S = lg_segments(a.k), rw = 64 / S, ngroups = a.m / rw;
     if constexpr (M > LG_HIP_MAX_ROWS) {                 // wide (prefill) block: matrix-core kernels, 32 weight rows per workgroup
-        if (a.m % 32) { lx.rc = fail(-2, "wide matmul: %d rows is not a multiple of 32", a.m); return; }
+        if (a.m % 32) { lx.rc = fail(-2, "wide matmul: %d rows is not a multiple of 32", a.m); return 1; }
         // S = 32: four workgroups per row block, each a quarter of the K segments, writing its own slab of a.out
         const dim3 grid(a.m / 32, (M + LG_WIDE - 1) / LG_WIDE, S == 32 ? 4 : 1);
         if (S == 32) LAUNCH(cls, (lg_k_mm_wide<M, 32, DUMP>), grid, dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
         else         LAUNCH(cls, (lg_k_mm_wide<M, 8, DUMP>), grid, dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+        return S == 32 ? 4 : 1;
     } else {
     const size_t lds = lds_mm(M, a.k);
-    if (S == 32) {
+    if (S == 32 && M >= 4 && slabs_ok && !DUMP) {
+        // blocks of four and more rows whose consumer adds four slabs: cut by K quarter (a quarter of the activations
+        // per workgroup, several workgroups per CU).  12B shape, 5 rows: ffn_down 16.9 -> 14.3 us, the rows kernel that
+        // adds the slabs 6.6 -> 7.5 us, the step 3.814 -> 3.775 ms (2 and 5 wavefronts per workgroup: 3.827, 3.924)
+        if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
+            const int oct = (a.m + 7) / 8, W = 4;
+            LAUNCH(cls, (lg_k_mm_kq<M>), dim3((oct + W - 1) / W, 4), dim3(64 * W), (size_t)M * (a.k / 1024) * 320, a);
+        }
+        return 4;
+    } else if (S == 32) {
         // 4 wavefronts (8 rows) per workgroup, or 5 when that makes exactly one workgroup per CU (2560 rows on 256 CUs):
         // with 320 workgroups a quarter of the CUs would hold two of them and the kernel would wait for those
         const int cus = cu_count();
@@ -727,6 +738,7 @@ static void launch_mm(Launcher &lx, int cls, const MmArgs &a) {
     }
     }
     (void)rw; (void)ngroups;
+    return 1;
 }
 
 // one block of M rows through the decoder (and the head when with_head)
@@ -953,9 +965,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             else
                 LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, a);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
-            launch_mm<M, false>(lx, KC_DOWN, d);
+            // (the rows kernel adds four slabs; the fused rows + PLE gate kernel of verify blocks takes whole sums)
+            pend_parts = launch_mm<M, false>(lx, KC_DOWN, d, !m->ple && m->down_kq);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
-            pend_parts = (M > LG_HIP_MAX_ROWS && lg_segments(y.nff) == 32) ? 4 : 1;
         }
         if (m->ple && y.winp_f) {   // per-layer embedding block, matrices kept in a float type: residual update, then the
             // gate on the f32 rows (gelu(.) * ipl in its epilogue), then the projection of the f32 gate rows
@@ -1029,7 +1041,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1066,6 +1078,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
+    else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
 }

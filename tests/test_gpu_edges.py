@@ -137,12 +137,13 @@ def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
         gpu.close(); o.close()
 
 
-@pytest.mark.parametrize("rows", [2, 5])
-def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, rows):
+@pytest.mark.parametrize("rows,name,over", [(2, "tiny_full", {}), (5, "tiny_full", {}), (6, "tiny", {"n_ff": 5120})])
+def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, rows, name, over):
     """The options that pick between kernels for the same arithmetic (row work inside the q/k/v matmul, the
-    attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay) change
+    attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay, ffn_down
+    cut by K quarter: the last case has the long FFN rows and no per-layer embeddings that kernel is for) change
     timing only: every combination leaves the same cache rows and the same logits rows of a verify block."""
-    path, spec = model_path("tiny_full")
+    path, spec = model_path(name, **over)
     V = spec["n_vocab"]
     rng = np.random.default_rng(rows)
     prompt = rng.integers(0, V, 300).astype(np.int32)
@@ -163,10 +164,10 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, r
             gpu.close()
 
     base = run()
-    for name in ("fuse_rows", "attn_rows", "head_mfma", "wide_prefill", "use_graph"):
-        print(f"rows={rows} option {name}=0", flush=True)
-        got = run(**{name: 0})
-        assert got[0] == base[0] and np.array_equal(got[1], base[1]), name
-        assert np.array_equal(got[2].view(np.uint32), base[2].view(np.uint32)), name
+    for opt in ("fuse_rows", "attn_rows", "head_mfma", "wide_prefill", "use_graph", "down_kq"):
+        print(f"rows={rows} option {opt}=0", flush=True)
+        got = run(**{opt: 0})
+        assert got[0] == base[0] and np.array_equal(got[1], base[1]), opt
+        assert np.array_equal(got[2].view(np.uint32), base[2].view(np.uint32)), opt
         for a, b in zip(got[3], base[3]):
-            assert np.array_equal(a, b), name
+            assert np.array_equal(a, b), opt

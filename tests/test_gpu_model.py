@@ -97,13 +97,15 @@ def test_gpu_against_the_reference_fixture_teacher_forced(lg, ob, gpu_required, 
 
 @pytest.mark.parametrize("name,rows,over", [("tiny", 2, {}), ("tiny", 4, {}), ("tiny", 5, {}), ("tiny_full", 3, {}), ("tiny_full", 4, {}), ("tiny_full_f32", 5, {}), ("tiny_full_f16", 2, {}), ("tiny_full_bf16", 8, {}),
                                             ("tiny_full", 6, {}), ("tiny_full", 7, {}), ("tiny_full", 8, {}),
-                                            ("tiny", 5, {"head_dim_full": 512}), ("tiny_full", 8, {"head_dim_full": 256})])
+                                            ("tiny", 5, {"head_dim_full": 512}), ("tiny_full", 8, {"head_dim_full": 256}),
+                                            ("tiny", 4, {"n_ff": 5120}), ("tiny", 5, {"n_ff": 5120}), ("tiny", 7, {"n_ff": 5120}), ("tiny", 8, {"n_ff": 5120})])
 def test_verify_equals_decode_and_accept_counts(lg, ob, gpu_required, model_path, name, rows, over):
     """Row j of a verify block is bit-identical to a plain decode at pos+j (the reference's central
     invariant, src/cuda/model-cuda.cuh:520-526), and with drafts whose first mismatch is planted the
     accepted count is known in advance (the acceptance tripwire, bench/mtp-accept.ps1:1-4).  The last two
     cases widen the heads of the global layers (512: two registers per lane in the attention kernel's
-    query/key preparation; 256: one, full)."""
+    query/key preparation; 256: one, full); the cases with an FFN of 5120 give ffn_down rows of 32 K segments,
+    which blocks of 4 to 8 rows of a model without per-layer embeddings cut by K quarter over four workgroups."""
     path, spec = model_path(name, **over)
     V = spec["n_vocab"]
     rng = np.random.default_rng(rows)
