@@ -23,11 +23,13 @@
 #define LG_MAXV      16       // float4 per lane of a residual row: n_embd <= 4096
 #define LG_HIP_MAX_ROWS_DEV 8   // widest draft block (same value as LG_HIP_MAX_ROWS in lg_hip.h)
 
-// Loads of weight tiles.  A weight byte is read once per step and never again by the CU that loads it, so the
-// loads carry the non-temporal hint: the tiles then do not displace from the caches the small vectors that one
-// kernel of the step writes for the next one to read.  The weight kernels themselves run no faster for it, the
-// step as a whole does (E4B shape, 5 rows: 2.65 -> 2.53 ms); the scope bits (sc0 / sc1) on the same loads change
-// nothing.
+// Loads of weight tiles.  The weights of a step (gigabytes) pass through the memory-side cache once per step;
+// loaded plainly they push out of it what the step re-reads every time and what fits there: the K/V windows, the
+// norm vectors, the PLE gate tiles, the per-layer inputs.  With the non-temporal hint they do not, and the kernels
+// that read those (attention tiles, row kernels, PLE gate) run 0.2-0.4 us faster each while the weight kernels
+// themselves run no faster: E4B shape, 5 rows, 2.65 -> 2.53 ms per step.  Loading any one large matrix class plainly
+// again (ffn_down, or the attention output projection) gives most of that back; the scope bits (sc0 / sc1) on the same
+// loads change nothing, and non-temporal stores of kernel outputs gain nothing either.
 typedef unsigned lg_ntv4u __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 lg_ldw16(const void *p) {
     const lg_ntv4u v = __builtin_nontemporal_load((const lg_ntv4u *)p);
