@@ -67,101 +67,126 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
     const int n = lane & 31, h = lane >> 5, c = 8 * part + wave;
     // operands of row tile `tile` in the wide q8 layout (lg_q8_off): per 16-byte unit the two halves of the
     // 32 rows side by side, so lane (n, h) reads 8 of 512 consecutive bytes; rows past `rows` hold
-    // whatever the buffer holds and their results are dropped by the caller
-    const int8_t *atile = q_in + (size_t)tile * 32 * k + (size_t)(h * 32 + n) * 8;
-    const float2 *dstile = lg_q8_ds<R>(q_in, k) + (size_t)tile * 32 * nb + n;
+    // whatever the buffer holds and their results are dropped by the caller.
+    // Every load of the loop is a buffer load: a wavefront-uniform base (the row tile, the row block) in scalar
+    // registers, a 32-bit lane offset computed once, and the step's offset in a scalar register, so a step spends no
+    // vector instructions on addresses.
+    const auto rsrc = [](const void *base) {                 // (the bases are wavefront-uniform; said so, the descriptor lives in scalar registers)
+        const uint64_t b = (uint64_t)base;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+        return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, 0x7FFFFFFF, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t r_act = rsrc(q_in + (size_t)tile * 32 * k);
+    const __amdgpu_buffer_rsrc_t r_ds = rsrc(lg_q8_ds<R>(q_in, k) + (size_t)tile * 32 * nb);
+    const int vo_a0 = (h * 32 + n) * 8 + c * 512, vo_a1 = vo_a0 + S * 512, vo_d = (c * 32 + n) * 8;
 
     // wavefronts 0..3 fetch the step's 256 (row, segment) slots: slot -> tile, lane inside the tile, row of the block
     const int slot = (wave & 3) * 64 + lane;
-    int st_tile, st_lane, st_m, st_c;
-    const uint8_t *tbase;
+    int st_tile, st_lane, st_m, st_c, vo_w;
+    const uint8_t *wbase;
     if (RB) {       // slot = (segment, row): the 32 rows of block rb are lanes 32*(rb&1) .. +31 of tile (rb/2, segment*nit + it)
         st_c = slot >> 5; st_m = slot & 31; st_lane = 32 * (rb & 1) + st_m; st_tile = 0;
-        tbase = w + ((size_t)(rb >> 1) * nb + (size_t)st_c * nit) * LG_TILE;
+        wbase = w + (size_t)(rb >> 1) * nb * LG_TILE;
+        vo_w = st_c * nit * LG_TILE;
     } else {
         if (S == 8) { st_tile = slot >> 6; st_lane = slot & 63; st_m = st_tile * 8 + (st_lane >> 3); st_c = st_lane & 7; }
         else        { st_tile = slot >> 4; st_c = slot & 7; const int r = (slot >> 3) & 1; st_lane = r * 32 + 8 * part + st_c; st_m = st_tile * 2 + r; }
-        tbase = w + (size_t)(rb * TPB + st_tile) * nit * LG_TILE;
+        wbase = w + (size_t)rb * TPB * nit * LG_TILE;
+        vo_w = st_tile * nit * LG_TILE;
     }
-    // A chunk of U steps is requested while the previous one is consumed (enough bytes in flight to
-    // cover the memory latency), parked in LDS in one go, and followed by a single barrier.
-    uint4 tq[G::U]; uint32_t ts[G::U];
-    uint2 b0[G::U], b1[G::U], nb0[G::U], nb1[G::U]; float2 xs[G::U], nxs[G::U];
-    auto fetch = [&](int it0) {
-        #pragma unroll
-        for (int u = 0; u < G::U; ++u) {
-            const int it = it0 + u < nit ? it0 + u : nit - 1;    // clamp: never read past the row block
-            if (wave < 4) {
-                const uint8_t *t = tbase + (size_t)it * LG_TILE;
-                tq[u] = *(const uint4 *)(t + st_lane * 16);
-                ts[u] = *(const uint16_t *)(t + 1024 + st_lane * 2);
-            }
-            nb0[u] = *(const uint2 *)(atile + (size_t)(it * 2 * S + c) * 512);
-            nb1[u] = *(const uint2 *)(atile + (size_t)(it * 2 * S + S + c) * 512);
-            nxs[u] = dstile[(size_t)(it * S + c) * 32];
+    const __amdgpu_buffer_rsrc_t r_w = rsrc(wbase);
+    const int vo_wq = vo_w + st_lane * 16, vo_ws = vo_w + 1024 + st_lane * 2;
+    // What a step needs from memory: the lane's slot of the weight tiles (wavefronts 0..3), its 16 operand bytes of
+    // the activation block and the block's {scale, sum}.  Two sets, used in turn: step it+1 is requested before the
+    // barrier of step it and first waited for after the barrier of step it+1.
+    struct Ops { lg_v4i tq; uint32_t ts; uint2 b0, b1; float2 xs; };
+    auto fetch = [&](Ops &o, int it_) {
+        const int it = __builtin_amdgcn_readfirstlane(it_);   // (uniform: keeps the step offsets in scalar registers)
+        if (wave < 4) {
+            o.tq = __builtin_amdgcn_raw_buffer_load_b128(r_w, vo_wq, it * LG_TILE, 0);
+            o.ts = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r_w, vo_ws, it * LG_TILE, 0);
         }
+        const auto a0 = __builtin_amdgcn_raw_buffer_load_b64(r_act, vo_a0, it * (2 * S * 512), 0);
+        const auto a1 = __builtin_amdgcn_raw_buffer_load_b64(r_act, vo_a1, it * (2 * S * 512), 0);
+        const auto ds = __builtin_amdgcn_raw_buffer_load_b64(r_ds, vo_d, it * (S * 32 * 8), 0);
+        o.b0 = make_uint2((unsigned)a0[0], (unsigned)a0[1]); o.b1 = make_uint2((unsigned)a1[0], (unsigned)a1[1]);
+        o.xs = make_float2(__int_as_float(ds[0]), __int_as_float(ds[1]));
+    };
+    auto park = [&](const Ops &o, unsigned char *cbase) {     // the tile slots into LDS, in operand order
+        uint2 *aw = (uint2 *)cbase;
+        float *dwf = (float *)(cbase + G::aw_bytes);
+        aw[(st_c * 2 + 0) * G::AW_STRIDE + st_m] = make_uint2((unsigned)o.tq[0], (unsigned)o.tq[1]);
+        aw[(st_c * 2 + 1) * G::AW_STRIDE + st_m] = make_uint2((unsigned)o.tq[2], (unsigned)o.tq[3]);
+        dwf[st_c * 32 + st_m] = lg_h2f((uint16_t)o.ts);
     };
     float p[16];
     #pragma unroll
     for (int i = 0; i < 16; ++i) p[i] = 0.0f;
-    lg_v16i magic, acc;
+    lg_v16i magic;
     #pragma unroll
     for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;      // 12582912.0f
-    fetch(0);
-    for (int it0 = 0; it0 < nit; it0 += G::U) {
-        unsigned char *cbase = smem + (size_t)((it0 / G::U) & 1) * G::U * G::step_bytes;
-        if (wave < 4) {                                       // park in operand order
-            #pragma unroll
-            for (int u = 0; u < G::U; ++u) {
-                uint2 *aw = (uint2 *)(cbase + (size_t)u * G::step_bytes);
-                float *dwf = (float *)((unsigned char *)aw + G::aw_bytes);
-                aw[(st_c * 2 + 0) * G::AW_STRIDE + st_m] = make_uint2(tq[u].x, tq[u].y);
-                aw[(st_c * 2 + 1) * G::AW_STRIDE + st_m] = make_uint2(tq[u].z, tq[u].w);
-                dwf[st_c * 32 + st_m] = lg_h2f((uint16_t)ts[u]);
-            }
-        }
+    // kept in 16 registers of its own: left as a known constant the compiler rebuilds it in the accumulator
+    // registers before every MFMA (23 moves per step)
+    asm volatile("" : "+v"(magic));
+    auto compute = [&](const Ops &o, const unsigned char *cbase, int it) {
+        const uint2 *aw = (const uint2 *)cbase;
+        const float *dwf = (const float *)(cbase + G::aw_bytes);
+        // operand and the 16 weight scales of this lane's outputs: all five LDS reads go out together, ahead of the
+        // MFMA (interleaved with the epilogue, as the compiler would have them, each costs an LDS round trip)
+        const uint2 a = aw[(wave * 2 + h) * G::AW_STRIDE + n];
+        float4 d4[4];
         #pragma unroll
-        for (int u = 0; u < G::U; ++u) { b0[u] = nb0[u]; b1[u] = nb1[u]; xs[u] = nxs[u]; }
-        if (it0 + G::U < nit) fetch(it0 + G::U);
-        __syncthreads();
+        for (int g = 0; g < 4; ++g) d4[g] = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
+        __builtin_amdgcn_sched_barrier(0);
+        lg_v4i av, bv;
+        av[0] = (int)(a.x & 0x0F0F0F0Fu); av[1] = (int)(a.y & 0x0F0F0F0Fu);
+        av[2] = (int)((a.x >> 4) & 0x0F0F0F0Fu); av[3] = (int)((a.y >> 4) & 0x0F0F0F0Fu);
+        bv[0] = (int)o.b0.x; bv[1] = (int)o.b0.y; bv[2] = (int)o.b1.x; bv[3] = (int)o.b1.y;
+        // The accumulator starts at the bit pattern of 1.5 * 2^23: the integer dot (|dot| < 2^22) lands in the
+        // mantissa, so the result read as a float is 12582912 + dot exactly, and one float subtraction of
+        // 12582912 + 8*sum gives (float)(dot - 8*sum) exactly: one instruction per output instead of an
+        // integer subtract and a conversion.
+        const lg_v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, magic, 0, 0, 0);
+        const int corr = 8 * __float_as_int(o.xs.y);
+        const float cf = 12582912.0f + (float)corr;
         #pragma unroll
-        for (int u = 0; u < G::U; ++u) {
-            if (it0 + u >= nit) break;
-            const int it = it0 + u;
-            const uint2 *aw = (const uint2 *)(cbase + (size_t)u * G::step_bytes);
-            const float *dwf = (const float *)((const unsigned char *)aw + G::aw_bytes);
-            // operand and the 16 weight scales of this lane's outputs: all five LDS reads go out together, ahead of the
-            // MFMA (interleaved with the epilogue, as the compiler would have them, each costs an LDS round trip)
-            const uint2 a = aw[(wave * 2 + h) * G::AW_STRIDE + n];
-            float4 d4[4];
+        for (int g = 0; g < 4; ++g) {
+            const float dv[4] = { d4[g].x, d4[g].y, d4[g].z, d4[g].w };
             #pragma unroll
-            for (int g = 0; g < 4; ++g) d4[g] = *(const float4 *)(dwf + wave * 32 + 8 * g + 4 * h);
-            __builtin_amdgcn_sched_barrier(0);
-            lg_v4i av, bv;
-            av[0] = (int)(a.x & 0x0F0F0F0Fu); av[1] = (int)(a.y & 0x0F0F0F0Fu);
-            av[2] = (int)((a.x >> 4) & 0x0F0F0F0Fu); av[3] = (int)((a.y >> 4) & 0x0F0F0F0Fu);
-            bv[0] = (int)b0[u].x; bv[1] = (int)b0[u].y; bv[2] = (int)b1[u].x; bv[3] = (int)b1[u].y;
-            // The accumulator starts at the bit pattern of 1.5 * 2^23: the integer dot (|dot| < 2^22) lands in the
-            // mantissa, so the result read as a float is 12582912 + dot exactly, and one float subtraction of
-            // 12582912 + 8*sum gives (float)(dot - 8*sum) exactly: one instruction per output instead of an
-            // integer subtract and a conversion.
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, magic, 0, 0, 0);
-            const int corr = 8 * __float_as_int(xs[u].y);
-            const float cf = 12582912.0f + (float)corr;
-            #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float dv[4] = { d4[g].x, d4[g].y, d4[g].z, d4[g].w };
-                #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float fdot = __int_as_float(acc[4 * g + j]) - cf;
-                    if (DUMP) {
-                        const int row = 32 * rb + 8 * g + 4 * h + j;
-                        if (tile * LG_WIDE + n < rows) dots[((size_t)(tile * LG_WIDE + n) * m_total + row) * nb + (c * nit + it)] = (int)fdot;
-                    }
-                    p[4 * g + j] = lg_fmaf(xs[u].x * dv[j], fdot, p[4 * g + j]);
+            for (int j = 0; j < 4; ++j) {
+                const float fdot = __int_as_float(acc[4 * g + j]) - cf;
+                if (DUMP) {
+                    const int row = 32 * rb + 8 * g + 4 * h + j;
+                    if (tile * LG_WIDE + n < rows) dots[((size_t)(tile * LG_WIDE + n) * m_total + row) * nb + (c * nit + it)] = (int)fdot;
                 }
+                p[4 * g + j] = lg_fmaf(o.xs.x * dv[j], fdot, p[4 * g + j]);
             }
         }
+    };
+    Ops oa, ob;
+    unsigned char *const c0 = smem, *const c1 = smem + G::step_bytes;
+    fetch(oa, 0);
+    int it = 0;
+    // (no condition around a fetch inside the loop: with one, the wait for the older set has to assume that the newer
+    // one was never requested, and becomes a wait for everything)
+    for (; it + 2 < nit; it += 2) {
+        if (wave < 4) park(oa, c0);
+        fetch(ob, it + 1);
+        __syncthreads();
+        compute(oa, c0, it);
+        if (wave < 4) park(ob, c1);
+        fetch(oa, it + 2);
+        __syncthreads();
+        compute(ob, c1, it + 1);
+    }
+    if (wave < 4) park(oa, c0);                              // the last one or two steps
+    if (it + 1 < nit) fetch(ob, it + 1);
+    __syncthreads();
+    compute(oa, c0, it);
+    if (it + 1 < nit) {
+        if (wave < 4) park(ob, c1);
+        __syncthreads();
+        compute(ob, c1, it + 1);
     }
     // adjacent-pair tree over the eight segments (one per wavefront)
     __syncthreads();
