@@ -822,12 +822,20 @@ __global__ __launch_bounds__(512, HD > 256 ? 2 : 4) void lg_k_attn_u(AttnArgs a,
             #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 const int eb = __float_as_int(half ? e1 : e0);
-                #pragma unroll 8
-                for (int k = 0; k < 16; ++k) {
-                    const uint2 v = *(const uint2 *)(vl + (16 * half + k) * Geo::VS);
-                    const float es = __int_as_float(__builtin_amdgcn_readlane(eb, 4 * k));
-                    acc.x = lg_fma_hlo_s(es, v.x, acc.x); acc.y = lg_fma_hhi_s(es, v.x, acc.y);
-                    acc.z = lg_fma_hlo_s(es, v.y, acc.z); acc.w = lg_fma_hhi_s(es, v.y, acc.w);
+                // eight slots' values requested together, then their 32 fma (lane numbers of the weights are constants:
+                // left as a loop, every slot pays a scalar add, its wait states and an LDS round trip of its own)
+                #pragma unroll
+                for (int k0 = 0; k0 < 16; k0 += 8) {
+                    uint2 v[8];
+                    #pragma unroll
+                    for (int k = 0; k < 8; ++k) v[k] = *(const uint2 *)(vl + (16 * half + k0 + k) * Geo::VS);
+                    __builtin_amdgcn_sched_barrier(0);
+                    #pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const float es = __int_as_float(__builtin_amdgcn_readlane(eb, 4 * (k0 + k)));
+                        acc.x = lg_fma_hlo_s(es, v[k].x, acc.x); acc.y = lg_fma_hhi_s(es, v[k].x, acc.y);
+                        acc.z = lg_fma_hlo_s(es, v[k].y, acc.z); acc.w = lg_fma_hhi_s(es, v[k].y, acc.w);
+                    }
                 }
             }
             if (live) {
