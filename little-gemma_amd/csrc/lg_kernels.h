@@ -902,8 +902,11 @@ __device__ __forceinline__ HeadVec<NV> lg_head_load(const float *src, int hd) {
     HeadVec<NV> h;
     #pragma unroll
     for (int v = 0; v < NV; ++v) {
+        // lanes past the vector load its first elements and never use them (every sum and store below is guarded by
+        // the lane's range): an unconditional load, where a choice between the loaded value and zeros made the
+        // compiler wait for the first vector before it requested the next
         const int e0 = 256 * v + 4 * lane;
-        h.x[v] = e0 < hd ? *(const float4 *)(src + e0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        h.x[v] = *(const float4 *)(src + (e0 < hd ? e0 : 0));
     }
     return h;
 }
@@ -1070,7 +1073,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
     const int tnew = (FQ && a.kcw) ? ctl->pos : 0x7FFFFFFF;
     {   // stage q (G heads of this row) and the tile's K/V rows; loads are issued in groups ahead of
         // the LDS stores (named temporaries + scheduling barrier, see lg_copy_batched)
-        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
         HeadVec<NV> hq[2], hj[LG_ATTN_JOBS], wq, wk;
         RopeVals<NV> rv;
         int njobs = 0, r0 = 0;
@@ -1082,7 +1085,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
             rv = lg_rope_load<NV>(a.rope_tab, a.rope_ff, hd);
             const int rlo = t0 > tnew ? t0 - tnew : 0, rhi = (t0 + 31 < pj ? t0 + 31 : pj) - tnew;   // block rows in this tile
             if (pj >= tnew && rhi >= rlo) { njobs = rhi - rlo + 1; r0 = rlo; }
-            wk = njobs == 0 ? wq : lg_head_load<NV>(a.k_norm, hd);   // no K rows to build: k_norm may not exist
+            wk = lg_head_load<NV>(njobs == 0 ? a.q_norm : a.k_norm, hd);   // no K rows to build: k_norm may not exist (a choice of address, not of loaded values: that one waits for the loads)
             #pragma unroll
             for (int u = 0; u < LG_ATTN_JOBS; ++u) {          // slots 0,1: K rows wv, wv+4; slots 2,3: V rows 3-wv, 7-wv
                 const bool isv = u >= LG_ATTN_JOBS / 2;
