@@ -36,6 +36,13 @@ __device__ __forceinline__ uint4 lg_ldw16(const void *p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ uint16_t lg_ldw2(const void *p) { return __builtin_nontemporal_load((const uint16_t *)p); }
+// Buffer descriptor over memory that starts at a wavefront-uniform address (raw buffer, byte offsets, no bounds
+// to speak of): loads through it take the lane's offset in one vector register and a per-load offset in a scalar one.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t lg_buffer_rsrc(const void *base) {
+    const uint64_t b = (uint64_t)base;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, 0x7FFFFFFF, 0x00020000);
+}
 // Tile `it` of a wavefront's run of weight tiles: 16 bytes of nibbles per lane, and the lane's row scale.
 __device__ __forceinline__ uint4 lg_ldt16(const uint8_t *base, int it, int lane) { return lg_ldw16(base + (size_t)it * LG_TILE + lane * 16); }
 __device__ __forceinline__ uint16_t lg_ldt2(const uint8_t *base, int it, int lane) { return lg_ldw2(base + (size_t)it * LG_TILE + 1024 + lane * 2); }

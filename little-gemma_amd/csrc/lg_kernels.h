@@ -1236,42 +1236,55 @@ struct MergeArgs {
 };
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const StepCtl *ctl) {
-    __shared__ float wts[512];                                // exp(m_tile - M) of up to 512 tiles at a time
+    __shared__ float wts[512], pls[512];                      // exp(m_tile - M) and the sums of up to 512 tiles at a time
     const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
     const int pos = ctl->pos + a.pos_off, pj = pos + j;
     const int first = lg_win_start(pos, a.window) >> 5;
     const int lo = (lg_win_start(pj, a.window) >> 5) - first, hi = (pj >> 5) - first;
     const size_t base = ((size_t)j * a.H + head) * a.tiles_max;
-    float mx = -INFINITY;
-    for (int n = lo + (int)threadIdx.x; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
+    // rows with at most one tile per thread (every sliding layer, global layers up to 8192 keys) read each tile's
+    // maximum and sum once, with the pass that finds the row's maximum
+    const bool once = hi - lo < LG_WG;
+    const int mine = lo + (int)threadIdx.x <= hi ? lo + (int)threadIdx.x : hi;
+    const float pm1 = a.pm[base + mine], pl1 = a.pl[base + mine];
+    float mx = pm1;
+    for (int n = lo + (int)threadIdx.x + LG_WG; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
     mx = lg_max_n(mx, 64);
     __shared__ float wmx[LG_WG / 64];
     if ((threadIdx.x & 63) == 0) wmx[threadIdx.x >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
     float L = 0.0f, o[2] = { 0.0f, 0.0f };
+    const int tl = (int)threadIdx.x < hd ? (int)threadIdx.x : hd - 1;   // (lanes past a short head repeat its last dim; their sums are never used)
     for (int c0 = lo; c0 <= hi; c0 += 512) {
         const int cn = hi - c0 + 1 < 512 ? hi - c0 + 1 : 512;
-        __syncthreads();
-        for (int n = threadIdx.x; n < cn; n += LG_WG) wts[n] = lg_expf(a.pm[base + c0 + n] - mx);
+        if (once) {
+            if ((int)threadIdx.x < cn) { wts[threadIdx.x] = lg_expf(pm1 - mx); pls[threadIdx.x] = pl1; }
+        } else {
+            __syncthreads();
+            for (int n = threadIdx.x; n < cn; n += LG_WG) { wts[n] = lg_expf(a.pm[base + c0 + n] - mx); pls[n] = a.pl[base + c0 + n]; }
+        }
         __syncthreads();
         // a batch of partials is one memory round trip (they were written by other CUs a moment ago), so the
         // batch is made large enough to hold all the tiles of a sliding layer; fma in tile order
+        // (buffer loads: the row's partials as the base in scalar registers, the lane's dim as the lane offset, the
+        // tile's offset in a scalar register; as flat loads every one of them cost a dozen vector instructions of
+        // 64-bit address arithmetic ahead of the first fma)
         constexpr int U = 24;
+        const __amdgpu_buffer_rsrc_t rp = lg_buffer_rsrc(a.pacc + (base + c0) * hd);
         for (int n0 = 0; n0 < cn; n0 += U) {
-            float plu[U], pau[U], pbu[U];                     // sums, dims 0..255, dims 256..511 (hd = 512 only)
+            float pau[U], pbu[U];                             // dims 0..255, dims 256..511 (hd = 512 only)
             const bool wide = hd > LG_WG;
             #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int n = n0 + u < cn ? n0 + u : cn - 1;
-                plu[u] = a.pl[base + c0 + n];
-                pau[u] = (int)threadIdx.x < hd ? a.pacc[(base + c0 + n) * hd + threadIdx.x] : 0.0f;
+                const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
+                pau[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, tl * 4, n * hd * 4, 0));
             }
             if (wide) {
                 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int n = n0 + u < cn ? n0 + u : cn - 1;
-                    pbu[u] = a.pacc[(base + c0 + n) * hd + LG_WG + threadIdx.x];
+                    const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
+                    pbu[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, (LG_WG + (int)threadIdx.x) * 4, n * hd * 4, 0));
                 }
             }
             __builtin_amdgcn_sched_barrier(0);                // every load of the batch issued before the first fma waits
@@ -1279,7 +1292,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
             for (int u = 0; u < U; ++u) {
                 if (n0 + u < cn) {                            // (a guard, not a break: the arrays stay in registers)
                     const float wn = wts[n0 + u];
-                    L = lg_fmaf(plu[u], wn, L);
+                    L = lg_fmaf(pls[n0 + u], wn, L);
                     o[0] = lg_fmaf(pau[u], wn, o[0]);
                     if (wide) o[1] = lg_fmaf(pbu[u], wn, o[1]);
                 }

@@ -71,11 +71,7 @@ __device__ __forceinline__ void lg_mfma_block(const uint8_t *w, int k, int rb, i
     // Every load of the loop is a buffer load: a wavefront-uniform base (the row tile, the row block) in scalar
     // registers, a 32-bit lane offset computed once, and the step's offset in a scalar register, so a step spends no
     // vector instructions on addresses.
-    const auto rsrc = [](const void *base) {                 // (the bases are wavefront-uniform; said so, the descriptor lives in scalar registers)
-        const uint64_t b = (uint64_t)base;
-        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
-        return __builtin_amdgcn_make_buffer_rsrc((void *)(((uint64_t)hi << 32) | lo), 0, 0x7FFFFFFF, 0x00020000);
-    };
+    const auto rsrc = [](const void *base) { return lg_buffer_rsrc(base); };
     const __amdgpu_buffer_rsrc_t r_act = rsrc(q_in + (size_t)tile * 32 * k);
     const __amdgpu_buffer_rsrc_t r_ds = rsrc(lg_q8_ds<R>(q_in, k) + (size_t)tile * 32 * nb);
     const int vo_a0 = (h * 32 + n) * 8 + c * 512, vo_a1 = vo_a0 + S * 512, vo_d = (c * 32 + n) * 8;
