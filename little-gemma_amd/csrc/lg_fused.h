@@ -175,6 +175,7 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
     const int g0 = blockIdx.x * 2 + gsel, gi = g0 < ngroups ? g0 : ngroups - 1;
     const int it_lo = part * nit / KP, nt = (part + 1) * nit / KP - it_lo;
     const uint8_t *wg = a.w + (size_t)gi * nit * LG_TILE;
+    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, k);   // the rows first, then the tiles
     uint4 wq[TMAX]; uint32_t ws[TMAX];
     #pragma unroll
     for (int u = 0; u < TMAX; ++u) {
@@ -182,7 +183,8 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
         wq[u] = lg_ldt16(wg, it, lane);
         ws[u] = lg_ldt2(wg, it, lane);
     }
-    lg_load_q8<M>(a.q_in, k, lq);
+    __builtin_amdgcn_sched_barrier(0);
+    lg_load_q8_commit<M>(rows, a.q_in, k, lq);
     __syncthreads();
     const int c = lane & 7;
     float sc[TMAX][M], fd[TMAX][M];
@@ -302,12 +304,20 @@ __global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
             nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
-    if (np > 0) fetch(0, 0);
     unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
-    {   // the wavefront's K segment of the activations, once (wave-private, no barrier)
+    {   // the wavefront's K segment of the activations, once (wave-private, no barrier); its first loads go out
+        // ahead of the first weight tiles
         const uint4 *src = (const uint4 *)(a.q_in + (size_t)s * nit * (LG_MU_DWORDS * 4));
         const int nu = nit * (LG_MU_DWORDS / 4);
-        for (int i0 = lane; i0 < nu; i0 += 256) {
+        {   // (every lane takes part, past the end with the last unit again: the tiles are requested in here)
+            const int i0 = min(lane, nu - 1), i1 = min(lane + 64, nu - 1), i2 = min(lane + 128, nu - 1), i3 = min(lane + 192, nu - 1);
+            const uint4 t0v = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
+            __builtin_amdgcn_sched_barrier(0);
+            if (np > 0) fetch(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            ((uint4 *)la)[i0] = t0v; ((uint4 *)la)[i1] = t1; ((uint4 *)la)[i2] = t2; ((uint4 *)la)[i3] = t3;
+        }
+        for (int i0 = lane + 256; i0 < nu; i0 += 256) {
             const int i1 = min(i0 + 64, nu - 1), i2 = min(i0 + 128, nu - 1), i3 = min(i0 + 192, nu - 1);
             const uint4 t0v = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
             __builtin_amdgcn_sched_barrier(0);
@@ -413,8 +423,8 @@ __global__ __launch_bounds__(320, 2) void lg_k_mm_kq(MmArgs a) {
             w.s[u] = lg_ldw2(ws + (size_t)it * LG_TILE);
         }
     };
-    fetch(nxt, 0);                                            // (weights depend on nothing)
     {   // the quarter of the activations: per (row, tile) two runs of 8 units and one run of 8 {scale, sum} = 20 x 16 bytes
+        // (their first pass is requested ahead of the first weight tiles and stored after them: loads return in order)
         const int n = M * nit * 20, T = blockDim.x;
         const uint4 *gq = (const uint4 *)a.q_in, *gd = (const uint4 *)(a.q_in + (size_t)M * a.k);
         auto where = [&](int i, int &dst) -> const uint4 * {
@@ -423,7 +433,18 @@ __global__ __launch_bounds__(320, 2) void lg_k_mm_kq(MmArgs a) {
             return r < 16 ? gq + ((size_t)j * (a.k >> 4) + it * 64 + (r >> 3) * 32 + 8 * q + (r & 7))
                           : gd + ((((size_t)j * nb + it * 32 + 8 * q) >> 1) + (r - 16));
         };
-        for (int i0 = threadIdx.x; i0 < n; i0 += 4 * T) {    // four loads in flight per thread (past the end: the last unit again)
+        {   // four loads in flight per thread (past the end: the last unit again); every thread takes part in the first pass
+            const int i0 = threadIdx.x;
+            int d0, d1, d2, d3;
+            const uint4 *s0 = where(min(i0, n - 1), d0), *s1 = where(min(i0 + T, n - 1), d1);
+            const uint4 *s2 = where(min(i0 + 2 * T, n - 1), d2), *s3 = where(min(i0 + 3 * T, n - 1), d3);
+            const uint4 v0 = *s0, v1 = *s1, v2 = *s2, v3 = *s3;
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(nxt, 0);                                    // (weights depend on nothing)
+            __builtin_amdgcn_sched_barrier(0);
+            lq[d0] = v0; lq[d1] = v1; lq[d2] = v2; lq[d3] = v3;
+        }
+        for (int i0 = threadIdx.x + 4 * T; i0 < n; i0 += 4 * T) {
             int d0, d1, d2, d3;
             const uint4 *s0 = where(min(i0, n - 1), d0), *s1 = where(min(i0 + T, n - 1), d1);
             const uint4 *s2 = where(min(i0 + 2 * T, n - 1), d2), *s3 = where(min(i0 + 3 * T, n - 1), d3);

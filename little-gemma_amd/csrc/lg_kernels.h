@@ -102,6 +102,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) xv[v] = xr[t + 256 * v];
     }
+    const bool has_os = s.dout != nullptr && s.os != nullptr;
+    const float osv = has_os ? s.os[0] : 1.0f;               // (requested with the rows, not after the first sum)
     if (s.dout) {
         const float4 *dr = (const float4 *)(s.dout + (size_t)j * E), *wr = (const float4 *)s.w_post;
         #pragma unroll
@@ -127,8 +129,6 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
         ss = lg_block_sum256(ss, red[0]);
         const float sc = 1.0f / sqrtf(ss / (float)E + s.eps);
-        const bool has_os = s.os != nullptr;
-        const float osv = has_os ? s.os[0] : 1.0f;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
             const float4 w = wpost[v];
@@ -229,6 +229,30 @@ __device__ __forceinline__ void lg_copy_batched(const T *src, T *dst, int n) {
 template <int M>
 __device__ __forceinline__ void lg_load_q8(const int8_t *q, int k, int8_t *lq) {
     lg_copy_batched<uint4>((const uint4 *)q, (uint4 *)lq, M * k * 5 / 64);
+}
+// The same copy in two halves, for kernels that also have weight tiles to request: the rows' first batch is
+// requested first (lg_load_q8_issue), then the tiles, then the batch is stored and the rest copied
+// (lg_load_q8_commit).  Loads return in the order they were requested, so the rows (written a moment ago, on their
+// way from the memory-side cache) are in LDS while the tiles (from HBM) are still arriving; requested after the
+// tiles, the rows' stores wait for every tile.
+struct CopyBatch { uint4 t0, t1, t2, t3, t4, t5, t6, t7; };
+template <int M>
+__device__ __forceinline__ CopyBatch lg_load_q8_issue(const int8_t *q, int k) {
+    const uint4 *src = (const uint4 *)q;
+    const int nt = blockDim.x, last = M * k * 5 / 64 - 1, i0 = threadIdx.x;
+    CopyBatch b;
+    b.t0 = src[min(i0, last)]; b.t1 = src[min(i0 + nt, last)]; b.t2 = src[min(i0 + 2 * nt, last)]; b.t3 = src[min(i0 + 3 * nt, last)];
+    b.t4 = src[min(i0 + 4 * nt, last)]; b.t5 = src[min(i0 + 5 * nt, last)]; b.t6 = src[min(i0 + 6 * nt, last)]; b.t7 = src[min(i0 + 7 * nt, last)];
+    __builtin_amdgcn_sched_barrier(0);
+    return b;
+}
+template <int M>
+__device__ __forceinline__ void lg_load_q8_commit(const CopyBatch &b, const int8_t *q, int k, int8_t *lq) {
+    uint4 *dst = (uint4 *)lq;
+    const int nt = blockDim.x, n = M * k * 5 / 64, last = n - 1, i0 = threadIdx.x;
+    dst[min(i0, last)] = b.t0; dst[min(i0 + nt, last)] = b.t1; dst[min(i0 + 2 * nt, last)] = b.t2; dst[min(i0 + 3 * nt, last)] = b.t3;
+    dst[min(i0 + 4 * nt, last)] = b.t4; dst[min(i0 + 5 * nt, last)] = b.t5; dst[min(i0 + 6 * nt, last)] = b.t6; dst[min(i0 + 7 * nt, last)] = b.t7;
+    if (n > 8 * nt) lg_copy_batched<uint4>((const uint4 *)q + 8 * nt, dst + 8 * nt, n - 8 * nt);
 }
 
 // Input of a draft head (src/mtp.c:268-276): cat = [dequant(token_embd[token]) * sqrt(nb), h_prev],
@@ -366,9 +390,11 @@ __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
         wg[g] = a.w + (size_t)gi * nit * LG_TILE;
         row[g] = gi * RW + lane / S;
     }
+    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, a.k); // the rows first, then the tiles
     WChunk<G, U> first;
     lg_mm_fetch<G, U>(first, wg, 0, nit, lane);
-    lg_load_q8<M>(a.q_in, a.k, lq);
+    __builtin_amdgcn_sched_barrier(0);
+    lg_load_q8_commit<M>(rows, a.q_in, a.k, lq);
     __syncthreads();
     if (g0 >= ngroups) return;
     float acc[G][M];
@@ -523,13 +549,22 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
             nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
-    fetch(0);
     unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
     {
-        // four loads in flight per lane before the first store (left as a plain loop the copy is one round trip per 16 bytes)
+        // four loads in flight per lane before the first store (left as a plain loop the copy is one round trip per 16
+        // bytes); the first four are requested ahead of the first weight tiles and stored after them: loads return in
+        // the order they were requested, and the rows come from nearer than the tiles
         const uint4 *src = (const uint4 *)(a.q_in + (size_t)s * nit * (LG_MU_DWORDS * 4));
         const int nu = nit * (LG_MU_DWORDS / 4);
-        for (int i0 = lane; i0 < nu; i0 += 256) {
+        {
+            const int i0 = min(lane, nu - 1), i1 = min(lane + 64, nu - 1), i2 = min(lane + 128, nu - 1), i3 = min(lane + 192, nu - 1);
+            const uint4 t0 = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(0);
+            __builtin_amdgcn_sched_barrier(0);
+            ((uint4 *)la)[i0] = t0; ((uint4 *)la)[i1] = t1; ((uint4 *)la)[i2] = t2; ((uint4 *)la)[i3] = t3;
+        }
+        for (int i0 = lane + 256; i0 < nu; i0 += 256) {
             const int i1 = min(i0 + 64, nu - 1), i2 = min(i0 + 128, nu - 1), i3 = min(i0 + 192, nu - 1);
             const uint4 t0 = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3];
             __builtin_amdgcn_sched_barrier(0);
@@ -655,11 +690,21 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
     int8_t *lq = (int8_t *)smem;                              // one row: [E] int8, then [E/32] {scale, sum}
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
     float2 *lds = (float2 *)(smem + (size_t)E);
-    __shared__ float gbuf[32], ipl[32], red[4];
+    __shared__ float gbuf[32], red[4];
     const int j = blockIdx.y;
     const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
-    // the whole row group (nit <= 16 tiles) is requested before anything else: with this few workgroups the kernel
-    // is a chain of memory round trips, and fetching the tiles two at a time adds one per pair
+    // Every load of the kernel is requested up front, the row's first (loads return in order: the row work then starts
+    // while the tiles are still arriving), then the whole row group (nit <= 16 tiles: with this few workgroups the
+    // kernel is a chain of memory round trips, and fetching the tiles two at a time adds one per pair), then the
+    // per-layer input of the lane's gate column (kept in a register until the end: parked in LDS on arrival, it made
+    // the kernel wait for everything requested before it, ahead of the row's own loads).
+    const int t = threadIdx.x, nq = E >> 2;
+    float4 xv[LG_ROWV], dv[LG_ROWV], wp[LG_ROWV];
+    {
+        const float4 *wr = (const float4 *)a.w_post, *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; dv[v] = dr[t + 256 * v]; wp[v] = wr[t + 256 * v]; }
+    }
     uint4 wq[LG_MAXV]; uint32_t wsc[LG_MAXV];
     #pragma unroll
     for (int u = 0; u < LG_MAXV; ++u) {
@@ -668,13 +713,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
         wq[u] = *(const uint4 *)(wg[0] + (size_t)it * LG_TILE + lane * 16);
         wsc[u] = *(const uint16_t *)(wg[0] + (size_t)it * LG_TILE + 1024 + lane * 2);
     }
-    if (threadIdx.x < 32) ipl[threadIdx.x] = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + threadIdx.x];
+    const float iplv = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + wave * 8 + (lane >> 3)];   // of this lane's gate column
     {
-        const int t = threadIdx.x, nq = E >> 2;
-        float4 xv[LG_ROWV], dv[LG_ROWV], wp[LG_ROWV];
-        const float4 *wr = (const float4 *)a.w_post, *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
-        #pragma unroll
-        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; dv[v] = dr[t + 256 * v]; wp[v] = wr[t + 256 * v]; }
         float ss = 0.0f;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
@@ -710,7 +750,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
             }
         }
         p = lg_sum_seg<8>(p);
-        if (c == 0) gbuf[wave * 8 + (lane >> 3)] = lg_gelu(p) * ipl[wave * 8 + (lane >> 3)];
+        if (c == 0) gbuf[wave * 8 + (lane >> 3)] = lg_gelu(p) * iplv;
     }
     __syncthreads();
     if (threadIdx.x < 32) {
