@@ -1114,6 +1114,41 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
     {   // stage q (G heads of this row) and the tile's K/V rows; loads are issued in groups ahead of
         // the LDS stores (named temporaries + scheduling barrier, see lg_copy_batched)
         const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+        const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
+        // (per_row is a power of two and the tile's first ring row is wavefront-uniform: shifts and one scalar
+        // remainder, where a division per element cost a hundred vector instructions ahead of the tile's loads)
+        const int lgpr = 31 - __builtin_clz(per_row), ring0 = t0 % a.seq;
+        // element u of the batch that starts at i0: LDS offset (halves) in `lo`, cache offset in `go`, validity in `ok`
+        auto place = [&](int i0, int u, int &lo, int &lk, size_t &go, bool &ok, bool &own) {
+            const int idx = min(i0 + u * LG_WG, nk8 - 1);
+            const int sl = idx >> lgpr, e0 = (idx & (per_row - 1)) << 3, t = t0 + sl;
+            ok = t >= startj && t <= pj;
+            own = ok && t >= tnew;                            // a row of the block: built by `prepare`, not read from the cache
+            ok = ok && !own;
+            lo = sl * kst + e0; lk = sl * ksk + e0;
+            // the slot's ring row, whether the row is live or not: what a dead slot holds is read and zeroed below
+            int rr = ring0 + sl;
+            if (rr >= a.seq) rr -= a.seq;
+            if (rr >= a.seq) rr %= a.seq;                     // (rings of fewer than 32 rows)
+            go = (size_t)rr * a.kv_dim + (size_t)kvh * hd + e0;
+        };
+        auto keep = [](uint4 v, bool ok) {                   // zero the rows no query of this block may see
+            const uint32_t mk = ok ? 0xFFFFFFFFu : 0u;
+            return make_uint4(v.x & mk, v.y & mk, v.z & mk, v.w & mk);
+        };
+        auto putk = [&](int lk, uint4 v) {                   // four 4-byte stores: K rows are only 4-byte aligned
+            uint32_t *d = (uint32_t *)(kt + lk);
+            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+        };
+        // The tile's first batch (all of it up to 256-wide heads) is requested before anything else of this block:
+        // its addresses need nothing from memory, and placed after the row's vectors its address arithmetic reused
+        // their registers and waited for them.
+        int l0, l1, l2, l3, m0, m1, m2, m3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3, ow0, ow1, ow2, ow3;
+        place(threadIdx.x, 0, l0, m0, g0, ok0, ow0); place(threadIdx.x, 1, l1, m1, g1, ok1, ow1);
+        place(threadIdx.x, 2, l2, m2, g2, ok2, ow2); place(threadIdx.x, 3, l3, m3, g3, ok3, ow3);
+        const uint4 fk0 = a.kc4(g0), fk1 = a.kc4(g1), fk2 = a.kc4(g2), fk3 = a.kc4(g3);
+        const uint4 fv0 = a.vc4(g0), fv1 = a.vc4(g1), fv2 = a.vc4(g2), fv3 = a.vc4(g3);
+        __builtin_amdgcn_sched_barrier(0);
         HeadVec<NV> hq[2], hj[LG_ATTN_JOBS], wq, wk;
         RopeVals<NV> rv;
         int njobs = 0, r0 = 0;
@@ -1172,31 +1207,16 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, c
                 }
             }
         };
-        const int per_row = hd >> 3, nk8 = 32 * per_row;     // 16-byte chunks per tile row / per tile
-        for (int i0 = threadIdx.x; i0 < nk8; i0 += 4 * LG_WG) {
-            // element u of the batch: LDS offset (halves) in `lo`, cache offset in `go`, validity in `ok`
-            auto place = [&](int u, int &lo, int &lk, size_t &go, bool &ok, bool &own) {
-                const int idx = min(i0 + u * LG_WG, nk8 - 1);
-                const int sl = idx / per_row, e0 = (idx - sl * per_row) << 3, t = t0 + sl;
-                ok = t >= startj && t <= pj;
-                own = ok && t >= tnew;                        // a row of the block: built by `prepare`, not read from the cache
-                ok = ok && !own;
-                lo = sl * kst + e0; lk = sl * ksk + e0;
-                go = (size_t)((ok ? t : pj) % a.seq) * a.kv_dim + (size_t)kvh * hd + e0;
-            };
-            int l0, l1, l2, l3, m0, m1, m2, m3; size_t g0, g1, g2, g3; bool ok0, ok1, ok2, ok3, ow0, ow1, ow2, ow3;
-            place(0, l0, m0, g0, ok0, ow0); place(1, l1, m1, g1, ok1, ow1); place(2, l2, m2, g2, ok2, ow2); place(3, l3, m3, g3, ok3, ow3);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!ow0) { putk(m0, keep(fk0, ok0));  *(uint4 *)(vt + l0) = keep(fv0, ok0); }
+        if (!ow1) { putk(m1, keep(fk1, ok1));  *(uint4 *)(vt + l1) = keep(fv1, ok1); }
+        if (!ow2) { putk(m2, keep(fk2, ok2));  *(uint4 *)(vt + l2) = keep(fv2, ok2); }
+        if (!ow3) { putk(m3, keep(fk3, ok3));  *(uint4 *)(vt + l3) = keep(fv3, ok3); }
+        for (int i0 = threadIdx.x + 4 * LG_WG; i0 < nk8; i0 += 4 * LG_WG) {      // (512-wide heads: a second batch)
+            place(i0, 0, l0, m0, g0, ok0, ow0); place(i0, 1, l1, m1, g1, ok1, ow1); place(i0, 2, l2, m2, g2, ok2, ow2); place(i0, 3, l3, m3, g3, ok3, ow3);
             const uint4 k0 = a.kc4(g0), k1 = a.kc4(g1), k2 = a.kc4(g2), k3 = a.kc4(g3);
             const uint4 v0 = a.vc4(g0), v1 = a.vc4(g1), v2 = a.vc4(g2), v3 = a.vc4(g3);
             __builtin_amdgcn_sched_barrier(0);
-            auto keep = [](uint4 v, bool ok) {               // zero the rows no query of this block may see
-                const uint32_t mk = ok ? 0xFFFFFFFFu : 0u;
-                return make_uint4(v.x & mk, v.y & mk, v.z & mk, v.w & mk);
-            };
-            auto putk = [&](int lk, uint4 v) {               // four 4-byte stores: K rows are only 4-byte aligned
-                uint32_t *d = (uint32_t *)(kt + lk);
-                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
-            };
             if (!ow0) { putk(m0, keep(k0, ok0));  *(uint4 *)(vt + l0) = keep(v0, ok0); }
             if (!ow1) { putk(m1, keep(k1, ok1));  *(uint4 *)(vt + l1) = keep(v1, ok1); }
             if (!ow2) { putk(m2, keep(k2, ok2));  *(uint4 *)(vt + l2) = keep(v2, ok2); }
