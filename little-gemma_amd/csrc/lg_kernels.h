@@ -444,13 +444,20 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
             nwd[u] = lg_ldt2(wt, it, lane);
         }
     };
-    fetch(0);
     // The units were written by the previous kernel on other XCDs, so the first read of each 128-byte
     // unit from this XCD misses its L2; walked one unit ahead, those misses would queue up behind each
-    // other.  One vector load per unit, issued now, brings the segment's lines in side by side.
-    int touch = 0;
-    for (int i = lane; i < nunits; i += 64)
-        touch |= *(const volatile int *)((const int *)a.q_in + ((size_t)s * nunits + i) * 32);
+    // other.  One vector load per unit, issued now, brings the segment's lines in side by side.  They go out ahead
+    // of the first weight tiles and nothing waits for them before the end (a wait here would also be one for the tiles).
+    // (nunits <= 16: k <= 4096 and at most three rows.)  The load is written as an instruction of its own: a volatile
+    // load is followed by a wait for every load in flight, a plain one with no use before the end is moved there.  Its
+    // register stays reserved until the use at the end of the kernel, by when the loop's own waits for the later
+    // weight loads have also covered this older one.
+    int touch;
+    {
+        const int *tp = (const int *)a.q_in + ((size_t)s * nunits + (lane < nunits ? lane : nunits - 1)) * 32;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(touch) : "v"(tp) : "memory");
+    }
+    fetch(0);
     int cur[32], nxt[32];
     #pragma unroll
     for (int i = 0; i < 32; ++i) cur[i] = au[i];
