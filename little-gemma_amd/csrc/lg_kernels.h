@@ -848,6 +848,24 @@ __global__ __launch_bounds__(LG_WG) void lg_k_accept(AcceptArgs a, StepCtl *ctl)
     __shared__ int si[LG_HIP_MAX_ROWS_DEV][LG_WG / 64];
     __shared__ int s_adv;
     const int step = ctl->step, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the block's tokens and this thread's slice of every row's hidden state are requested with the partials: read
+    // when they are needed (the tokens one after the other in the accept loop, the accepted row after it) each costs
+    // a memory round trip of its own at the end of the step
+    int tk[M];
+    #pragma unroll
+    for (int j = 0; j < M; ++j) tk[j] = a.toks[(size_t)step * M + j];
+    constexpr int HS = 4;                                     // float4 per thread and row: E <= 4096
+    float4 hrow[M][HS];
+    const bool hregs = a.E <= HS * 4 * LG_WG && (a.E & 3) == 0;
+    if (hregs) {
+        #pragma unroll
+        for (int j = 0; j < M; ++j)
+            #pragma unroll
+            for (int u = 0; u < HS; ++u) {
+                const int q4 = (int)threadIdx.x + u * LG_WG;
+                hrow[j][u] = ((const float4 *)(a.hidden_rows + (size_t)j * a.E))[q4 < (a.E >> 2) ? q4 : 0];
+            }
+    }
     float v[M]; int idx[M];
     #pragma unroll
     for (int j = 0; j < M; ++j) { v[j] = -INFINITY; idx[j] = 0x7fffffff; }
@@ -875,16 +893,27 @@ __global__ __launch_bounds__(LG_WG) void lg_k_accept(AcceptArgs a, StepCtl *ctl)
                 if (sv[j][w] > bv || (sv[j][w] == bv && si[j][w] < bi)) { bv = sv[j][w]; bi = si[j][w]; }
             best[j] = bi;
         }
-        const int32_t *tk = a.toks + (size_t)step * M;
         int adv = 1;
-        while (adv < M && best[adv - 1] == tk[adv]) adv++;
+        #pragma unroll
+        for (int j = 1; j < M; ++j) if (adv == j && best[j - 1] == tk[j]) adv = j + 1;
         for (int j = 0; j < M; ++j) a.out[(size_t)step * M + j] = best[j];
         a.adv[step] = adv;
         s_adv = adv;
     }
     __syncthreads();
     const int adv = s_adv;
-    for (int i = threadIdx.x; i < a.E; i += LG_WG) a.g_hidden[i] = a.hidden_rows[(size_t)(adv - 1) * a.E + i];
+    if (hregs) {
+        #pragma unroll
+        for (int u = 0; u < HS; ++u) {
+            const int q4 = (int)threadIdx.x + u * LG_WG;
+            float4 h = hrow[0][u];
+            #pragma unroll
+            for (int j = 1; j < M; ++j) if (adv - 1 == j) h = hrow[j][u];
+            if (q4 < (a.E >> 2)) ((float4 *)a.g_hidden)[q4] = h;
+        }
+    } else {
+        for (int i = threadIdx.x; i < a.E; i += LG_WG) a.g_hidden[i] = a.hidden_rows[(size_t)(adv - 1) * a.E + i];
+    }
     __syncthreads();
     if (threadIdx.x == 0) { ctl->pos += adv; ctl->step = step + 1; }
 }
