@@ -886,11 +886,15 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge_split(MergeArgs a, cons
     const int nt = hi - lo + 1;
     constexpr int U = 64;
     float pa[U];
-    auto fetch = [&](int t0) {                                // tiles t0 .. t0+63 of this row (past the end: the last one again)
+    // (buffer loads: the row's partials as the base in scalar registers, the lane's dim as the lane offset, the tile's
+    // offset in a scalar register; a flat load each cost a dozen vector instructions of 64-bit address arithmetic)
+    const __amdgpu_buffer_rsrc_t rp = lg_buffer_rsrc(a.pacc + base * hd);
+    auto fetch = [&](int t0_) {                               // tiles t0 .. t0+63 of this row (past the end: the last one again)
+        const int t0 = __builtin_amdgcn_readfirstlane(t0_);
         #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int n = t0 + u < nt ? t0 + u : nt - 1;
-            pa[u] = a.pacc[(base + n) * hd + d];
+            pa[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, d * 4, n * hd * 4, 0));
         }
     };
     fetch(wave * U);                                          // the partials do not depend on the weights
