@@ -724,10 +724,12 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
     } else if (M >= 4 && a.k >= 2048 && !DUMP) {
         // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over two wavefronts
-        // (over four was no faster)
+        // (over four was no faster at 8 and 10 tiles per group)
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
             const size_t l2 = ((lds + 15) & ~(size_t)15) + (size_t)2 * M * 64 * 4;
-            LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
+            // (over four wavefronts from 12 tiles per group on: 12B shape, k = 3840 and 4096, 3.662 -> 3.645 ms per step)
+            if ((a.k >> 8) >= 12) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, a);
+            else                  LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
         }
     } else {
         // Two row groups per workgroup when there are very many groups, and for blocks of 4+ rows when one group per

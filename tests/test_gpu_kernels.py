@@ -45,7 +45,8 @@ def test_matmul_config2_full_size(lg, ob, gpu_required, rows):
     assert np.abs(r["out"] - want).max() <= 1e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("m,k,rows", [(8, 256, 1), (2560, 10240, 5), (2048, 256, 8), (512, 3840, 3), (264, 15360, 8)])
+@pytest.mark.parametrize("m,k,rows", [(8, 256, 1), (2560, 10240, 5), (2048, 256, 8), (512, 3840, 3), (264, 15360, 8),
+                                      (512, 3840, 5), (264, 4096, 8), (72, 3072, 4)])   # (the last three: a row group's tiles cut over four wavefronts)
 def test_matmul_edge_shapes(lg, ob, gpu_required, m, k, rows):
     rng = np.random.default_rng(m + k)
     w = random_q4_0(rng, m, k)
