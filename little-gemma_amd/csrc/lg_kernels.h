@@ -241,8 +241,11 @@ __device__ __forceinline__ CopyBatch lg_load_q8_issue(const int8_t *q, int k) {
     const uint4 *src = (const uint4 *)q;
     const int nt = blockDim.x, last = M * k * 5 / 64 - 1, i0 = threadIdx.x;
     CopyBatch b;
-    b.t0 = src[min(i0, last)]; b.t1 = src[min(i0 + nt, last)]; b.t2 = src[min(i0 + 2 * nt, last)]; b.t3 = src[min(i0 + 3 * nt, last)];
-    b.t4 = src[min(i0 + 4 * nt, last)]; b.t5 = src[min(i0 + 5 * nt, last)]; b.t6 = src[min(i0 + 6 * nt, last)]; b.t7 = src[min(i0 + 7 * nt, last)];
+    b.t0 = src[min(i0, last)]; b.t1 = src[min(i0 + nt, last)];
+    if (last >= 2 * nt) {                                     // (short rows, k = 256: two units per thread hold them all)
+        b.t2 = src[min(i0 + 2 * nt, last)]; b.t3 = src[min(i0 + 3 * nt, last)];
+        b.t4 = src[min(i0 + 4 * nt, last)]; b.t5 = src[min(i0 + 5 * nt, last)]; b.t6 = src[min(i0 + 6 * nt, last)]; b.t7 = src[min(i0 + 7 * nt, last)];
+    }
     __builtin_amdgcn_sched_barrier(0);
     return b;
 }
@@ -250,8 +253,11 @@ template <int M>
 __device__ __forceinline__ void lg_load_q8_commit(const CopyBatch &b, const int8_t *q, int k, int8_t *lq) {
     uint4 *dst = (uint4 *)lq;
     const int nt = blockDim.x, n = M * k * 5 / 64, last = n - 1, i0 = threadIdx.x;
-    dst[min(i0, last)] = b.t0; dst[min(i0 + nt, last)] = b.t1; dst[min(i0 + 2 * nt, last)] = b.t2; dst[min(i0 + 3 * nt, last)] = b.t3;
-    dst[min(i0 + 4 * nt, last)] = b.t4; dst[min(i0 + 5 * nt, last)] = b.t5; dst[min(i0 + 6 * nt, last)] = b.t6; dst[min(i0 + 7 * nt, last)] = b.t7;
+    dst[min(i0, last)] = b.t0; dst[min(i0 + nt, last)] = b.t1;
+    if (last >= 2 * nt) {
+        dst[min(i0 + 2 * nt, last)] = b.t2; dst[min(i0 + 3 * nt, last)] = b.t3;
+        dst[min(i0 + 4 * nt, last)] = b.t4; dst[min(i0 + 5 * nt, last)] = b.t5; dst[min(i0 + 6 * nt, last)] = b.t6; dst[min(i0 + 7 * nt, last)] = b.t7;
+    }
     if (n > 8 * nt) lg_copy_batched<uint4>((const uint4 *)q + 8 * nt, dst + 8 * nt, n - 8 * nt);
 }
 
