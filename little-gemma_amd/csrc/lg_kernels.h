@@ -1349,6 +1349,31 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
     const bool once = hi - lo < LG_WG;
     const int mine = lo + (int)threadIdx.x <= hi ? lo + (int)threadIdx.x : hi;
     const float pm1 = a.pm[base + mine], pl1 = a.pl[base + mine];
+    // a batch of partials is one memory round trip (they were written by other CUs a moment ago), so the batch is
+    // made large enough to hold all the tiles of a sliding layer.  Buffer loads: the row's partials as the base in
+    // scalar registers, the lane's dim as the lane offset, the tile's offset in a scalar register (as flat loads every
+    // one of them cost a dozen vector instructions of 64-bit address arithmetic).  The first batch does not depend on
+    // the weights and is requested here, with the maxima.
+    constexpr int U = 24;
+    float pau[U], pbu[U];                                     // dims 0..255, dims 256..511 (hd = 512 only)
+    const bool wide = hd > LG_WG;
+    const int tl = (int)threadIdx.x < hd ? (int)threadIdx.x : hd - 1;   // (lanes past a short head repeat its last dim; their sums are never used)
+    auto fetch = [&](int c0, int cn, int n0) {
+        const __amdgpu_buffer_rsrc_t rp = lg_buffer_rsrc(a.pacc + (base + c0) * hd);
+        #pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
+            pau[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, tl * 4, n * hd * 4, 0));
+        }
+        if (wide) {
+            #pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
+                pbu[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, (LG_WG + (int)threadIdx.x) * 4, n * hd * 4, 0));
+            }
+        }
+    };
+    fetch(lo, hi - lo + 1 < 512 ? hi - lo + 1 : 512, 0);
     float mx = pm1;
     for (int n = lo + (int)threadIdx.x + LG_WG; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
     mx = lg_max_n(mx, 64);
@@ -1357,7 +1382,6 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
     __syncthreads();
     mx = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
     float L = 0.0f, o[2] = { 0.0f, 0.0f };
-    const int tl = (int)threadIdx.x < hd ? (int)threadIdx.x : hd - 1;   // (lanes past a short head repeat its last dim; their sums are never used)
     for (int c0 = lo; c0 <= hi; c0 += 512) {
         const int cn = hi - c0 + 1 < 512 ? hi - c0 + 1 : 512;
         if (once) {
@@ -1367,28 +1391,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const Step
             for (int n = threadIdx.x; n < cn; n += LG_WG) { wts[n] = lg_expf(a.pm[base + c0 + n] - mx); pls[n] = a.pl[base + c0 + n]; }
         }
         __syncthreads();
-        // a batch of partials is one memory round trip (they were written by other CUs a moment ago), so the
-        // batch is made large enough to hold all the tiles of a sliding layer; fma in tile order
-        // (buffer loads: the row's partials as the base in scalar registers, the lane's dim as the lane offset, the
-        // tile's offset in a scalar register; as flat loads every one of them cost a dozen vector instructions of
-        // 64-bit address arithmetic ahead of the first fma)
-        constexpr int U = 24;
-        const __amdgpu_buffer_rsrc_t rp = lg_buffer_rsrc(a.pacc + (base + c0) * hd);
-        for (int n0 = 0; n0 < cn; n0 += U) {
-            float pau[U], pbu[U];                             // dims 0..255, dims 256..511 (hd = 512 only)
-            const bool wide = hd > LG_WG;
-            #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
-                pau[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, tl * 4, n * hd * 4, 0));
-            }
-            if (wide) {
-                #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
-                    pbu[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, (LG_WG + (int)threadIdx.x) * 4, n * hd * 4, 0));
-                }
-            }
+        for (int n0 = 0; n0 < cn; n0 += U) {                  // fma in tile order
+            if (c0 != lo || n0 != 0) fetch(c0, cn, n0);
             __builtin_amdgcn_sched_barrier(0);                // every load of the batch issued before the first fma waits
             #pragma unroll
             for (int u = 0; u < U; ++u) {
