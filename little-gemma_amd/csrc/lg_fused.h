@@ -127,8 +127,10 @@ struct RowsMmArgs {
     MmArgs  mm;
     RowWork rows;
 };
+#define LG_ROWSMM_FIELDS(X, v) X(const float *, rx, rows.x, v) X(const float *, rdout, rows.dout, v) X(const float *, rw_post, rows.w_post, v) X(const float *, rw_pre, rows.w_pre, v) X(const uint8_t *, mw, mm.w, v) X(int, rE, rows.E, v) X(int, mk, mm.k, v) X(int, mm_, mm.m, v) X(const float *, ros, rows.os, v) X(float *, rx_out, rows.x_out, v) X(float, reps, rows.eps, v) X(float *, mout, mm.out, v) X(const int8_t *, mq_in, mm.q_in, v) X(int32_t *, mdots, mm.dots, v)
 template <int M, int NV, int NW>
-__global__ __launch_bounds__(LG_WG) void lg_k_rows_mm(RowsMmArgs a) {
+__global__ __launch_bounds__(LG_WG) void lg_k_rows_mm(LG_ROWSMM_FIELDS(LG_XP, _) int p_end_) {
+    RowsMmArgs a; LG_ROWSMM_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float red[2 * LG_HIP_MAX_ROWS_DEV * 4];
     const int k = a.mm.k;
@@ -164,7 +166,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_mm(RowsMmArgs a) {
 // chain p = fma(xd*dw, (float)dot, p) then runs through the parts in order (part p starts from the value part
 // p-1 left in LDS), so every sum is formed in the order of lg_mm_groups and the result is the same bits.
 template <int M, int KP>
-__global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(MmArgs a) {
+__global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(LG_MM_FIELDS(LG_XP, _) int p_end_) {
+    MmArgs a; LG_MM_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int TMAX = (16 + KP - 1) / KP;                  // k <= 4096: at most 16 tiles per group
     const int k = a.k, nb = k >> 5, nit = nb >> 3, ngroups = a.m >> 3;
@@ -286,7 +289,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_mmf(MmfArgs a) {
 // first tiles of the next block are requested while the last of this one are multiplied, and the segment sums
 // go through one of two LDS buffers in turn, so a block costs one barrier.
 template <int M>
-__global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
+__global__ __launch_bounds__(512, 2) void lg_k_head_m(LG_HEAD_FIELDS(LG_XP, _) int p_end_) {
+    HeadArgs a; LG_HEAD_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];     // [8 segments][nit][80 dwords]
     __shared__ float red[2][8][LG_HIP_MAX_ROWS_DEV][64];
     constexpr int CH = 2;
@@ -401,7 +405,8 @@ __global__ __launch_bounds__(512, 2) void lg_k_head_m(HeadArgs a) {
 // which is the bottom of the 32-segment tree.  The quarter's partial sums go to slab q of `out` ([4][M][m]); the
 // consumer adds the top of the tree, (p0+p1)+(p2+p3).
 template <int M>
-__global__ __launch_bounds__(320, 2) void lg_k_mm_kq(MmArgs a) {
+__global__ __launch_bounds__(320, 2) void lg_k_mm_kq(LG_MM_FIELDS(LG_XP, _) int p_end_) {
+    MmArgs a; LG_MM_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int q = blockIdx.y, nb = a.k >> 5, nit = nb >> 5;
@@ -526,7 +531,8 @@ struct AttnRowsGeo {
     }
 };
 template <int M, int HD>
-__global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(AttnArgs a, const StepCtl *ctl, int tp) {
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int tp, LG_ATTN_FIELDS(LG_XP, _) int p_end_) {
+    AttnArgs a; LG_ATTN_FIELDS(LG_XI, a)
     using Geo = AttnRowsGeo<HD>;
     extern __shared__ __align__(16) unsigned char smem[];
     const int G = a.H / a.nkv, units = M * G;
@@ -875,7 +881,8 @@ __global__ __launch_bounds__(512, HD > 256 ? 2 : 4) void lg_k_attn_u(AttnArgs a,
 // order, each running its 64 fma back to back from registers and handing (L, o) to the next through LDS.  Same
 // order, same bits: weights exp(m_t - M), L and the output as fma chains over the tiles ascending, divide, q8.
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge_split(MergeArgs a, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge_split(const StepCtl *ctl, LG_MERGE_FIELDS(LG_XP, _) int p_end_) {
+    MergeArgs a; LG_MERGE_FIELDS(LG_XI, a)
     __shared__ float wts[256], pls[256], hand[2][64], wmx[4];
     const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int d = blockIdx.z * 64 + lane;                     // hd is a multiple of 64

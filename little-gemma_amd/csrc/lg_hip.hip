@@ -707,7 +707,7 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         // adds the slabs 6.6 -> 7.5 us, the step 3.814 -> 3.775 ms (2 and 5 wavefronts per workgroup: 3.827, 3.924)
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
             const int oct = (a.m + 7) / 8, W = 4;
-            LAUNCH(cls, (lg_k_mm_kq<M>), dim3((oct + W - 1) / W, 4), dim3(64 * W), (size_t)M * (a.k / 1024) * 320, a);
+            LAUNCH(cls, (lg_k_mm_kq<M>), dim3((oct + W - 1) / W, 4), dim3(64 * W), (size_t)M * (a.k / 1024) * 320, LG_MM_FIELDS(LG_XA, a) 0);
         }
         return 4;
     } else if (S == 32) {
@@ -717,26 +717,26 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         const int W = (ngroups % 5 == 0 && ngroups / 5 <= cus && ngroups / 4 > cus) ? 5 : 4;
         // chunks of four tiles for the longest rows (15 tiles per lane at k = 15360: 3.96 against 4.00 ms per step at
         // the 12B shape), of two otherwise (10 tiles at k = 10240: 2.602 against 2.618 ms at the E4B shape)
-        if ((a.k >> 5) / 32 >= 12) LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP, 4>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
-        else                       LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
+        if ((a.k >> 5) / 32 >= 12) LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP, 4>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
+        else                       LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     } else if (ngroups >= 4096) {
         const int W = 4;
-        LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, a);
+        LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     } else if (M >= 4 && a.k >= 2048 && !DUMP) {
         // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over two wavefronts
         // (over four was no faster at 8 and 10 tiles per group)
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
             const size_t l2 = ((lds + 15) & ~(size_t)15) + (size_t)2 * M * 64 * 4;
             // (over four wavefronts from 12 tiles per group on: 12B shape, k = 3840 and 4096, 3.662 -> 3.645 ms per step)
-            if ((a.k >> 8) >= 12) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, a);
-            else                  LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, a);
+            if ((a.k >> 8) >= 12) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, LG_MM_FIELDS(LG_XA, a) 0);
+            else                  LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, LG_MM_FIELDS(LG_XA, a) 0);
         }
     } else {
         // Two row groups per workgroup when there are very many groups, and for blocks of 4+ rows when one group per
         // workgroup would leave some CUs with two of them: their activations (16 KB at M = 5) are then staged twice
         // on the CUs that set the kernel's time.  (Short rows, k < 1024, have too little to stage for that to matter.)
         const int W = (ngroups >= 1024 || (M >= 4 && a.k >= 1024 && ngroups > cu_count())) ? 2 : 1;
-        LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, a);
+        LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     }
     }
     (void)rw; (void)ngroups;
@@ -827,7 +827,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
         // verify blocks: the tail of the row work (store, norm weight, q8) cut over one workgroup per float4 of a lane
         const int slices = M <= LG_HIP_MAX_ROWS ? (E + 1023) / 1024 : 1;
-        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, s, m->ctl);
+        LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, m->ctl, LG_ROW_FIELDS(LG_XA, s) 0);
         if (s.x_out) cur ^= 1;
         have_x = true; pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
     };
@@ -852,10 +852,10 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             const dim3 grid((a.m / 8 + NW - 1) / NW);
             const size_t lds = lds_mm(M, a.k);
             switch (NVr) {
-                case 1: LAUNCH(cls, (lg_k_rows_mm<M, 1, NW>), grid, dim3(LG_WG), lds, f); break;
-                case 2: LAUNCH(cls, (lg_k_rows_mm<M, 2, NW>), grid, dim3(LG_WG), lds, f); break;
-                case 3: LAUNCH(cls, (lg_k_rows_mm<M, 3, NW>), grid, dim3(LG_WG), lds, f); break;
-                default: LAUNCH(cls, (lg_k_rows_mm<M, 4, NW>), grid, dim3(LG_WG), lds, f); break;
+                case 1: LAUNCH(cls, (lg_k_rows_mm<M, 1, NW>), grid, dim3(LG_WG), lds, LG_ROWSMM_FIELDS(LG_XA, f) 0); break;
+                case 2: LAUNCH(cls, (lg_k_rows_mm<M, 2, NW>), grid, dim3(LG_WG), lds, LG_ROWSMM_FIELDS(LG_XA, f) 0); break;
+                case 3: LAUNCH(cls, (lg_k_rows_mm<M, 3, NW>), grid, dim3(LG_WG), lds, LG_ROWSMM_FIELDS(LG_XA, f) 0); break;
+                default: LAUNCH(cls, (lg_k_rows_mm<M, 4, NW>), grid, dim3(LG_WG), lds, LG_ROWSMM_FIELDS(LG_XA, f) 0); break;
             }
             row_work_done();
         }
@@ -931,23 +931,23 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                     const size_t lds = y.hd == 256 ? AttnRowsGeo<256>::bytes(M * G) : y.hd == 128 ? AttnRowsGeo<128>::bytes(M * G) : AttnRowsGeo<64>::bytes(M * G);
                     const int tp = attention_rows_tp(tiles, y.nkv);
                     const dim3 grid((tiles + tp - 1) / tp, y.nkv);
-                    if (y.hd == 256)      LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
-                    else if (y.hd == 128) LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
-                    else                  LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), lds, a, m->ctl, tp);
+                    if (y.hd == 256)      LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+                    else if (y.hd == 128) LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+                    else                  LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
                 }
             } else
             if (fused_post) {
                 a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
                 a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
                 a.kcw = y.owns ? kv->k[L] : nullptr; a.vcw = y.owns ? kv->v[L] : nullptr; a.eps = m->eps;
-                if (y.hd <= 256) LAUNCH(KC_ATTN, (lg_k_attn<true, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
-                else             LAUNCH(KC_ATTN, (lg_k_attn<true, 2>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), a, m->ctl);
+                if (y.hd <= 256) LAUNCH(KC_ATTN, (lg_k_attn<true, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), m->ctl, LG_ATTN_FIELDS(LG_XA, a) 0);
+                else             LAUNCH(KC_ATTN, (lg_k_attn<true, 2>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, true), m->ctl, LG_ATTN_FIELDS(LG_XA, a) 0);
             } else {
-                LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), a, m->ctl);
+                LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), m->ctl, LG_ATTN_FIELDS(LG_XA, a) 0);
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
-            if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(LG_WG), 0, g, m->ctl);
-            else LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, g, m->ctl);
+            if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(LG_WG), 0, m->ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
+            else LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, m->ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
         }
         {   // attention output projection
             MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, nullptr };
@@ -963,9 +963,9 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
             else if constexpr (mfma)
-                LAUNCH(KC_GATEUP, (lg_k_geglu_m<M>), dim3(y.nff / 32), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, a);
+                LAUNCH(KC_GATEUP, (lg_k_geglu_m<M>), dim3(y.nff / 32), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, LG_GEGLU_FIELDS(LG_XA, a) 0);
             else
-                LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, a);
+                LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, LG_GEGLU_FIELDS(LG_XA, a) 0);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
             // (the rows kernel adds four slabs; the fused rows + PLE gate kernel of verify blocks takes whole sums)
             pend_parts = launch_mm<M, false>(lx, KC_DOWN, d, !m->ple && m->down_kq);
@@ -988,7 +988,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             } else {
                 // the residual update after ffn_down and its q8 happen inside the gate kernel (no rows kernel here)
                 RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps };
-                LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32, M), dim3(LG_WG), lds_mm(1, E), r);
+                LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32, M), dim3(LG_WG), lds_mm(1, E), LG_RPG_FIELDS(LG_XA, r) 0);
                 cur ^= 1;
                 pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
             }
@@ -1012,11 +1012,11 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         HeadArgs h{ head_m ? m->emb_rb : m->emb, E, m->n_vocab, passes, m->hq, m->softcap, m->store_logits ? m->logits : nullptr, m->pval, m->pidx };
         if (head_m) {
             if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS)
-                LAUNCH(KC_HEAD, (lg_k_head_m<M>), dim3(grid), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, h);
+                LAUNCH(KC_HEAD, (lg_k_head_m<M>), dim3(grid), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, LG_HEAD_FIELDS(LG_XA, h) 0);
         } else
-        LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(grid), dim3(LG_WG), lds_mm(M, E), h);
+        LAUNCH(KC_HEAD, (lg_k_mm_head<M>), dim3(grid), dim3(LG_WG), lds_mm(M, E), LG_HEAD_FIELDS(LG_XA, h) 0);
         AcceptArgs c{ m->pval, m->pidx, grid, m->sched, m->out, m->adv, m->hidden_rows, m->g_hidden, E };
-        LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), dim3(LG_WG), 0, c, m->ctl);
+        LAUNCH(KC_ACCEPT, (lg_k_accept<M>), dim3(1), dim3(LG_WG), 0, m->ctl, LG_ACCEPT_FIELDS(LG_XA, c) 0);
     } else if (!lx.rc && !dry) {
         hipLaunchKernelGGL(lg_k_advance, dim3(1), dim3(1), 0, m->stream, m->ctl, M);
     }
@@ -1530,7 +1530,7 @@ static int read_back_q8(const int8_t *dq, int rows, int k, int8_t *xq, float *xd
 template <int M>
 static void rows_isolated(hipStream_t st, const RowArgs &s, StepCtl *ctl) {
     const int slices = (s.E + 1023) / 1024;                   // as a verify step launches it: the tail sliced over workgroups
-    hipLaunchKernelGGL((lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, st, s, ctl);
+    hipLaunchKernelGGL((lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, st, ctl, LG_ROW_FIELDS(LG_XA, s) 0);
 }
 extern "C" int lg_hip_rows_norm_q8(const float *x, const float *dout, const float *w_post, const float *out_scale,
                                    const float *w_pre, int rows, int E, float eps, float *x_out, float *h_out,
@@ -1576,13 +1576,13 @@ static int enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs 
             if (rc) return rc;
             const int tp = attention_rows_tp(tiles, a.nkv);
             const dim3 grid((tiles + tp - 1) / tp, a.nkv);
-            if (a.hd == 256)      hipLaunchKernelGGL((lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
-            else if (a.hd == 128) hipLaunchKernelGGL((lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
-            else                  hipLaunchKernelGGL((lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), l2, st, a, ctl, tp);
+            if (a.hd == 256)      hipLaunchKernelGGL((lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), l2, st, ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+            else if (a.hd == 128) hipLaunchKernelGGL((lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), l2, st, ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+            else                  hipLaunchKernelGGL((lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), l2, st, ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
         }
-    } else hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, a, ctl);
-    if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && a.hd % 64 == 0) hipLaunchKernelGGL((lg_k_attn_merge_split<M>), dim3(a.H, M, a.hd / 64), dim3(LG_WG), 0, st, g, ctl);
-    else hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, g, ctl);
+    } else hipLaunchKernelGGL((lg_k_attn<false, 1>), dim3(tiles, a.nkv, M), dim3(LG_WG), lds, st, ctl, LG_ATTN_FIELDS(LG_XA, a) 0);
+    if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && a.hd % 64 == 0) hipLaunchKernelGGL((lg_k_attn_merge_split<M>), dim3(a.H, M, a.hd / 64), dim3(LG_WG), 0, st, ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
+    else hipLaunchKernelGGL((lg_k_attn_merge<M>), dim3(a.H, M), dim3(LG_WG), 0, st, ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
     return 0;
 }
 

@@ -25,6 +25,16 @@ struct StepCtl {            // device-resident step state
 //           ->  q8(h) in global memory (+ optional f32 copy h_out).
 // The row lives in registers as float4 per lane; lane l holds elements 256*v + 4*l .. +3, which
 // is also the lane assignment of the defined sum-of-squares order.
+// Kernel arguments are passed one by one, not as a struct: the first dozen dwords of a kernel's arguments can be
+// handed to its wavefronts in scalar registers at launch (-amdgpu-kernarg-preload-count), which a struct passed by
+// value is not, and a kernel whose first loads need only those starts them without waiting for a load of its
+// arguments.  Each argument struct lists its fields once, most urgent first (LG_*_FIELDS: type, parameter name,
+// member); the lists expand to the kernel's parameters (LG_XP), to the arguments of a launch (LG_XA) and to the
+// struct's reassembly inside the kernel (LG_XI), so the kernel bodies and the host code keep using the structs.
+#define LG_XP(T, id, mem, v) T p_##id,
+#define LG_XA(T, id, mem, v) (v).mem,
+#define LG_XI(T, id, mem, v) (v).mem = p_##id;
+
 struct RowArgs {
     const float   *x;        // [M][E] residual stream; nullptr when the rows are embeddings
     const float   *dout;     // [M][E] previous sub-layer output to be rmsnormed and added, or nullptr
@@ -43,6 +53,7 @@ struct RowArgs {
     int            E;
     float          eps;
 };
+#define LG_ROW_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(int, E, E, v) X(int, dparts, dparts, v) X(const float *, os, os, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(float, eps, eps, v) X(const uint8_t *, emb, emb, v) X(const int32_t *, toks, toks, v) X(int, emb_nit, emb_nit, v) X(int, emb_seg, emb_seg, v) X(float, emb_scale, emb_scale, v)
 
 // Sum over the 256 lanes of a workgroup in adjacent-pair tree order; every thread gets the result.
 // `scratch4` must not be in use by an earlier call that other wavefronts may still be reading: each call
@@ -81,7 +92,8 @@ __device__ __forceinline__ size_t lg_q8_ds_idx(int k, int j, int b) {
 #define LG_MU_DWORDS 80                     // dwords per block of the lg_k_geglu_m activation order
 #define LG_ROWV ((LG_MAXV + 3) / 4)        // float4 per thread of a residual row, 256 threads per row
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_rows(RowArgs s, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG) void lg_k_rows(const StepCtl *ctl, LG_ROW_FIELDS(LG_XP, _) int p_end_) {
+    RowArgs s; LG_ROW_FIELDS(LG_XI, s)
     __shared__ float red[2][4];
     const int t = threadIdx.x, j = blockIdx.x;
     // gridDim.y > 1: every workgroup of a row forms the row's sums, workgroup y stores and quantizes only the
@@ -375,12 +387,14 @@ struct MmArgs {
     const int8_t  *q_in;     // q8 activation buffer of the M input rows
     int32_t       *dots;     // DUMP only: [M][m][k/32]
 };
+#define LG_MM_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, m, m, v) X(float *, out, out, v) X(int32_t *, dots, dots, v)
 
 // Plain matmul: out[j][i] f32.  blockDim = 64*W wavefronts, each wavefront takes G neighbouring
 // row groups (G*64/S rows); grid covers ceil(groups / (W*G)) workgroups.
 // U: weight tiles per chunk (requested together, the next chunk while the current one is consumed)
 template <int M, int S, int G, bool DUMP, int U = LG_U>
-__global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(MmArgs a) {
+__global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(LG_MM_FIELDS(LG_XP, _) int p_end_) {
+    MmArgs a; LG_MM_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
@@ -419,6 +433,7 @@ struct GegluArgs {
     const int8_t  *q_in;     // verify blocks: unit order (below); wide blocks: lg_q8_off
     int8_t        *gq;       // q8 activation buffer of the result, width n_ff
 };
+#define LG_GEGLU_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, n_ff, n_ff, v) X(int8_t *, gq, gq, v)
 // Gate/up + GeGLU for verify blocks (M <= 8): a wavefront is 64 weight rows x one of
 // the 8 K segments, so every lane of it multiplies its own weight block with the SAME activation
 // block.  The activations then travel through the scalar cache into SGPRs (loads from the constant
@@ -430,7 +445,8 @@ struct GegluArgs {
 // 3 x {scale, sum}, 2 unused; a unit is requested while the previous one is consumed.
 typedef const __attribute__((address_space(4))) int *lg_cint;
 template <int M>
-__global__ __launch_bounds__(512, 2) void lg_k_geglu_t(GegluArgs a) {
+__global__ __launch_bounds__(512, 2) void lg_k_geglu_t(LG_GEGLU_FIELDS(LG_XP, _) int p_end_) {
+    GegluArgs a; LG_GEGLU_FIELDS(LG_XI, a)
     __shared__ float red[8][M][64];
     constexpr int NU = (M + 2) / 3, CH = 2;
     const int lane = threadIdx.x & 63;
@@ -545,7 +561,8 @@ typedef int lg_v4i __attribute__((ext_vector_type(4)));
 typedef int lg_v16i __attribute__((ext_vector_type(16)));
 typedef unsigned lg_v2u __attribute__((ext_vector_type(2)));
 template <int M>
-__global__ __launch_bounds__(512, 2) void lg_k_geglu_m(GegluArgs a) {
+__global__ __launch_bounds__(512, 2) void lg_k_geglu_m(LG_GEGLU_FIELDS(LG_XP, _) int p_end_) {
+    GegluArgs a; LG_GEGLU_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];     // [8 segments][nit][80 dwords]
     __shared__ float red[8][LG_HIP_MAX_ROWS_DEV][64];
     constexpr int CH = 2;
@@ -697,8 +714,10 @@ struct RowsPleGateArgs {
     float         *x_out;               // [M][E]
     float          eps;
 };
+#define LG_RPG_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const uint8_t *, gw, g.w, v) X(int, gk, g.k, v) X(int, gple, g.ple, v) X(const float *, gipl, g.ipl, v) X(int, glayer, g.layer, v) X(int, gnl, g.n_layer, v) X(int8_t *, gpq, g.pq, v) X(const int8_t *, gq_in, g.q_in, v) X(float *, x_out, x_out, v) X(float, eps, eps, v)
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(RowsPleGateArgs a) {
+__global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, _) int p_end_) {
+    RowsPleGateArgs a; LG_RPG_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;                              // one row: [E] int8, then [E/32] {scale, sum}
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
@@ -787,8 +806,10 @@ struct HeadArgs {
     float *logits;          // [M][n_vocab] or nullptr
     float *pval; int *pidx; // [gridDim.x][M]
 };
+#define LG_HEAD_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, n_vocab, n_vocab, v) X(int, passes, passes, v) X(float, softcap, softcap, v) X(float *, logits, logits, v) X(float *, pval, pval, v) X(int *, pidx, pidx, v)
 template <int M>
-__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_head(HeadArgs a) {
+__global__ __launch_bounds__(LG_WG, 2) void lg_k_mm_head(LG_HEAD_FIELDS(LG_XP, _) int p_end_) {
+    HeadArgs a; LG_HEAD_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
@@ -848,8 +869,10 @@ struct AcceptArgs {
     int32_t *adv;            // [n_steps]
     const float *hidden_rows; float *g_hidden; int E;
 };
+#define LG_ACCEPT_FIELDS(X, v) X(const float *, pval, pval, v) X(const int *, pidx, pidx, v) X(int, n_part, n_part, v) X(int, E, E, v) X(const int32_t *, toks, toks, v) X(const float *, hidden_rows, hidden_rows, v) X(int32_t *, out, out, v) X(int32_t *, adv, adv, v) X(float *, g_hidden, g_hidden, v)
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_accept(AcceptArgs a, StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG) void lg_k_accept(StepCtl *ctl, LG_ACCEPT_FIELDS(LG_XP, _) int p_end_) {
+    AcceptArgs a; LG_ACCEPT_FIELDS(LG_XI, a)
     __shared__ float sv[LG_HIP_MAX_ROWS_DEV][LG_WG / 64];
     __shared__ int si[LG_HIP_MAX_ROWS_DEV][LG_WG / 64];
     __shared__ int s_adv;
@@ -1114,6 +1137,7 @@ struct AttnArgs {
     __device__ __forceinline__ uint4 kc4s(size_t off) const { return lg_ldw16(kc + off); }
     __device__ __forceinline__ uint4 vc4s(size_t off) const { return lg_ldw16(vc + off); }
 };
+#define LG_ATTN_FIELDS(X, v) X(int, H, H, v) X(int, nkv, nkv, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int, seq, seq, v) X(int, kv_dim, kv_dim, v) X(const uint16_t *, kc, kc, v) X(const uint16_t *, vc, vc, v) X(const float *, qkv, qkv, v) X(const float *, q_norm, q_norm, v) X(const float *, k_norm, k_norm, v) X(const float *, rope_tab, rope_tab, v) X(const float *, rope_ff, rope_ff, v) X(int, ld, ld, v) X(int, k_off, k_off, v) X(int, v_off, v_off, v) X(uint16_t *, kcw, kcw, v) X(uint16_t *, vcw, vcw, v) X(const float *, q, q, v) X(float *, pm, pm, v) X(float *, pl, pl, v) X(float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(float, eps, eps, v)
 
 __device__ __forceinline__ int lg_win_start(int pos, int window) {
     return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -1131,7 +1155,8 @@ __device__ __forceinline__ int lg_win_start(int pos, int window) {
 // The ring has at least LG_WIDE_ROWS spare rows, so no row another workgroup still reads is overwritten.
 #define LG_ATTN_JOBS (2 * ((LG_HIP_MAX_ROWS_DEV + 3) / 4)) // K and V rows one wavefront may have to build
 template <bool FQ, int NV>
-__global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(AttnArgs a, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(const StepCtl *ctl, LG_ATTN_FIELDS(LG_XP, _) int p_end_) {
+    AttnArgs a; LG_ATTN_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
     const int hd = a.hd, G = a.H / a.nkv;
     const int kst = hd + 8;                                   // padded V tile row (halves): 16-byte rows, read along the row
@@ -1336,8 +1361,10 @@ struct MergeArgs {
     int8_t *xq;                // q8 activation buffer of the attention output, width H*hd (input of attn_output)
     float *xf;                 // optional f32 copy [M][H*hd]
 };
+#define LG_MERGE_FIELDS(X, v) X(const float *, pm, pm, v) X(const float *, pl, pl, v) X(const float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(int, H, H, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int8_t *, xq, xq, v) X(float *, xf, xf, v)
 template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(MergeArgs a, const StepCtl *ctl) {
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_MERGE_FIELDS(LG_XP, _) int p_end_) {
+    MergeArgs a; LG_MERGE_FIELDS(LG_XI, a)
     __shared__ float wts[512], pls[512];                      // exp(m_tile - M) and the sums of up to 512 tiles at a time
     const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
     const int pos = ctl->pos + a.pos_off, pj = pos + j;
