@@ -178,7 +178,7 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(LG_MM_FIELDS(LG_XP, _) in
     const int g0 = blockIdx.x * 2 + gsel, gi = g0 < ngroups ? g0 : ngroups - 1;
     const int it_lo = part * nit / KP, nt = (part + 1) * nit / KP - it_lo;
     const uint8_t *wg = a.w + (size_t)gi * nit * LG_TILE;
-    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, k);   // the rows first, then the tiles
+    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, k, 128 * KP);   // the rows first, then the tiles
     uint4 wq[TMAX]; uint32_t ws[TMAX];
     #pragma unroll
     for (int u = 0; u < TMAX; ++u) {
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(128 * KP) void lg_k_mm_ks(LG_MM_FIELDS(LG_XP, _) in
         ws[u] = lg_ldt2(wg, it, lane);
     }
     __builtin_amdgcn_sched_barrier(0);
-    lg_load_q8_commit<M>(rows, a.q_in, k, lq);
+    lg_load_q8_commit<M>(rows, a.q_in, k, lq, 128 * KP);
     __syncthreads();
     const int c = lane & 7;
     float sc[TMAX][M], fd[TMAX][M];
@@ -408,7 +408,7 @@ template <int M>
 __global__ __launch_bounds__(320, 2) void lg_k_mm_kq(LG_MM_FIELDS(LG_XP, _) int p_end_) {
     MmArgs a; LG_MM_FIELDS(LG_XI, a)
     extern __shared__ __align__(16) unsigned char smem[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = a.nthreads >> 6;
     const int q = blockIdx.y, nb = a.k >> 5, nit = nb >> 5;
     uint4 *lq = (uint4 *)smem;                                // [M][nit][2 halves][8 segments] 16-byte units
     float2 *lds = (float2 *)(smem + (size_t)M * nit * 256);   // [M][nit][8 segments] {scale, sum}
@@ -430,7 +430,7 @@ __global__ __launch_bounds__(320, 2) void lg_k_mm_kq(LG_MM_FIELDS(LG_XP, _) int 
     };
     {   // the quarter of the activations: per (row, tile) two runs of 8 units and one run of 8 {scale, sum} = 20 x 16 bytes
         // (their first pass is requested ahead of the first weight tiles and stored after them: loads return in order)
-        const int n = M * nit * 20, T = blockDim.x;
+        const int n = M * nit * 20, T = a.nthreads;
         const uint4 *gq = (const uint4 *)a.q_in, *gd = (const uint4 *)(a.q_in + (size_t)M * a.k);
         auto where = [&](int i, int &dst) -> const uint4 * {
             const int jt = i / 20, r = i - jt * 20, j = jt / nit, it = jt - j * nit;

@@ -690,7 +690,8 @@ static int cu_count() {
 // Plain matmul launch: picks the segment count from k and the workgroup shape from the row count
 // (small matrices get one wavefront per workgroup so that every CU has work).
 template <int M, bool DUMP>
-static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = false) {
+static int launch_mm(Launcher &lx, int cls, const MmArgs &a_in, bool slabs_ok = false) {
+    MmArgs a = a_in;                                      // (+ the workgroup size of the launch, set below)
     const int S = lg_segments(a.k), rw = 64 / S, ngroups = a.m / rw;
     if constexpr (M > LG_HIP_MAX_ROWS) {                 // wide (prefill) block: matrix-core kernels, 32 weight rows per workgroup
         if (a.m % 32) { lx.rc = fail(-2, "wide matmul: %d rows is not a multiple of 32", a.m); return 1; }
@@ -707,6 +708,7 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         // adds the slabs 6.6 -> 7.5 us, the step 3.814 -> 3.775 ms (2 and 5 wavefronts per workgroup: 3.827, 3.924)
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
             const int oct = (a.m + 7) / 8, W = 4;
+            a.nthreads = 64 * W;
             LAUNCH(cls, (lg_k_mm_kq<M>), dim3((oct + W - 1) / W, 4), dim3(64 * W), (size_t)M * (a.k / 1024) * 320, LG_MM_FIELDS(LG_XA, a) 0);
         }
         return 4;
@@ -717,10 +719,12 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         const int W = (ngroups % 5 == 0 && ngroups / 5 <= cus && ngroups / 4 > cus) ? 5 : 4;
         // chunks of four tiles for the longest rows (15 tiles per lane at k = 15360: 3.96 against 4.00 ms per step at
         // the 12B shape), of two otherwise (10 tiles at k = 10240: 2.602 against 2.618 ms at the E4B shape)
+        a.nthreads = 64 * W;
         if ((a.k >> 5) / 32 >= 12) LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP, 4>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
         else                       LAUNCH(cls, (lg_k_mm<M, 32, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     } else if (ngroups >= 4096) {
         const int W = 4;
+        a.nthreads = 64 * W;
         LAUNCH(cls, (lg_k_mm<M, 8, 2, DUMP>), dim3((ngroups + 2 * W - 1) / (2 * W)), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     } else if (M >= 4 && a.k >= 2048 && !DUMP) {
         // blocks of four and more rows: two row groups per workgroup, the tiles of each cut over two wavefronts
@@ -728,6 +732,7 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
             const size_t l2 = ((lds + 15) & ~(size_t)15) + (size_t)2 * M * 64 * 4;
             // (over four wavefronts from 12 tiles per group on: 12B shape, k = 3840 and 4096, 3.662 -> 3.645 ms per step)
+            a.nthreads = (a.k >> 8) >= 12 ? 512 : 256;
             if ((a.k >> 8) >= 12) LAUNCH(cls, (lg_k_mm_ks<M, 4>), dim3((ngroups + 1) / 2), dim3(512), l2, LG_MM_FIELDS(LG_XA, a) 0);
             else                  LAUNCH(cls, (lg_k_mm_ks<M, 2>), dim3((ngroups + 1) / 2), dim3(256), l2, LG_MM_FIELDS(LG_XA, a) 0);
         }
@@ -736,6 +741,7 @@ static int launch_mm(Launcher &lx, int cls, const MmArgs &a, bool slabs_ok = fal
         // workgroup would leave some CUs with two of them: their activations (16 KB at M = 5) are then staged twice
         // on the CUs that set the kernel's time.  (Short rows, k < 1024, have too little to stage for that to matter.)
         const int W = (ngroups >= 1024 || (M >= 4 && a.k >= 1024 && ngroups > cu_count())) ? 2 : 1;
+        a.nthreads = 64 * W;
         LAUNCH(cls, (lg_k_mm<M, 8, 1, DUMP>), dim3((ngroups + W - 1) / W), dim3(64 * W), lds, LG_MM_FIELDS(LG_XA, a) 0);
     }
     }
@@ -827,6 +833,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
         // verify blocks: the tail of the row work (store, norm weight, q8) cut over one workgroup per float4 of a lane
         const int slices = M <= LG_HIP_MAX_ROWS ? (E + 1023) / 1024 : 1;
+        s.slices = slices;
         LAUNCH(KC_ROWS, (lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, m->ctl, LG_ROW_FIELDS(LG_XA, s) 0);
         if (s.x_out) cur ^= 1;
         have_x = true; pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
@@ -916,6 +923,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             a.kc = kv->k[y.src]; a.vc = kv->v[y.src]; a.seq = kv->seq[y.src]; a.kv_dim = y.kd; a.window = window;
             a.pm = kv->pm; a.pl = kv->pl; a.pacc = kv->pacc; a.tiles_max = kv->tiles_max; a.pos_off = pos_off;
             const int tiles = layer_tiles(L);
+            a.gx = tiles; a.gz = M;
             const bool shared = rows_shared(L);
             // prompt blocks (the queries arrive prepared: lg_k_qkv_post ran): eight (row, head) units per workgroup with the
             // queries in registers
@@ -1528,8 +1536,10 @@ static int read_back_q8(const int8_t *dq, int rows, int k, int8_t *xq, float *xd
 }
 
 template <int M>
-static void rows_isolated(hipStream_t st, const RowArgs &s, StepCtl *ctl) {
+static void rows_isolated(hipStream_t st, const RowArgs &s_in, StepCtl *ctl) {
+    RowArgs s = s_in;
     const int slices = (s.E + 1023) / 1024;                   // as a verify step launches it: the tail sliced over workgroups
+    s.slices = slices;
     hipLaunchKernelGGL((lg_k_rows<M>), dim3(M, slices), dim3(LG_WG), 0, st, ctl, LG_ROW_FIELDS(LG_XA, s) 0);
 }
 extern "C" int lg_hip_rows_norm_q8(const float *x, const float *dout, const float *w_post, const float *out_scale,
@@ -1567,7 +1577,9 @@ extern "C" int lg_hip_rows_norm_q8(const float *x, const float *dout, const floa
 // (the same choice of kernels as a verify step makes: many (tile, kv head) pairs -> one workgroup per pair serves all
 // rows; many tiles per row -> the merge is cut by dims)
 template <int M>
-static int enqueue_attention(hipStream_t st, const AttnArgs &a, const MergeArgs &g, StepCtl *ctl, int tiles, size_t lds) {
+static int enqueue_attention(hipStream_t st, const AttnArgs &a_in, const MergeArgs &g, StepCtl *ctl, int tiles, size_t lds) {
+    AttnArgs a = a_in;
+    a.gx = tiles; a.gz = M;                               // the grid of lg_k_attn, which reads it from its arguments
     if (attention_rows_shared(M, tiles, a.nkv, a.hd, a.seq)) {
         if constexpr (M > 1 && M <= LG_HIP_MAX_ROWS) {
             const int units = M * (a.H / a.nkv);

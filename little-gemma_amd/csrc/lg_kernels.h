@@ -52,8 +52,9 @@ struct RowArgs {
     float          emb_scale;
     int            E;
     float          eps;
+    int            slices;   // workgroups per row (gridDim.y): as an argument it arrives with the others, the launch dimensions need a load of their own
 };
-#define LG_ROW_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(int, E, E, v) X(int, dparts, dparts, v) X(const float *, os, os, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(float, eps, eps, v) X(const uint8_t *, emb, emb, v) X(const int32_t *, toks, toks, v) X(int, emb_nit, emb_nit, v) X(int, emb_seg, emb_seg, v) X(float, emb_scale, emb_scale, v)
+#define LG_ROW_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(int, E, E, v) X(int, dparts, dparts, v) X(int, slices, slices, v) X(const float *, os, os, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(float, eps, eps, v) X(const uint8_t *, emb, emb, v) X(const int32_t *, toks, toks, v) X(int, emb_nit, emb_nit, v) X(int, emb_seg, emb_seg, v) X(float, emb_scale, emb_scale, v)
 
 // Sum over the 256 lanes of a workgroup in adjacent-pair tree order; every thread gets the result.
 // `scratch4` must not be in use by an earlier call that other wavefronts may still be reading: each call
@@ -98,11 +99,11 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(const StepCtl *ctl, LG_ROW_FI
     const int t = threadIdx.x, j = blockIdx.x;
     // gridDim.y > 1: every workgroup of a row forms the row's sums, workgroup y stores and quantizes only the
     // float4 t + 256*y of each lane (the tail of the kernel is the longest part of it and splits freely)
-    const int vs = gridDim.y > 1 ? (int)blockIdx.y : -1;
+    const int vs = s.slices > 1 ? (int)blockIdx.y : -1;
     const int E = s.E, nq = E >> 2;                          // float4 quads in a row; thread t owns quads t + 256*v
     float4 xv[LG_ROWV], dv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
     // issue every load up front: one memory round trip for the whole row
-    if (s.emb) {
+    if (!s.x) {                                              // (rows that are token lookups have no residual yet)
         const int tok = s.toks[ctl->step * M + j];
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
@@ -227,8 +228,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_quant_flat(const float *x, int row
 // per thread instead of one per element.  Indices past the end are clamped to the last element,
 // which is then copied more than once with the same value: no branches.
 template <typename T>
-__device__ __forceinline__ void lg_copy_batched(const T *src, T *dst, int n) {
-    const int nt = blockDim.x;
+__device__ __forceinline__ void lg_copy_batched(const T *src, T *dst, int n, int nt_known = 0) {
+    const int nt = nt_known ? nt_known : (int)blockDim.x;
     for (int i0 = threadIdx.x; i0 < n; i0 += 8 * nt) {
         const int last = n - 1;
         const int a0 = min(i0, last), a1 = min(i0 + nt, last), a2 = min(i0 + 2 * nt, last), a3 = min(i0 + 3 * nt, last);
@@ -249,9 +250,9 @@ __device__ __forceinline__ void lg_load_q8(const int8_t *q, int k, int8_t *lq) {
 // tiles, the rows' stores wait for every tile.
 struct CopyBatch { uint4 t0, t1, t2, t3, t4, t5, t6, t7; };
 template <int M>
-__device__ __forceinline__ CopyBatch lg_load_q8_issue(const int8_t *q, int k) {
+__device__ __forceinline__ CopyBatch lg_load_q8_issue(const int8_t *q, int k, int nt) {
     const uint4 *src = (const uint4 *)q;
-    const int nt = blockDim.x, last = M * k * 5 / 64 - 1, i0 = threadIdx.x;
+    const int last = M * k * 5 / 64 - 1, i0 = threadIdx.x;
     CopyBatch b;
     b.t0 = src[min(i0, last)]; b.t1 = src[min(i0 + nt, last)];
     if (last >= 2 * nt) {                                     // (short rows, k = 256: two units per thread hold them all)
@@ -262,15 +263,15 @@ __device__ __forceinline__ CopyBatch lg_load_q8_issue(const int8_t *q, int k) {
     return b;
 }
 template <int M>
-__device__ __forceinline__ void lg_load_q8_commit(const CopyBatch &b, const int8_t *q, int k, int8_t *lq) {
+__device__ __forceinline__ void lg_load_q8_commit(const CopyBatch &b, const int8_t *q, int k, int8_t *lq, int nt) {
     uint4 *dst = (uint4 *)lq;
-    const int nt = blockDim.x, n = M * k * 5 / 64, last = n - 1, i0 = threadIdx.x;
+    const int n = M * k * 5 / 64, last = n - 1, i0 = threadIdx.x;
     dst[min(i0, last)] = b.t0; dst[min(i0 + nt, last)] = b.t1;
     if (last >= 2 * nt) {
         dst[min(i0 + 2 * nt, last)] = b.t2; dst[min(i0 + 3 * nt, last)] = b.t3;
         dst[min(i0 + 4 * nt, last)] = b.t4; dst[min(i0 + 5 * nt, last)] = b.t5; dst[min(i0 + 6 * nt, last)] = b.t6; dst[min(i0 + 7 * nt, last)] = b.t7;
     }
-    if (n > 8 * nt) lg_copy_batched<uint4>((const uint4 *)q + 8 * nt, dst + 8 * nt, n - 8 * nt);
+    if (n > 8 * nt) lg_copy_batched<uint4>((const uint4 *)q + 8 * nt, dst + 8 * nt, n - 8 * nt, nt);
 }
 
 // Input of a draft head (src/mtp.c:268-276): cat = [dequant(token_embd[token]) * sqrt(nb), h_prev],
@@ -386,8 +387,9 @@ struct MmArgs {
     float         *out;      // [M][m]
     const int8_t  *q_in;     // q8 activation buffer of the M input rows
     int32_t       *dots;     // DUMP only: [M][m][k/32]
+    int            nthreads; // threads per workgroup (blockDim.x): as an argument it arrives with the others
 };
-#define LG_MM_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, m, m, v) X(float *, out, out, v) X(int32_t *, dots, dots, v)
+#define LG_MM_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, m, m, v) X(int, nthreads, nthreads, v) X(float *, out, out, v) X(int32_t *, dots, dots, v)
 
 // Plain matmul: out[j][i] f32.  blockDim = 64*W wavefronts, each wavefront takes G neighbouring
 // row groups (G*64/S rows); grid covers ceil(groups / (W*G)) workgroups.
@@ -399,7 +401,7 @@ __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(LG_MM_FIELDS
     int8_t *lq = (int8_t *)smem;
     float2 *lds = (float2 *)(smem + (size_t)M * a.k);
     constexpr int RW = 64 / S;                                // rows per group
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = a.nthreads >> 6;
     const int nit = (a.k >> 5) / S, ngroups = a.m / RW;
     const int g0 = (blockIdx.x * nw + wave) * G;
     const uint8_t *wg[G];
@@ -410,11 +412,11 @@ __global__ __launch_bounds__(S == 32 ? 320 : LG_WG, 2) void lg_k_mm(LG_MM_FIELDS
         wg[g] = a.w + (size_t)gi * nit * LG_TILE;
         row[g] = gi * RW + lane / S;
     }
-    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, a.k); // the rows first, then the tiles
+    const CopyBatch rows = lg_load_q8_issue<M>(a.q_in, a.k, a.nthreads); // the rows first, then the tiles
     WChunk<G, U> first;
     lg_mm_fetch<G, U>(first, wg, 0, nit, lane);
     __builtin_amdgcn_sched_barrier(0);
-    lg_load_q8_commit<M>(rows, a.q_in, a.k, lq);
+    lg_load_q8_commit<M>(rows, a.q_in, a.k, lq, a.nthreads);
     __syncthreads();
     if (g0 >= ngroups) return;
     float acc[G][M];
@@ -1131,13 +1133,14 @@ struct AttnArgs {
     const float *q_norm, *k_norm, *rope_tab, *rope_ff;
     uint16_t *kcw, *vcw;     // this layer's own cache, to receive the block's rows (nullptr: it reads another layer's)
     float eps;
+    int gx, gz;              // lg_k_attn: its launch dimensions x and z (as arguments they arrive with the others)
     __device__ __forceinline__ uint4 kc4(size_t off) const { return *(const uint4 *)(kc + off); }
     __device__ __forceinline__ uint4 vc4(size_t off) const { return *(const uint4 *)(vc + off); }
     // for the kernels that stage a tile once for all the rows of a block: no second reader, so non-temporal
     __device__ __forceinline__ uint4 kc4s(size_t off) const { return lg_ldw16(kc + off); }
     __device__ __forceinline__ uint4 vc4s(size_t off) const { return lg_ldw16(vc + off); }
 };
-#define LG_ATTN_FIELDS(X, v) X(int, H, H, v) X(int, nkv, nkv, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int, seq, seq, v) X(int, kv_dim, kv_dim, v) X(const uint16_t *, kc, kc, v) X(const uint16_t *, vc, vc, v) X(const float *, qkv, qkv, v) X(const float *, q_norm, q_norm, v) X(const float *, k_norm, k_norm, v) X(const float *, rope_tab, rope_tab, v) X(const float *, rope_ff, rope_ff, v) X(int, ld, ld, v) X(int, k_off, k_off, v) X(int, v_off, v_off, v) X(uint16_t *, kcw, kcw, v) X(uint16_t *, vcw, vcw, v) X(const float *, q, q, v) X(float *, pm, pm, v) X(float *, pl, pl, v) X(float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(float, eps, eps, v)
+#define LG_ATTN_FIELDS(X, v) X(int, gx, gx, v) X(int, gz, gz, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int, seq, seq, v) X(int, kv_dim, kv_dim, v) X(const uint16_t *, kc, kc, v) X(const uint16_t *, vc, vc, v) X(int, H, H, v) X(int, nkv, nkv, v) X(const float *, qkv, qkv, v) X(const float *, q_norm, q_norm, v) X(const float *, k_norm, k_norm, v) X(const float *, rope_tab, rope_tab, v) X(const float *, rope_ff, rope_ff, v) X(int, ld, ld, v) X(int, k_off, k_off, v) X(int, v_off, v_off, v) X(uint16_t *, kcw, kcw, v) X(uint16_t *, vcw, vcw, v) X(const float *, q, q, v) X(float *, pm, pm, v) X(float *, pl, pl, v) X(float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(float, eps, eps, v)
 
 __device__ __forceinline__ int lg_win_start(int pos, int window) {
     return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -1170,7 +1173,7 @@ __global__ __launch_bounds__(LG_WG, NV > 1 ? 2 : 4) void lg_k_attn(const StepCtl
     float *es = (float *)(vt + 32 * kst);                     // [G][32]
     float *hv = (float *)(smem + (((size_t)((unsigned char *)(es + G * 32 + G) - smem) + 15) & ~(size_t)15));   // FQ: [4 wavefronts][hd] staging
     // dispatched last rows and last tiles first: those hold the block's own K/V rows, the longest workgroups
-    const int kvh = blockIdx.y, j = (int)gridDim.z - 1 - (int)blockIdx.z, bx = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int kvh = blockIdx.y, j = a.gz - 1 - (int)blockIdx.z, bx = a.gx - 1 - (int)blockIdx.x;
     const int pos0 = ctl->pos + a.pos_off, pj = pos0 + j;
     const int startj = lg_win_start(pj, a.window);
     const int n = (lg_win_start(pos0, a.window) >> 5) + bx;
