@@ -573,12 +573,13 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(LG_GEGLU_FIELDS(LG_XP, _)
     const int t = blockIdx.x, nb = a.k >> 5, nit = nb >> 3;
     const uint8_t *wt = a.w + ((size_t)t * nb + (size_t)s * nit) * LG_TILE;
     uint4 wq[CH], nwq[CH]; uint32_t wd[CH], nwd[CH];
+    const __amdgpu_buffer_rsrc_t rw = lg_buffer_rsrc(wt);
     auto fetch = [&](int it0) {
         #pragma unroll
         for (int u = 0; u < CH; ++u) {
             const int it = it0 + u < nit ? it0 + u : nit - 1;
-            nwq[u] = lg_ldt16(wt, it, lane);
-            nwd[u] = lg_ldt2(wt, it, lane);
+            nwq[u] = lg_ldt16b(rw, it, lane);
+            nwd[u] = lg_ldt2b(rw, it, lane);
         }
     };
     unsigned char *la = smem + (size_t)s * nit * (LG_MU_DWORDS * 4);
