@@ -176,6 +176,20 @@ int  lg_hip_matmul_q4q8(const void *w, int k, int m, const float *x, int rows, f
 int  lg_hip_rows_norm_q8(const float *x, const float *dout, const float *w_post, const float *out_scale,
                          const float *w_pre, int rows, int E, float eps, float *x_out, float *h_out,
                          int8_t *xq, float *xd, int32_t *xsum);
+/* The kernel a verify block runs between ffn_down and the per-layer projection, on its own: the FFN residual update
+ * x_out = x + rmsnorm(dout) * w_post, the inp_gate matmul on the q8 of x_out, gelu(.) * ipl and the q8 of that
+ * (rmsnorm_add_kernel, matmul_q(inp_gate) and geglu_kernel of the per-layer-input block,
+ * src/cuda/model-cuda.cuh:1251-1258; src/cpu/model-cpu.c:413-420).  w_gate = ple plain q4_0 rows of E weights, ipl =
+ * [rows][ple].  rows 1..8, E a multiple of 256 up to 4096, ple = 256 (the width model_commit accepts).  Outputs (each may be
+ * NULL): x_out [rows][E] f32, pq [rows][ple] int8, pd / psum [rows][ple/32]. */
+int  lg_hip_rows_ple_gate(const float *x, const float *dout, const float *w_post, const void *w_gate, const float *ipl,
+                          int rows, int E, int ple, float eps, float *x_out, int8_t *pq, float *pd, int32_t *psum);
+/* The per-layer inputs of a block, on their own (build_per_layer_n, src/cuda/model-cuda.cuh:1121-1147):
+ * out = (rmsnorm(pmp / sqrt(E)) * proj_norm + tok_row * sqrt(ple)) / sqrt(2) per (row, layer), pmp = the raw
+ * per_layer_model_proj output [rows][n_layer*ple], pte = n_tok plain q4_0 rows of n_layer*ple (per_layer_token_embd),
+ * toks = the rows' token ids (< n_tok).  out [rows][n_layer*ple]. */
+int  lg_hip_ple_inputs(const float *pmp, const float *proj_norm, const void *pte, int n_tok, const int32_t *toks,
+                       int rows, int n_layer, int ple, int E, float eps, float *out);
 /* Matmul against a matrix kept in f32 (the per-layer-embedding matrices of QAT conversions; the reference's int8
  * backend multiplies such weights by the f32 activations unquantized, src/cuda/model-cuda-i8.cu:645-653, :846-895):
  * w = m rows of k floats, x = rows x k floats, out = rows x m floats.  Any number of rows (8 per workgroup row). */

@@ -1573,6 +1573,69 @@ extern "C" int lg_hip_rows_norm_q8(const float *x, const float *dout, const floa
     return read_back_q8(dq, rows, E, xq, xd, xsum);
 }
 
+// ---- isolated per-layer-embedding kernels (tests) ----------------------------------------------------
+// lg_k_rows_plegate on its own: the residual update x + rmsnorm(dout) * w_post of `rows` rows, then the inp_gate
+// matmul (w_gate: ple plain q4_0 rows of E) on the q8 of the new rows, gelu(.) * ipl and the q8 of that.
+extern "C" int lg_hip_rows_ple_gate(const float *x, const float *dout, const float *w_post, const void *w_gate, const float *ipl,
+                                    int rows, int E, int ple, float eps, float *x_out, int8_t *pq, float *pd, int32_t *psum) {
+    if (!x || !dout || !w_post || !w_gate || !ipl) return fail(-1, "rows_ple_gate: null input");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || E < 256 || E % 256 || E > 4096 || ple != 256)
+        return fail(-2, "rows_ple_gate: rows %d (1..%d), E %d (a multiple of 256 up to 4096), ple %d (256 is built)", rows, LG_HIP_MAX_ROWS, E, ple);
+    if (lg_hip_device_count() < 1) return fail(-3, "rows_ple_gate: no HIP device");
+    std::vector<uint8_t> tiled(lg_hip_repacked_bytes(E, ple));
+    int rc = lg_hip_repack_q4_0(w_gate, E, ple, tiled.data());
+    if (rc) return rc;
+    Scratch sc;
+    float *dx, *dd, *dw, *di, *dxo; uint8_t *dg; int8_t *dq;
+    const size_t n = (size_t)rows * E;
+    if (sc.get(&dx, n) || sc.get(&dd, n) || sc.get(&dw, (size_t)E) || sc.get(&di, (size_t)rows * ple) || sc.get(&dxo, n) ||
+        sc.get(&dg, tiled.size()) || sc.get(&dq, (size_t)rows * ple * 5 / 4)) return -7;
+    HIP_TRY(hipMemcpy(dx, x, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dd, dout, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dw, w_post, (size_t)E * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(di, ipl, (size_t)rows * ple * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dg, tiled.data(), tiled.size(), hipMemcpyHostToDevice));
+    PleGateArgs a{ dg, E, ple, nullptr, di, 0, 1, dq };
+    RowsPleGateArgs r{ a, dx, dd, dw, dxo, eps };
+    switch (rows) {
+#define CASE(M) case M: rc = set_lds(lg_k_rows_plegate<M>, lds_mm(1, E)); \
+        if (!rc) hipLaunchKernelGGL((lg_k_rows_plegate<M>), dim3(ple / 32, M), dim3(LG_WG), lds_mm(1, E), nullptr, LG_RPG_FIELDS(LG_XA, r) 0); break;
+        CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+    }
+    if (rc) return rc;
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    if (x_out) HIP_TRY(hipMemcpy(x_out, dxo, n * 4, hipMemcpyDeviceToHost));
+    return read_back_q8(dq, rows, ple, pq, pd, psum);
+}
+
+// lg_k_ipl on its own: the per-layer inputs of `rows` tokens from the raw per_layer_model_proj output
+// (pmp [rows][n_layer*ple]) and the tokens' rows of per_layer_token_embd (pte: n_tok plain q4_0 rows of n_layer*ple).
+extern "C" int lg_hip_ple_inputs(const float *pmp, const float *proj_norm, const void *pte, int n_tok, const int32_t *toks,
+                                 int rows, int n_layer, int ple, int E, float eps, float *out) {
+    if (!pmp || !proj_norm || !pte || !toks || !out) return fail(-1, "ple_inputs: null argument");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || n_layer < 1 || ple < 32 || ple % 32 || ple > 256 || n_tok < 1 || E < 1)
+        return fail(-2, "ple_inputs: rows %d (1..%d), n_layer %d, ple %d (a multiple of 32 up to 256), %d token rows", rows, LG_HIP_MAX_ROWS, n_layer, ple, n_tok);
+    for (int j = 0; j < rows; ++j) if (toks[j] < 0 || toks[j] >= n_tok) return fail(-2, "ple_inputs: token %d of row %d (table of %d rows)", toks[j], j, n_tok);
+    if (lg_hip_device_count() < 1) return fail(-3, "ple_inputs: no HIP device");
+    Scratch sc;
+    const size_t w = (size_t)n_layer * ple, tb = (size_t)n_tok * (w / 32 * 18);
+    float *dp, *dn; uint8_t *dt; int32_t *dk; StepCtl *ctl;
+    if (sc.get(&dp, rows * w) || sc.get(&dn, (size_t)ple) || sc.get(&dt, tb) || sc.get(&dk, (size_t)rows) || sc.get(&ctl, 1)) return -7;
+    HIP_TRY(hipMemcpy(dp, pmp, rows * w * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dn, proj_norm, (size_t)ple * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dt, pte, tb, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dk, toks, (size_t)rows * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    IplArgs i{ dp, ple, n_layer, rows, dn, dt, dk, 1.0f / sqrtf((float)E), sqrtf((float)ple), 1.0f / sqrtf(2.0f), eps };
+    hipLaunchKernelGGL(lg_k_ipl, dim3(n_layer, rows), dim3(64), 0, nullptr, i, ctl);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(out, dp, rows * w * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
 // the two launches of an isolated attention: tile partials, then the ordered merge
 // (the same choice of kernels as a verify step makes: many (tile, kv head) pairs -> one workgroup per pair serves all
 // rows; many tiles per row -> the merge is cut by dims)

@@ -61,6 +61,9 @@ def load_hip():
     L.lg_hip_attention.argtypes = [f32p, u16p, u16p] + [C.c_int] * 7 + [f32p, C.c_int, C.c_void_p]
     L.lg_hip_matmul_f32w.argtypes = [f32p, C.c_int, C.c_int, f32p, C.c_int, f32p]
     L.lg_hip_rows_norm_q8.argtypes = [f32p] + [C.c_void_p] * 4 + [C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 5
+    L.lg_hip_rows_ple_gate.argtypes = [f32p, f32p, f32p, u8p, f32p, C.c_int, C.c_int, C.c_int, C.c_float] + [C.c_void_p] * 4
+    i32p_ = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+    L.lg_hip_ple_inputs.argtypes = [f32p, f32p, u8p, C.c_int, i32p_, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, f32p]
     L.lg_hip_kv_layout.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
     L.lg_hip_kv_write.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
     L.lg_hip_kv_read.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, u16p]
@@ -354,6 +357,34 @@ def rows_norm_q8(x, dout=None, w_post=None, out_scale=None, w_pre=None, eps=1e-6
     hip_check(H.lg_hip_rows_norm_q8(x, *[_opt(a) for a in keep], rows, E, eps, _opt(x_out), _opt(h), _opt(xq), _opt(xd), _opt(xsum)),
               "rows_norm_q8")
     return dict(x_out=x_out, h=h, xq=xq, xd=xd, xsum=xsum)
+
+
+def rows_ple_gate(x, dout, w_post, w_gate_q4_0, ipl, eps=1e-6):
+    """Isolated rows + per-layer gate kernel through the C ABI.  x, dout: [rows, E]; w_gate_q4_0: ple q4_0 rows of E;
+    ipl: [rows, ple].  Returns dict(x_out, pq, pd, psum)."""
+    H = load_hip()
+    x = np.ascontiguousarray(x, np.float32)
+    rows, E = x.shape
+    ipl = np.ascontiguousarray(ipl, np.float32)
+    ple = ipl.shape[1]
+    x_out = np.zeros_like(x)
+    pq = np.zeros((rows, ple), np.int8); pd = np.zeros((rows, ple // 32), np.float32); psum = np.zeros((rows, ple // 32), np.int32)
+    hip_check(H.lg_hip_rows_ple_gate(x, np.ascontiguousarray(dout, np.float32), np.ascontiguousarray(w_post, np.float32),
+                                     np.ascontiguousarray(w_gate_q4_0, np.uint8), ipl, rows, E, ple, eps,
+                                     _opt(x_out), _opt(pq), _opt(pd), _opt(psum)), "rows_ple_gate")
+    return dict(x_out=x_out, pq=pq, pd=pd, psum=psum)
+
+
+def ple_inputs(pmp, proj_norm, pte_q4_0, n_tok, toks, n_layer, ple, E, eps=1e-6):
+    """Isolated per-layer-input kernel through the C ABI.  pmp: [rows, n_layer*ple] raw projection; pte_q4_0: n_tok
+    q4_0 rows of n_layer*ple; toks: [rows].  Returns [rows, n_layer*ple]."""
+    H = load_hip()
+    pmp = np.ascontiguousarray(pmp, np.float32)
+    out = np.zeros_like(pmp)
+    hip_check(H.lg_hip_ple_inputs(pmp, np.ascontiguousarray(proj_norm, np.float32), np.ascontiguousarray(pte_q4_0, np.uint8),
+                                  n_tok, np.ascontiguousarray(toks, np.int32), pmp.shape[0], n_layer, ple, E, eps, out),
+              "ple_inputs")
+    return out
 
 
 def matmul_f32w(w, x):

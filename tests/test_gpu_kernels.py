@@ -115,6 +115,65 @@ def test_rows_kernel_matches_oracle(lg, ob, gpu_required, rows, E, with_dout, wi
         assert np.array_equal(r["xd"][j].view(np.uint32), d.view(np.uint32)), f"row {j}: scales"
 
 
+@pytest.mark.parametrize("rows,E,ple", [(1, 2560, 256), (5, 2560, 256), (8, 1536, 256), (4, 256, 256), (3, 3840, 256)])
+def test_rows_ple_gate_kernel_matches_oracle(lg, ob, gpu_required, rows, E, ple):
+    """The kernel between ffn_down and the per-layer projection in isolation: FFN residual update, inp_gate matmul on
+    the q8 of the new row, gelu(.) * per-layer input, q8 -- every output the oracle's, bit for bit."""
+    rng = np.random.default_rng(rows * 7 + E + ple)
+    L = ob.lib()
+    x = rng.normal(0, 1, (rows, E)).astype(np.float32)
+    dout = rng.normal(0, 3, (rows, E)).astype(np.float32)
+    w_post = (1 + 0.1 * rng.normal(0, 1, E)).astype(np.float32)
+    wg = random_q4_0(rng, ple, E)
+    ipl = rng.normal(0, 1, (rows, ple)).astype(np.float32)
+    ipl[0, :32] = 0.0                                    # a zero group in the result: scale 0, no NaN
+    print(f"rows + ple gate rows={rows} E={E} ple={ple}", flush=True)
+    r = lg.hiplib.rows_ple_gate(x, dout, w_post, wg, ipl, eps=1e-6)
+    xn = np.zeros_like(x)
+    for j in range(rows):
+        o = np.zeros(E, np.float32)
+        L.lgo_rmsnorm(o, np.ascontiguousarray(dout[j]), w_post.ctypes.data, E, 1e-6, 1)
+        xn[j] = x[j] + o
+    assert np.array_equal(r["x_out"].view(np.uint32), xn.view(np.uint32)), "residual"
+    _, _, _, gate, _ = oracle_matmul(ob, wg, E, ple, xn)
+    for j in range(rows):
+        g = np.array([L.lgo_gelu(float(v), 1) for v in gate[j]], np.float32) * ipl[j]
+        q = np.zeros(ple, np.int8); d = np.zeros(ple // 32, np.float32); sm = np.zeros(ple // 32, np.int32)
+        L.lgo_quant_q8(np.ascontiguousarray(g), ple, q, d, sm)
+        assert np.array_equal(r["pq"][j], q) and np.array_equal(r["psum"][j], sm), f"row {j}: q8 of the gated row"
+        assert np.array_equal(r["pd"][j].view(np.uint32), d.view(np.uint32)), f"row {j}: scales"
+
+
+@pytest.mark.parametrize("rows,n_layer,ple,E", [(1, 42, 256, 2560), (5, 42, 256, 2560), (8, 3, 32, 256), (4, 5, 128, 1536)])
+def test_ple_inputs_kernel_matches_oracle(lg, ob, gpu_required, rows, n_layer, ple, E):
+    """The per-layer inputs of a block in isolation: (rmsnorm(proj / sqrt(E)) * w + token row * sqrt(ple)) / sqrt(2),
+    the token rows read from plain q4_0 -- the oracle's values, bit for bit (the oracle's order of operations:
+    oracle/lg_oracle.c, the per-layer-input part of forward_i8)."""
+    rng = np.random.default_rng(rows + n_layer + ple)
+    L = ob.lib()
+    n_tok, w = 37, n_layer * ple
+    pmp = rng.normal(0, 20, (rows, w)).astype(np.float32)
+    pmp[0, :ple] = 0.0                                   # a zero row under the norm: eps only
+    norm = (1 + 0.1 * rng.normal(0, 1, ple)).astype(np.float32)
+    pte = random_q4_0(rng, n_tok, w)
+    toks = rng.integers(0, n_tok, rows).astype(np.int32)
+    toks[0] = n_tok - 1
+    print(f"ple inputs rows={rows} layers={n_layer} ple={ple}", flush=True)
+    got = lg.hiplib.ple_inputs(pmp, norm, pte, n_tok, toks, n_layer, ple, E, eps=1e-6)
+    dw, codes = q4_0_codes(pte, n_tok, w)                # scales [n_tok, w/32], codes [n_tok, w/32, 32]
+    table = ((codes.astype(np.int32) - 8).astype(np.float32) * dw.astype(np.float32)[:, :, None]).reshape(n_tok, w)
+    ts, ps, r2 = np.float32(np.sqrt(np.float32(ple))), np.float32(1) / np.float32(np.sqrt(np.float32(E))), np.float32(1) / np.float32(np.sqrt(np.float32(2)))
+    for j in range(rows):
+        tok = table[toks[j]] * ts
+        p = pmp[j] * ps
+        for Lr in range(n_layer):
+            seg = np.ascontiguousarray(p[Lr * ple:(Lr + 1) * ple])
+            o = np.zeros(ple, np.float32)
+            L.lgo_rmsnorm(o, seg, norm.ctypes.data, ple, 1e-6, 1)
+            want = (o + tok[Lr * ple:(Lr + 1) * ple]) * r2
+            assert np.array_equal(got[j, Lr * ple:(Lr + 1) * ple].view(np.uint32), want.view(np.uint32)), f"row {j} layer {Lr}"
+
+
 def test_matmul_is_linear_in_the_scales(lg, gpu_required):
     """Size-independent property: doubling every weight scale doubles every output exactly
     (powers of two commute with rounding), negating codes around 8 negates it."""
