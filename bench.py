@@ -258,7 +258,7 @@ def main():
     timed_tokens = int(adv[a.warmup:].sum())
     value = timed_tokens / (ms * 1e-3)
 
-    # per-kernel-class device time of one step (un-captured, event pair per launch)
+    # per-kernel-class device time of one step (un-captured, start/stop events filled in by each launch)
     prof = gpu.profile_step(blocks[0], ctx, repeats=3)
     step_bytes = sum(c["bytes"] for c in prof)
     # the roofline kernel: the class that moves the most bytes per step (gate/up + GeGLU: 47% of them at the E4B
@@ -269,9 +269,9 @@ def main():
                 "frac": dom_gbs / HBM_PEAK_GBS,
                 "traffic": MEASURED_TRAFFIC.get((a.workload, dom["name"], a.rows)),
                 "traffic_source": TRAFFIC_SOURCE if (a.workload, dom["name"], a.rows) in MEASURED_TRAFFIC else None,
-                "timing": "one HIP event pair per launch on the library's stream, un-captured; an event pair adds the command "
-                          "processor's packet handling (about 1.5 us per launch) to the kernel's begin-to-end time that the "
-                          "rocprofv3 trace under profiles/ reports, so frac reads lower here than from the trace",
+                "timing": "HIP start/stop events filled in by each launch itself (hipExtLaunchKernelGGL on the library's "
+                          "stream, un-captured): the kernel's own begin-to-end time, what the rocprofv3 kernel trace under "
+                          "profiles/ reports for the same kernel",
                 "bytes_per_launch": dom["bytes"] / max(dom["launches"], 1), "ms_per_launch": dom["ms"] / max(dom["launches"], 1),
                 "launches_per_step": dom["launches"]}
     step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9

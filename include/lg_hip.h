@@ -144,7 +144,8 @@ int  lg_hip_schedule_wait(lg_hip_model *m, int32_t *out, int32_t *adv, int32_t *
 /* Times n_steps already-loaded steps with device events on the library's stream; *ms = total. */
 int  lg_hip_schedule_time(lg_hip_model *m, lg_hip_kv *kv, int n_steps, float *ms);
 
-/* ---- measurement: run one step un-captured with an event pair around every kernel and sum
+/* ---- measurement: run one step un-captured, every kernel launched with a start and a stop event of its own
+ * (hipExtLaunchKernelGGL: the kernel's begin-to-end time, without the packet handling around it), and sum
  * the durations per kernel class.  names/ms/launches/bytes are caller arrays of `cap` entries;
  * returns the number of classes filled.  bytes[i] = weight + KV bytes the class must read per
  * step (algorithmic, not measured). */

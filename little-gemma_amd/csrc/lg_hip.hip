@@ -3,6 +3,7 @@
 // Host side: weight layout, scratch, the launch sequence of one step, graph capture, the
 // device-resident step schedule and the measurement helpers.  Device side: lg_kernels.h.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
@@ -660,21 +661,28 @@ struct Launcher {
     lg_hip_model *m;
     bool dry;              // only raise LDS limits, launch nothing (done once before a capture)
     int rc = 0;
-    void begin(int cls) {
-        if (!m->prof.on || rc) return;
-        hipEvent_t a, b;
-        if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { rc = fail(-9, "event create failed"); return; }
-        m->prof.ev.push_back(a); m->prof.ev.push_back(b); m->prof.cls.push_back(cls);
-        (void)hipEventRecord(a, m->stream);
+    // per-class timing: an event pair that the launch itself fills in (begin and end of the kernel's own execution,
+    // what a kernel trace reports; a pair recorded around the launch also counts the packet handling, ~1.5 us)
+    bool events(int cls, hipEvent_t *a, hipEvent_t *b) {
+        if (rc) return false;
+        if (hipEventCreate(a) != hipSuccess || hipEventCreate(b) != hipSuccess) { rc = fail(-9, "event create failed"); return false; }
+        m->prof.ev.push_back(*a); m->prof.ev.push_back(*b); m->prof.cls.push_back(cls);
+        return true;
     }
     void end() {
-        if (m->prof.on && !rc) (void)hipEventRecord(m->prof.ev.back(), m->stream);
         if (!rc) { hipError_t e = hipGetLastError(); if (e != hipSuccess) rc = fail(-100 - (int)e, "kernel launch failed: %s", hipGetErrorString(e)); }
     }
 };
+// (the kernel's parameter types come from the kernel, the arguments are converted to them one by one)
+template <typename... P, typename... A>
+static void launch_timed(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t st, hipEvent_t e0, hipEvent_t e1, A &&...a) {
+    hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, st, e0, e1, 0, static_cast<P>(a)...);
+}
 
-#define LAUNCH(cls, kernel, grid, block, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { lx.begin(cls); \
-    hipLaunchKernelGGL(kernel, grid, block, lds, lx.m->stream, __VA_ARGS__); lx.end(); } } while (0)
+#define LAUNCH(cls, kernel, grid, block, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { \
+    if (lx.m->prof.on) { hipEvent_t e0_, e1_; if (lx.events(cls, &e0_, &e1_)) launch_timed(kernel, grid, block, lds, lx.m->stream, e0_, e1_, __VA_ARGS__); } \
+    else hipLaunchKernelGGL(kernel, grid, block, lds, lx.m->stream, __VA_ARGS__); \
+    lx.end(); } } while (0)
 
 // Compute units of the current device (asked once).
 static int cu_count() {
