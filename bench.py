@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 lg = importlib.import_module("little-gemma_amd")
 
 HBM_PEAK_GBS = 8000.0
+i32a = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
 # HBM bytes per launch of the dominant kernel (gate/up + GeGLU at the E4B shape), from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in the file named below (scaled by the copy-kernel calibration given
 # there): reads 29.40 MB for M = 5 (29.27 MB for M = 1), writes 0.15 MB (0.03 MB).  Counters cannot be read
@@ -168,6 +169,41 @@ def ref_f32_gap(model_dir):
     return out
 
 
+def xcd_handover():
+    """Placement of workgroups over the XCDs and the cost of a flag hand-over inside one XCD / across XCDs."""
+    import ctypes as C
+    H = lg.hiplib.load_hip()
+    H.lg_hip_xcd_map.argtypes = [C.c_int] * 4 + [i32a, i32a]
+    H.lg_hip_xcd_handover.argtypes = [C.c_int] * 7 + [i32a, C.POINTER(C.c_float)]
+    placement = []
+    for grid, block, lds in ((256, 256, 0), (256, 512, 96 * 1024), (320, 512, 0), (512, 256, 0), (2048, 64, 0)):
+        xcc = np.zeros((4, grid), np.int32); hw = np.zeros((4, grid), np.int32)
+        lg.hiplib.hip_check(H.lg_hip_xcd_map(grid, block, lds, 4, xcc, hw), "xcd_map")
+        turn = bool(np.all(xcc == (np.arange(grid) % 8)[None, :]))
+        cu = ((hw >> 8) & 15) | (((hw >> 12) & 1) << 4) | (((hw >> 13) & 7) << 5)          # cu, sh, se fields of HW_ID
+        per_cu = [int(np.unique(np.stack([xcc[l], cu[l]]), axis=1, return_counts=True)[1].max()) for l in range(4)]
+        placement.append({"grid": grid, "block": block, "lds": lds, "workgroup_i_on_xcd_i_mod_8": turn,
+                          "xcd_of_first_16": xcc[0, :16].tolist(), "same_in_4_launches": bool(np.all(xcc == xcc[0])),
+                          "per_xcd": np.bincount(xcc[0], minlength=8).tolist(), "max_workgroups_on_one_cu": per_cu})
+    names = {0: "plain", 1: "sc0", 2: "sc1", 3: "sc0 sc1"}
+    rows = []
+    rounds = 200
+    for what, set_mode, sel, n in (("one XCD (workgroups 0,8,..,248)", 0, 0, 32), ("one XCD (workgroups 3,11,..)", 0, 3, 32),
+                                   ("spread (workgroups 0..31)", 1, 0, 32), ("spread (workgroups 0..7)", 1, 0, 8),
+                                   ("one XCD, 8 members", 0, 0, 8)):
+        for st, ld in ((0, 2), (0, 1), (2, 2), (3, 3), (0, 3), (0, 0)):
+            for nbytes in (0, 1024, 16384):
+                res = np.zeros((n, 4), np.int32); tick = C.c_float(0)
+                lg.hiplib.hip_check(H.lg_hip_xcd_handover(set_mode, sel, n, st, ld, nbytes, rounds, res, C.byref(tick)), "xcd_handover")
+                rows.append({"group": what, "members": n, "store": names[st], "load": names[ld], "bytes_per_member": nbytes,
+                             "us_per_round_max": round(float(res[:, 0].max()) * tick.value / rounds / 1e3, 4),
+                             "us_per_round_min": round(float(res[:, 0].min()) * tick.value / rounds / 1e3, 4),
+                             "stale_words": int(res[:, 1].sum()), "polls_given_up": int(res[:, 2].sum()),
+                             "xcds_seen": sorted(set(res[:, 3].tolist()))})
+    print(json.dumps({"metric": "workgroup placement over XCDs and flag hand-over cost", "rounds": rounds,
+                      "placement": placement, "handover": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -183,7 +219,13 @@ def main():
     ap.add_argument("--mtp-steps", type=int, default=24, help="steps of the draft-head loop measurement (4 chained device drafts + verify); 0 skips it")
     ap.add_argument("--launch-floor", action="store_true",
                     help="measure only what a captured chain of dependent kernels costs (empty, and with a 64-byte hand-over) and exit")
+    ap.add_argument("--xcd-handover", action="store_true",
+                    help="measure only where workgroups run (XCD of every workgroup) and what a flag hand-over among the "
+                         "workgroups of one XCD costs next to one spread over all XCDs, and exit")
     a = ap.parse_args()
+    if a.xcd_handover:
+        xcd_handover()
+        return
     if a.launch_floor:
         import ctypes as C
         H = lg.hiplib.load_hip()

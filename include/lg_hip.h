@@ -160,6 +160,22 @@ int  lg_hip_profile_step(lg_hip_model *m, lg_hip_kv *kv, const int32_t *toks, in
  * the same thing is its graph-vs-launch comparison, src/cuda/mtp-kernel.cuh:63-80). */
 int  lg_hip_launch_floor(int n_kernels, int mode, int grid, int block, int replays, float *us_per_kernel);
 
+/* Where the workgroups of a launch run and what a hand-over between the workgroups of ONE XCD costs (the chip has 8
+ * XCDs with an L2 each; no reference counterpart: the reference's decode graph overlaps independent matmuls on a second
+ * stream instead, src/cuda/model-cuda.cuh:917-935).
+ * lg_hip_xcd_map: XCC_ID and HW_ID registers of every workgroup of `launches` consecutive launches of grid x block
+ * threads with lds_bytes of dynamic LDS; xcc / hwid = [launches][grid].
+ * lg_hip_xcd_handover: n (2..32) workgroups of a 256-workgroup launch -- set_mode 0: the workgroups i with i % 8 == sel
+ * (one XCD when workgroups are dealt to the XCDs in turn); set_mode 1: workgroups sel*n .. sel*n+n-1 (spread over all
+ * XCDs) -- run `rounds` rounds of: store `bytes` each, wait for the stores, raise a flag, poll the n flags, read the
+ * neighbour's bytes back and check them.  store_scope / load_scope: 0 plain, 1 sc0, 2 sc1, 3 sc0 sc1.  res = [n][4]:
+ * { ticks of the device wall clock over the rounds, words that were not what the neighbour wrote, polls given up,
+ * XCD id }; *tick_ns = nanoseconds per tick.  Every wait is bounded: a combination that is not coherent reports
+ * mismatches or given-up polls, it does not hang. */
+int  lg_hip_xcd_map(int grid, int block, int lds_bytes, int launches, int32_t *xcc, int32_t *hwid);
+int  lg_hip_xcd_handover(int set_mode, int sel, int n, int store_scope, int load_scope, int bytes, int rounds,
+                         int32_t *res, float *tick_ns);
+
 /* ---- isolated kernels, host pointers in and out (parity tests of the parts) ----------------
  * q4_0 x q8_0 matmul (matmul_q_spec, src/cuda/model-cuda-i8.cu:1592-1602): w = m rows of k/32
  * 18-byte q4_0 blocks; x = rows x k floats, quantized on the device per 32 (d_quant_group,

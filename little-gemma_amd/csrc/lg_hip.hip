@@ -18,6 +18,7 @@
 #include "lg_kernels.h"
 #include "lg_mfma.h"
 #include "lg_fused.h"
+#include "lg_xcd.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
 #define LG_FUSE_ROWS_MAX 2         // widest block whose q/k/v matmul does the preceding row work itself
@@ -1855,4 +1856,63 @@ extern "C" int lg_hip_launch_floor(int n_kernels, int mode, int grid, int block,
     if (b) (void)hipFree(b);
     if (st) (void)hipStreamDestroy(st);
     return rc;
+}
+
+// ---- XCD placement and hand-over probes ------------------------------------------------------------
+// Which XCD every workgroup of a grid x block launch (with lds_bytes of dynamic LDS) ran on, `launches` times in a
+// row on one stream: xcc / hwid receive [launches][grid] values (XCC_ID and HW_ID registers).
+__global__ void lg_k_xcd_map_lds(int32_t *xcc, int32_t *hwid) {
+    extern __shared__ unsigned char smem[];
+    if (threadIdx.x == 0) { smem[0] = 1; xcc[blockIdx.x] = lg_xcc_id(); hwid[blockIdx.x] = (int32_t)lg_hw_id(); }
+}
+extern "C" int lg_hip_xcd_map(int grid, int block, int lds_bytes, int launches, int32_t *xcc, int32_t *hwid) {
+    if (grid < 1 || grid > 65536 || block < 1 || block > 1024 || lds_bytes < 0 || lds_bytes > 160 * 1024 || launches < 1 || !xcc || !hwid)
+        return fail(-2, "xcd_map: bad argument");
+    if (lg_hip_device_count() < 1) return fail(-3, "xcd_map: no HIP device");
+    Scratch sc;
+    int32_t *dx, *dh;
+    const size_t n = (size_t)grid * launches;
+    if (sc.get(&dx, n) || sc.get(&dh, n)) return -7;
+    if (lds_bytes > 48 * 1024) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(lg_k_xcd_map_lds), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+    for (int l = 0; l < launches; ++l)
+        hipLaunchKernelGGL(lg_k_xcd_map_lds, dim3(grid), dim3(block), (size_t)lds_bytes, nullptr, dx + (size_t)l * grid, dh + (size_t)l * grid);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(xcc, dx, n * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(hwid, dh, n * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// One hand-over experiment (lg_k_xcd_handover): n workgroups of a 256-workgroup launch, chosen by set_mode / sel,
+// exchange `bytes` each per round through flags; store_scope / load_scope 0..3 = plain, sc0, sc1, sc0 sc1.
+// res receives [n][4] = { ticks, mismatching words, polls given up, XCD id }; *tick_ns the length of a tick.
+extern "C" int lg_hip_xcd_handover(int set_mode, int sel, int n, int store_scope, int load_scope, int bytes, int rounds,
+                                   int32_t *res, float *tick_ns) {
+    if (set_mode < 0 || set_mode > 1 || n < 2 || n > 32 || sel < 0 || (set_mode == 0 ? sel >= LG_XCDS : (sel + 1) * n > 256) ||
+        store_scope < 0 || store_scope > 3 || load_scope < 0 || load_scope > 3 || bytes < 0 || bytes % 4 || bytes > (1 << 20) ||
+        rounds < 1 || rounds > 100000 || !res || !tick_ns)
+        return fail(-2, "xcd_handover: bad argument");
+    if (lg_hip_device_count() < 1) return fail(-3, "xcd_handover: no HIP device");
+    int dev = 0, khz = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    *tick_ns = khz > 0 ? 1e6f / (float)khz : 10.0f;
+    Scratch sc;
+    XcdProbeArgs a{};
+    a.n = n; a.words = bytes / 4; a.rounds = rounds; a.set_mode = set_mode; a.sel = sel; a.spin_limit = 4000;
+    if (sc.get(&a.flags, (size_t)64) || sc.get(&a.data, (size_t)2 * n * (a.words ? a.words : 1)) || sc.get(&a.res, (size_t)n * 4)) return -7;
+    HIP_TRY(hipMemset(a.flags, 0, 256));
+    HIP_TRY(hipMemset(a.res, 0xFF, (size_t)n * 16));
+    HIP_TRY(hipDeviceSynchronize());
+    const int combo = store_scope * 4 + load_scope;
+    switch (combo) {
+#define CASE(S, L) case S * 4 + L: hipLaunchKernelGGL((lg_k_xcd_handover<S, L>), dim3(256), dim3(256), 0, nullptr, a); break;
+        CASE(0, 0) CASE(0, 1) CASE(0, 2) CASE(0, 3) CASE(1, 0) CASE(1, 1) CASE(1, 2) CASE(1, 3)
+        CASE(2, 0) CASE(2, 1) CASE(2, 2) CASE(2, 3) CASE(3, 0) CASE(3, 1) CASE(3, 2) CASE(3, 3)
+#undef CASE
+    }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(res, a.res, (size_t)n * 16, hipMemcpyDeviceToHost));
+    return 0;
 }
