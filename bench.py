@@ -179,10 +179,10 @@ def xcd_handover():
     for grid, block, lds in ((256, 256, 0), (256, 512, 96 * 1024), (320, 512, 0), (512, 256, 0), (2048, 64, 0)):
         xcc = np.zeros((4, grid), np.int32); hw = np.zeros((4, grid), np.int32)
         lg.hiplib.hip_check(H.lg_hip_xcd_map(grid, block, lds, 4, xcc, hw), "xcd_map")
-        turn = bool(np.all(xcc == (np.arange(grid) % 8)[None, :]))
+        turn = bool(np.all((xcc - xcc[:, :1]) % 8 == (np.arange(grid) % 8)[None, :]))   # (the first XCD of a launch depends on what ran before)
         cu = ((hw >> 8) & 15) | (((hw >> 12) & 1) << 4) | (((hw >> 13) & 7) << 5)          # cu, sh, se fields of HW_ID
         per_cu = [int(np.unique(np.stack([xcc[l], cu[l]]), axis=1, return_counts=True)[1].max()) for l in range(4)]
-        placement.append({"grid": grid, "block": block, "lds": lds, "workgroup_i_on_xcd_i_mod_8": turn,
+        placement.append({"grid": grid, "block": block, "lds": lds, "consecutive_workgroups_on_consecutive_xcds": turn, "first_xcd_per_launch": xcc[:, 0].tolist(),
                           "xcd_of_first_16": xcc[0, :16].tolist(), "same_in_4_launches": bool(np.all(xcc == xcc[0])),
                           "per_xcd": np.bincount(xcc[0], minlength=8).tolist(), "max_workgroups_on_one_cu": per_cu})
     names = {0: "plain", 1: "sc0", 2: "sc1", 3: "sc0 sc1"}

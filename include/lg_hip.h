@@ -207,6 +207,21 @@ int  lg_hip_rows_ple_gate(const float *x, const float *dout, const float *w_post
  * toks = the rows' token ids (< n_tok).  out [rows][n_layer*ple]. */
 int  lg_hip_ple_inputs(const float *pmp, const float *proj_norm, const void *pte, int n_tok, const int32_t *toks,
                        int rows, int n_layer, int ple, int E, float eps, float *out);
+/* The feed-forward half of a layer for a verify block of 4..8 rows as ONE launch partitioned over the 8 XCDs of the
+ * chip (rmsnorm_add_n_kernel + rmsnorm_kernel with the q8 epilogue, matmul_q_spec(gate / up), geglu_n_kernel,
+ * matmul_q_spec(down): src/cuda/prefill-kernel.cuh:452-497), on its own: x_out = x + rmsnorm(dout) * w_post,
+ * h = rmsnorm(x_out) * w_pre, act = gelu(gate . q8(h)) * (up . q8(h)), out = down . q8(act).  gate / up = FF plain
+ * q4_0 rows of E weights, down = E rows of FF.  Shapes: E a multiple of 256 up to 4096 and FF a multiple of 256 that one
+ * of the built instantiations serves (E 512 / FF 2048, E 2560 / FF 10240, E 3840 / FF 15360); a device of 256 compute
+ * units in 8 XCDs.  Outputs (each may be NULL): x_out [rows][E], act [rows][FF], out [rows][E]; *kernel_ms = mean
+ * device time of `repeats` launches, each preceded by a fill of flush_mb MiB when flush_mb > 0 (so that the weights
+ * come from HBM as in a step, not from the memory-side cache); delay_w = units of 64 clocks the compute wavefronts wait
+ * before they request their weights; stamps (NULL or [256][2][16]) = device wall-clock ticks
+ * of every workgroup at its phase boundaries in the last launch, seen by its first wavefront and by the one that serves
+ * the hand-overs. */
+int  lg_hip_ffn_xcd(const float *x, const float *dout, const float *w_post, const float *w_pre, const void *gate,
+                    const void *up, const void *down, int rows, int E, int FF, float eps, float *x_out, float *act,
+                    float *out, int repeats, float *kernel_ms, int flush_mb, int delay_w, int64_t *stamps);
 /* Matmul against a matrix kept in f32 (the per-layer-embedding matrices of QAT conversions; the reference's int8
  * backend multiplies such weights by the f32 activations unquantized, src/cuda/model-cuda-i8.cu:645-653, :846-895):
  * w = m rows of k floats, x = rows x k floats, out = rows x m floats.  Any number of rows (8 per workgroup row). */

@@ -19,6 +19,7 @@
 #include "lg_mfma.h"
 #include "lg_fused.h"
 #include "lg_xcd.h"
+#include "lg_xffn.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
 #define LG_FUSE_ROWS_MAX 2         // widest block whose q/k/v matmul does the preceding row work itself
@@ -119,6 +120,7 @@ struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; }
 struct Layer {
     uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
     float *winp_f = nullptr, *wproj_f = nullptr;   // inp_gate / proj when the file keeps them in a float type (then winp / wproj are null)
+    uint8_t *xgu = nullptr, *xdn = nullptr;        // gate/up and ffn_down again as per-workgroup streams of the XCD-partitioned kernel (lg_xffn.h)
     float *attn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *post_attn = nullptr, *ffn_norm = nullptr,
           *post_ffw = nullptr, *post_norm = nullptr, *out_scale = nullptr;
     int is_local = 0, hd = 0, nkv = 0, nff = 0, qd = 0, kd = 0, qkv_m = 0, k_off = 0, v_off = 0, owns = 0, src = 0;
@@ -126,9 +128,9 @@ struct Layer {
 };
 
 enum KClass { KC_ROWS, KC_PMP, KC_QKV, KC_QKVPOST, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
-              KC_HEAD, KC_ACCEPT, KC_COUNT };
+              KC_HEAD, KC_ACCEPT, KC_FFN, KC_COUNT };
 static const char *k_class_names[KC_COUNT] = { "rows_norm_quant", "ple_model_proj", "qkv", "qkv_post", "attn_tiles", "attn_merge",
-    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept" };
+    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept", "ffn_xcd" };
 
 struct Profile {
     bool on = false;
@@ -167,6 +169,14 @@ struct lg_hip_model {
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
+    // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
+    int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
+    bool xffn_built = false;                 // streams and working memory exist
+    int xffn_cls = -1;                       // which instantiation serves the shape
+    int xffn_delay = 0;                      // option: units of 64 clocks its compute wavefronts wait before they request their weights
+    float *slabs = nullptr, *xact = nullptr; // [8][max_rows][E] partial sums of ffn_down; [8][max_rows][max FF/8] gelu(gate)*up per XCD
+    uint32_t *xq8 = nullptr;                 // [8][E/32][80] q8 rows per XCD
+    XcdSync *xsync = nullptr;
     std::map<std::string, hipGraphExec_t> graphs;
     Profile prof;
     // a draft head (src/mtp.c) is a model whose layers own no cache: they read `target`'s
@@ -309,6 +319,81 @@ static void push_rows(std::vector<const uint8_t *> &rows, const HostTensor *t, u
     for (uint64_t r = r0; r < r0 + n; ++r) rows.push_back((const uint8_t *)t->data + r * rb);
 }
 
+static int cu_count();
+
+// ---- weight streams of the XCD-partitioned feed-forward kernel (lg_xffn.h) --------------------------
+// Shapes it is instantiated for: { gate/up operands per workgroup, blocks per gate/up segment (capacity), ffn_down
+// chains per wavefront, blocks per ffn_down segment (capacity), q8 blocks of an XCD's activations (capacity) }.
+struct XffnClass { int ops, nc, uw, ndc, cbc; };
+static const XffnClass k_xffn_classes[] = { { 1, 2, 1, 8, 8 },       // E <= 512, FF <= 2048 (the small test models)
+                                            { 3, 10, 2, 10, 40 },    // E4B shape: E 2560, FF 10240
+                                            { 4, 15, 2, 15, 60 } };  // 12B shape: E 3840, FF 15360
+static size_t xffn_lds(const XffnGeo &g, int M) { return g.lds(M); }
+static int xffn_class_of(const XffnGeo &g) {
+    if (!g.ok || (g.SX != 1 && g.SX != 4) || g.lds(LG_HIP_MAX_ROWS) + 256 > 160 * 1024) return -1;
+    for (int c = 0; c < (int)(sizeof k_xffn_classes / sizeof k_xffn_classes[0]); ++c) {
+        const XffnClass &k = k_xffn_classes[c];
+        if (g.ops == k.ops && g.nit <= k.nc && (g.units + 7) / 8 <= k.uw && g.nitd <= k.ndc && g.CB <= k.cbc) return c;
+    }
+    return -1;
+}
+template <typename F>
+static void for_workgroups(F work) {                  // the 256 workgroup streams, on a few host threads
+    unsigned hw = std::thread::hardware_concurrency();
+    const int nt = (int)(hw ? (hw > 16 ? 16 : hw) : 4);
+    std::vector<std::thread> pool;
+    for (int t = 0; t < nt; ++t) pool.emplace_back([=]() { for (int wg = 256 * t / nt; wg < 256 * (t + 1) / nt; ++wg) work(wg); });
+    for (auto &th : pool) th.join();
+}
+// gate/up: workgroup (XCD x = wg % 8, rank r = wg / 8) owns the FFN columns x*C + r*CW .. + CW-1; its weight rows are
+// those columns' gate rows followed by their up rows, cut into operands of 32; per K segment and operand: the nibble
+// bytes as [pair of blocks][half h][row n] 8 + 8 bytes, then the f16 scales as [pair][row n] 2 + 2 bytes (an odd count
+// of blocks is padded with a zero block)
+static void xffn_pack_gu(const uint8_t *gate, const uint8_t *up, const XffnGeo &g, uint8_t *dst) {
+    const size_t rowb = (size_t)g.nb * 18;
+    memset(dst, 0, 256 * g.gu_bytes);
+    for_workgroups([&](int wg) {
+        const int x = wg & 7, r = wg >> 3, c0 = x * g.C + r * g.CW;
+        for (int sg = 0; sg < 8; ++sg)
+            for (int o = 0; o < g.ops; ++o) {
+                const int vr = g.R2 - 32 * o < 32 ? g.R2 - 32 * o : 32;
+                uint8_t *ob = dst + (size_t)wg * g.gu_bytes + (size_t)sg * g.gu_seg + (size_t)32 * o * g.rb;
+                for (int n = 0; n < vr; ++n) {
+                    const int li = 32 * o + n;
+                    const uint8_t *row = li < g.CW ? gate + (size_t)(c0 + li) * rowb : up + (size_t)(c0 + li - g.CW) * rowb;
+                    for (int it = 0; it < g.nit; ++it) {
+                        const uint8_t *blk = row + (size_t)(sg * g.nit + it) * 18;
+                        for (int h = 0; h < 2; ++h) memcpy(ob + (size_t)(((it >> 1) * 2 + h) * vr + n) * 16 + (it & 1) * 8, blk + 2 + 8 * h, 8);
+                        memcpy(ob + (size_t)g.nitp * vr * 16 + (size_t)((it >> 1) * vr + n) * 4 + (it & 1) * 2, blk, 2);
+                    }
+                }
+            }
+    });
+}
+// ffn_down: workgroup (x, r) owns the output rows r*RW .. + RW-1 and the K segments x*SX .. + SX-1 of them; per
+// (operand of 32 rows, segment): nibble bytes [pair of blocks][half][row], then scales [pair][row]
+static void xffn_pack_dn(const uint8_t *down, const XffnGeo &g, uint8_t *dst) {
+    const size_t rowb = (size_t)(g.FF >> 5) * 18;
+    memset(dst, 0, 256 * g.dn_bytes);
+    for_workgroups([&](int wg) {
+        const int x = wg & 7, r = wg >> 3;
+        for (int gr = 0; gr < g.groups; ++gr) {
+            const int vr = g.RW - 32 * gr < 32 ? g.RW - 32 * gr : 32;
+            for (int sx = 0; sx < g.SX; ++sx) {
+                uint8_t *ub = dst + (size_t)wg * g.dn_bytes + (size_t)(gr * g.SX * 32 + sx * vr) * g.rbd;
+                for (int n = 0; n < vr; ++n) {
+                    const uint8_t *row = down + (size_t)(r * g.RW + 32 * gr + n) * rowb;
+                    for (int it = 0; it < g.nitd; ++it) {
+                        const uint8_t *blk = row + (size_t)((x * g.SX + sx) * g.nitd + it) * 18;
+                        for (int h = 0; h < 2; ++h) memcpy(ub + (size_t)(((it >> 1) * 2 + h) * vr + n) * 16 + (it & 1) * 8, blk + 2 + 8 * h, 8);
+                        memcpy(ub + (size_t)g.nitdp * vr * 16 + (size_t)((it >> 1) * vr + n) * 4 + (it & 1) * 2, blk, 2);
+                    }
+                }
+            }
+        }
+    });
+}
+
 static const float *rope_table(lg_hip_model *m, int is_local, int hd, int *rc) {
     auto key = std::make_pair(is_local, hd);
     auto it = m->rope_tabs.find(key);
@@ -377,6 +462,13 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
 
     m->L.resize(nl);
     int max_qkv = 0, max_ff = 0, max_qd = 0;
+    // the XCD-partitioned feed-forward kernel: one shape for all layers, a chip of 256 CUs in 8 XCDs, blocks of 4+ rows
+    XffnGeo xg = lg_xffn_geo(E, m->ffn_len[0]);
+    // (its weight streams are second copies of the FFN matrices: built only when the option is asked for at commit)
+    bool xffn = max_rows >= 4 && !m->target && cu_count() == LG_XCDS * LG_XCD_WGS && xffn_class_of(xg) >= 0 &&
+                getenv("LG_HIP_XCD_FFN") && atoi(getenv("LG_HIP_XCD_FFN")) != 0;
+    for (int L = 1; L < nl && xffn; ++L) xffn = m->ffn_len[L] == m->ffn_len[0];
+    std::vector<uint8_t> xstage;
     for (int L = 0; L < nl; ++L) {
         Layer &y = m->L[L];
         y.is_local = m->is_local[L]; y.hd = m->head_dim[L]; y.nkv = m->n_head_kv[L]; y.nff = m->ffn_len[L];
@@ -428,6 +520,15 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         push_rows(rows, d, 0, E);
         if ((rc = upload_tiled(m, rows, y.nff, &y.wdown, stage))) return rc;
         rows.clear();
+        if (xffn) {                                               // (second copies: not counted into weight_bytes, which says what a step streams)
+            xstage.resize(256 * (xg.gu_bytes > xg.dn_bytes ? xg.gu_bytes : xg.dn_bytes));
+            xffn_pack_gu((const uint8_t *)g->data, (const uint8_t *)u->data, xg, xstage.data());
+            if (dev_alloc(m, &y.xgu, 256 * xg.gu_bytes)) return -7;
+            HIP_TRY(hipMemcpy(y.xgu, xstage.data(), 256 * xg.gu_bytes, hipMemcpyHostToDevice));
+            xffn_pack_dn((const uint8_t *)d->data, xg, xstage.data());
+            if (dev_alloc(m, &y.xdn, 256 * xg.dn_bytes)) return -7;
+            HIP_TRY(hipMemcpy(y.xdn, xstage.data(), 256 * xg.dn_bytes, hipMemcpyHostToDevice));
+        }
         if (m->ple) {
             if (m->ple != 256) return fail(-2, "model_commit: per-layer width %d (256 is built)", m->ple);
             const HostTensor *ig = find(m, lname(L, "inp_gate.weight")), *pj = find(m, lname(L, "proj.weight"));
@@ -487,6 +588,15 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         return -7;
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
         return -7;
+    if (xffn) {
+        if (dev_alloc(m, &m->slabs, (size_t)LG_XCDS * max_rows * E) || dev_alloc(m, &m->xact, (size_t)LG_XCDS * max_rows * xg.C) ||
+            dev_alloc(m, &m->xq8, (size_t)LG_XCDS * xg.nb * LG_MU_DWORDS) || dev_alloc(m, &m->xsync, (size_t)1)) return -7;
+        HIP_TRY(hipMemset(m->xsync, 0, sizeof(XcdSync)));
+        HIP_TRY(hipMemset(m->xq8, 0, (size_t)LG_XCDS * xg.nb * LG_MU_DWORDS * 4));        // row slots past the block are read as operand rows
+        m->xffn_built = true; m->xffn_cls = xffn_class_of(xg);
+        m->xcd_ffn = getenv("LG_HIP_XCD_FFN") && atoi(getenv("LG_HIP_XCD_FFN")) != 0;     // off unless asked for: the separate kernels are faster (see lg_xffn.h)
+        m->xffn_delay = 0x100;
+    }
     HIP_TRY(hipMemset(m->ctl, 0, sizeof(StepCtl)));
     HIP_TRY(hipMemset(m->g_hidden, 0, (size_t)E * 4));
     m->sched_cap = 4096;
@@ -802,6 +912,20 @@ static int attention_u_launch(L &&launch, int rows, int rw, int nkv, int hd, int
     }
 }
 
+// the XCD-partitioned feed-forward launch: 256 workgroups of 512 threads, the instantiation of the shape's class
+template <int M>
+static void launch_xffn(Launcher &lx, const XffnArgs &a, int cls) {
+    if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
+        const size_t lds = xffn_lds(lg_xffn_geo(a.E, a.FF), M);
+        switch (cls) {
+            case 0: LAUNCH(KC_FFN, (lg_k_ffn_xcd<M, 1, 2, 1, 8, 8>), dim3(256), dim3(LG_XFFN_THREADS), lds, LG_XFFN_FIELDS(LG_XA, a) 0); break;
+            case 1: LAUNCH(KC_FFN, (lg_k_ffn_xcd<M, 3, 10, 2, 10, 40>), dim3(256), dim3(LG_XFFN_THREADS), lds, LG_XFFN_FIELDS(LG_XA, a) 0); break;
+            case 2: LAUNCH(KC_FFN, (lg_k_ffn_xcd<M, 4, 15, 2, 15, 60>), dim3(256), dim3(LG_XFFN_THREADS), lds, LG_XFFN_FIELDS(LG_XA, a) 0); break;
+            default: lx.rc = fail(-2, "ffn_xcd: no instantiation for this shape");
+        }
+    }
+}
+
 template <int M>
 static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry) {
     Launcher lx{ m, dry };
@@ -975,6 +1099,15 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             // verify blocks: 1..3 rows through v_dot4 with scalar operands, 4..8 rows through the matrix cores
             // (its float work per tile does not grow with the row count); each has its own activation order
             constexpr bool mfma = M >= 4 && M <= LG_HIP_MAX_ROWS;
+            if (mfma && m->xffn_built && m->xcd_ffn && y.xgu && have_x && pend_dout && pend_parts == 1 && !pend_os) {
+                // the whole half as one launch partitioned by XCD: row work, gate/up + GeGLU and the XCD's K share of
+                // ffn_down; the consumer adds the 8 slabs (the top of the segment tree)
+                XffnArgs f{ y.xgu, y.xdn, m->x[cur], pend_dout, pend_w, y.ffn_norm, m->x[cur ^ 1], m->slabs, m->xq8, m->xact,
+                            m->xsync, m->ctl, E, y.nff, m->eps, 1 << 18, m->xffn_delay, nullptr };
+                launch_xffn<M>(lx, f, m->xffn_cls);
+                cur ^= 1;
+                pend_dout = m->slabs; pend_parts = LG_XCDS; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
+            } else {
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
             rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             if constexpr (M > LG_HIP_MAX_ROWS)
@@ -987,6 +1120,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             // (the rows kernel adds four slabs; the fused rows + PLE gate kernel of verify blocks takes whole sums)
             pend_parts = launch_mm<M, false>(lx, KC_DOWN, d, !m->ple && m->down_kq);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
+            }
         }
         if (m->ple && y.winp_f) {   // per-layer embedding block, matrices kept in a float type: residual update, then the
             // gate on the f32 rows (gelu(.) * ipl in its epilogue), then the projection of the f32 gate rows
@@ -1004,7 +1138,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 LAUNCH(KC_PLEGATE, (lg_k_mm_plegate_wide<M>), dim3(m->ple / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
             } else {
                 // the residual update after ffn_down and its q8 happen inside the gate kernel (no rows kernel here)
-                RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps };
+                RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps, pend_parts };
                 LAUNCH(KC_PLEGATE, (lg_k_rows_plegate<M>), dim3(m->ple / 32, M), dim3(LG_WG), lds_mm(1, E), LG_RPG_FIELDS(LG_XA, r) 0);
                 cur ^= 1;
                 pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
@@ -1060,7 +1194,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1098,6 +1232,8 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
+    else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
+    else if (!strcmp(name, "xcd_ffn_delay")) m->xffn_delay = value < 0 ? 0 : value > 0x3FF ? 0x3FF : value;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
 }
@@ -1212,7 +1348,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "");
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -1356,8 +1492,8 @@ static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int
         const Layer &y = m->L[L];
         b[KC_QKV] += (double)m->E * y.qkv_m * q;
         b[KC_O] += (double)y.qd * m->E * q;
-        b[KC_GATEUP] += 2.0 * m->E * y.nff * q;
-        b[KC_DOWN] += (double)y.nff * m->E * q;
+        if (m->xffn_built && m->xcd_ffn && rows >= 4) b[KC_FFN] += 3.0 * m->E * y.nff * q;
+        else { b[KC_GATEUP] += 2.0 * m->E * y.nff * q; b[KC_DOWN] += (double)y.nff * m->E * q; }
         if (m->ple) { const double pq = y.winp_f ? 4.0 : q; b[KC_PLEGATE] += (double)m->E * m->ple * pq; b[KC_PLEPROJ] += (double)m->ple * m->E * pq; }
         const int window = (y.is_local && m->window > 0) ? m->window : 0;
         const int last = pos + rows - 1, start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -1605,7 +1741,7 @@ extern "C" int lg_hip_rows_ple_gate(const float *x, const float *dout, const flo
     HIP_TRY(hipMemcpy(di, ipl, (size_t)rows * ple * 4, hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(dg, tiled.data(), tiled.size(), hipMemcpyHostToDevice));
     PleGateArgs a{ dg, E, ple, nullptr, di, 0, 1, dq };
-    RowsPleGateArgs r{ a, dx, dd, dw, dxo, eps };
+    RowsPleGateArgs r{ a, dx, dd, dw, dxo, eps, 1 };
     switch (rows) {
 #define CASE(M) case M: rc = set_lds(lg_k_rows_plegate<M>, lds_mm(1, E)); \
         if (!rc) hipLaunchKernelGGL((lg_k_rows_plegate<M>), dim3(ple / 32, M), dim3(LG_WG), lds_mm(1, E), nullptr, LG_RPG_FIELDS(LG_XA, r) 0); break;
@@ -1914,5 +2050,96 @@ extern "C" int lg_hip_xcd_handover(int set_mode, int sel, int n, int store_scope
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpy(res, a.res, (size_t)n * 16, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// ---- the XCD-partitioned feed-forward half on its own (tests, timing) ------------------------------
+// x_out = x + rmsnorm(dout) * w_post; h = rmsnorm(x_out) * w_pre; act = gelu(gate . q8(h)) * (up . q8(h));
+// out = down . q8(act): lg_k_ffn_xcd on host data, the 8 slabs added here in tree order.
+extern "C" int lg_hip_ffn_xcd(const float *x, const float *dout, const float *w_post, const float *w_pre,
+                              const void *gate, const void *up, const void *down, int rows, int E, int FF, float eps,
+                              float *x_out, float *act, float *out, int repeats, float *kernel_ms, int flush_mb, int delay_w, int64_t *stamps) {
+    if (!x || !dout || !w_post || !w_pre || !gate || !up || !down) return fail(-1, "ffn_xcd: null input");
+    const XffnGeo g = lg_xffn_geo(E, FF);
+    const int cls = xffn_class_of(g);
+    if (rows < 4 || rows > LG_HIP_MAX_ROWS || cls < 0) return fail(-2, "ffn_xcd: rows %d (4..%d), E %d, FF %d: no instantiation for this shape", rows, LG_HIP_MAX_ROWS, E, FF);
+    if (lg_hip_device_count() < 1) return fail(-3, "ffn_xcd: no HIP device");
+    if (cu_count() != LG_XCDS * LG_XCD_WGS) return fail(-3, "ffn_xcd: the kernel needs %d compute units in %d XCDs, this device has %d", LG_XCDS * LG_XCD_WGS, LG_XCDS, cu_count());
+    Scratch sc;
+    std::vector<uint8_t> stage(256 * (g.gu_bytes > g.dn_bytes ? g.gu_bytes : g.dn_bytes));
+    uint8_t *dgu, *ddn; float *dx, *dd, *dwp, *dwr, *dxo, *dslabs, *dact; uint32_t *dxq; XcdSync *dsync; StepCtl *ctl;
+    const size_t n = (size_t)rows * E;
+    if (sc.get(&dgu, 256 * g.gu_bytes) || sc.get(&ddn, 256 * g.dn_bytes) || sc.get(&dx, n) || sc.get(&dd, n) || sc.get(&dwp, (size_t)E) ||
+        sc.get(&dwr, (size_t)E) || sc.get(&dxo, n) || sc.get(&dslabs, LG_XCDS * n) || sc.get(&dact, (size_t)LG_XCDS * rows * g.C) ||
+        sc.get(&dxq, (size_t)LG_XCDS * g.nb * LG_MU_DWORDS) || sc.get(&dsync, (size_t)1) || sc.get(&ctl, (size_t)1)) return -7;
+    xffn_pack_gu((const uint8_t *)gate, (const uint8_t *)up, g, stage.data());
+    HIP_TRY(hipMemcpy(dgu, stage.data(), 256 * g.gu_bytes, hipMemcpyHostToDevice));
+    xffn_pack_dn((const uint8_t *)down, g, stage.data());
+    HIP_TRY(hipMemcpy(ddn, stage.data(), 256 * g.dn_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dx, x, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dd, dout, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dwp, w_post, (size_t)E * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dwr, w_pre, (size_t)E * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(dsync, 0, sizeof(XcdSync)));
+    HIP_TRY(hipMemset(dxq, 0, (size_t)LG_XCDS * g.nb * LG_MU_DWORDS * 4));
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    hipStream_t st;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    lg_hip_model shim;
+    shim.stream = st;
+    Launcher lx{ &shim, false };
+    // measurement runs: something else streams through the caches between two launches (the step's weights never
+    // come from a cache), and every workgroup records the device clock at its phase boundaries
+    unsigned char *dflush = nullptr;
+    unsigned long long *dstamps = nullptr;
+    if (flush_mb > 0 && sc.get(&dflush, (size_t)flush_mb << 20)) return -7;
+    if (stamps && sc.get(&dstamps, (size_t)512 * LG_XFFN_STAMPS)) return -7;
+    if (dstamps) HIP_TRY(hipMemset(dstamps, 0, (size_t)512 * LG_XFFN_STAMPS * 8));
+    XffnArgs f{ dgu, ddn, dx, dd, dwp, dwr, dxo, dslabs, dxq, dact, dsync, ctl, E, FF, eps, 1 << 16, delay_w, dstamps };
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        for (int r = 0; r < repeats + 1 && !lx.rc; ++r) {
+            if (r == 1) HIP_TRY(hipEventRecord(e0, st));
+            if (dflush) HIP_TRY(hipMemsetAsync(dflush, r, (size_t)flush_mb << 20, st));
+            switch (rows) {
+#define CASE(M) case M: launch_xffn<M>(lx, f, cls); break;
+                CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+            }
+        }
+        if (lx.rc) return lx.rc;
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipGetLastError());
+        float t = 0;
+        if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+        if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+        return 0;
+    };
+    int rc = body();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipStreamDestroy(st);
+    if (rc) return rc;
+    StepCtl c;
+    HIP_TRY(hipMemcpy(&c, ctl, sizeof c, hipMemcpyDeviceToHost));
+    if (c.err) return fail(-9, "ffn_xcd: the kernel reported %s%s (err 0x%x)", (c.err & LG_XFFN_ERR_PLACE) ? "a workgroup on an unexpected XCD " : "",
+                           (c.err & LG_XFFN_ERR_WAIT) ? "a hand-over that was given up" : "", c.err);
+    if (stamps) HIP_TRY(hipMemcpy(stamps, dstamps, (size_t)512 * LG_XFFN_STAMPS * 8, hipMemcpyDeviceToHost));
+    if (x_out) HIP_TRY(hipMemcpy(x_out, dxo, n * 4, hipMemcpyDeviceToHost));
+    if (act) {                                            // [rows][FF] from the 8 per-XCD pieces [rows][FF/8]
+        std::vector<float> pieces((size_t)LG_XCDS * rows * g.C);
+        HIP_TRY(hipMemcpy(pieces.data(), dact, pieces.size() * 4, hipMemcpyDeviceToHost));
+        for (int xc = 0; xc < LG_XCDS; ++xc)
+            for (int j = 0; j < rows; ++j)
+                memcpy(act + (size_t)j * FF + (size_t)xc * g.C, pieces.data() + ((size_t)xc * rows + j) * g.C, (size_t)g.C * 4);
+    }
+    if (out) {
+        std::vector<float> p(LG_XCDS * n);
+        HIP_TRY(hipMemcpy(p.data(), dslabs, p.size() * 4, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < n; ++i)
+            out[i] = ((p[i] + p[n + i]) + (p[2 * n + i] + p[3 * n + i])) + ((p[4 * n + i] + p[5 * n + i]) + (p[6 * n + i] + p[7 * n + i]));
+    }
     return 0;
 }

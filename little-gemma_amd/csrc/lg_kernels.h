@@ -121,6 +121,16 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(const StepCtl *ctl, LG_ROW_FI
         const float4 *dr = (const float4 *)(s.dout + (size_t)j * E), *wr = (const float4 *)s.w_post;
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { dv[v] = dr[t + 256 * v]; wpost[v] = wr[t + 256 * v]; }
+        if (s.dparts == 8) {                                 // ... over the 8 XCDs: the top three levels of the tree
+            const size_t slab = (size_t)M * nq;
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 *b = dr + t + 256 * v;
+                const float4 p1 = b[slab], p2 = b[2 * slab], p3 = b[3 * slab], p4 = b[4 * slab], p5 = b[5 * slab], p6 = b[6 * slab], p7 = b[7 * slab], p0 = dv[v];
+                dv[v] = make_float4(((p0.x + p1.x) + (p2.x + p3.x)) + ((p4.x + p5.x) + (p6.x + p7.x)), ((p0.y + p1.y) + (p2.y + p3.y)) + ((p4.y + p5.y) + (p6.y + p7.y)),
+                                    ((p0.z + p1.z) + (p2.z + p3.z)) + ((p4.z + p5.z) + (p6.z + p7.z)), ((p0.w + p1.w) + (p2.w + p3.w)) + ((p4.w + p5.w) + (p6.w + p7.w)));
+            }
+        }
         if (s.dparts == 4) {                                 // top of the K-segment tree of a matmul that was split over four workgroups
             const size_t slab = (size_t)M * nq;
             #pragma unroll
@@ -716,8 +726,9 @@ struct RowsPleGateArgs {
     const float   *x, *dout, *w_post;   // [M][E] residual, [M][E] ffn_down output, [E]
     float         *x_out;               // [M][E]
     float          eps;
+    int            dparts;              // 8: dout is eight [M][E] slabs of partial sums (one per XCD), added here in tree order; else 1
 };
-#define LG_RPG_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const uint8_t *, gw, g.w, v) X(int, gk, g.k, v) X(int, gple, g.ple, v) X(const float *, gipl, g.ipl, v) X(int, glayer, g.layer, v) X(int, gnl, g.n_layer, v) X(int8_t *, gpq, g.pq, v) X(const int8_t *, gq_in, g.q_in, v) X(float *, x_out, x_out, v) X(float, eps, eps, v)
+#define LG_RPG_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const uint8_t *, gw, g.w, v) X(int, gk, g.k, v) X(int, gple, g.ple, v) X(int, dparts, dparts, v) X(const float *, gipl, g.ipl, v) X(int, glayer, g.layer, v) X(int, gnl, g.n_layer, v) X(int8_t *, gpq, g.pq, v) X(const int8_t *, gq_in, g.q_in, v) X(float *, x_out, x_out, v) X(float, eps, eps, v)
 template <int M>
 __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, _) int p_end_) {
     RowsPleGateArgs a; LG_RPG_FIELDS(LG_XI, a)
@@ -739,6 +750,16 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, 
         const float4 *wr = (const float4 *)a.w_post, *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; dv[v] = dr[t + 256 * v]; wp[v] = wr[t + 256 * v]; }
+        if (a.dparts == 8) {                                  // the top three levels of the K-segment tree of an ffn_down cut over the 8 XCDs
+            const size_t slab = (size_t)M * nq;
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 *b = dr + t + 256 * v;
+                const float4 p1 = b[slab], p2 = b[2 * slab], p3 = b[3 * slab], p4 = b[4 * slab], p5 = b[5 * slab], p6 = b[6 * slab], p7 = b[7 * slab], p0 = dv[v];
+                dv[v] = make_float4(((p0.x + p1.x) + (p2.x + p3.x)) + ((p4.x + p5.x) + (p6.x + p7.x)), ((p0.y + p1.y) + (p2.y + p3.y)) + ((p4.y + p5.y) + (p6.y + p7.y)),
+                                    ((p0.z + p1.z) + (p2.z + p3.z)) + ((p4.z + p5.z) + (p6.z + p7.z)), ((p0.w + p1.w) + (p2.w + p3.w)) + ((p4.w + p5.w) + (p6.w + p7.w)));
+            }
+        }
     }
     uint4 wq[LG_MAXV]; uint32_t wsc[LG_MAXV];
     #pragma unroll

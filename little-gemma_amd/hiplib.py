@@ -375,6 +375,24 @@ def rows_ple_gate(x, dout, w_post, w_gate_q4_0, ipl, eps=1e-6):
     return dict(x_out=x_out, pq=pq, pd=pd, psum=psum)
 
 
+def ffn_xcd(x, dout, w_post, w_pre, gate_q4_0, up_q4_0, down_q4_0, FF, eps=1e-6, repeats=0, flush_mb=0, want_stamps=False, delay_w=0):
+    """The XCD-partitioned feed-forward half of a layer through the C ABI.  x, dout: [rows, E] (rows 4..8); gate / up:
+    FF q4_0 rows of E, down: E q4_0 rows of FF.  Returns dict(x_out, act [rows, FF], out [rows, E], kernel_ms)."""
+    H = load_hip()
+    H.lg_hip_ffn_xcd.argtypes = [f32p, f32p, f32p, f32p, u8p, u8p, u8p, C.c_int, C.c_int, C.c_int, C.c_float,
+                                 f32p, f32p, f32p, C.c_int, C.POINTER(C.c_float), C.c_int, C.c_int, C.c_void_p]
+    x = np.ascontiguousarray(x, np.float32)
+    rows, E = x.shape
+    x_out = np.zeros_like(x); act = np.zeros((rows, FF), np.float32); out = np.zeros_like(x)
+    ms = C.c_float(0)
+    stamps = np.zeros((256, 2, 16), np.int64) if want_stamps else None
+    hip_check(H.lg_hip_ffn_xcd(x, np.ascontiguousarray(dout, np.float32), np.ascontiguousarray(w_post, np.float32),
+                               np.ascontiguousarray(w_pre, np.float32), np.ascontiguousarray(gate_q4_0, np.uint8),
+                               np.ascontiguousarray(up_q4_0, np.uint8), np.ascontiguousarray(down_q4_0, np.uint8),
+                               rows, E, FF, eps, x_out, act, out, repeats, C.byref(ms), flush_mb, delay_w, _opt(stamps)), "ffn_xcd")
+    return dict(x_out=x_out, act=act, out=out, kernel_ms=ms.value, stamps=stamps)
+
+
 def ple_inputs(pmp, proj_norm, pte_q4_0, n_tok, toks, n_layer, ple, E, eps=1e-6):
     """Isolated per-layer-input kernel through the C ABI.  pmp: [rows, n_layer*ple] raw projection; pte_q4_0: n_tok
     q4_0 rows of n_layer*ple; toks: [rows].  Returns [rows, n_layer*ple]."""

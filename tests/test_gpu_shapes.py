@@ -22,10 +22,11 @@ def seed_both(gpu, o, ob, okv, ctx, seed):
         gpu.kv_write(L, 0, k.view(np.uint16)); gpu.kv_write(L, 1, v.view(np.uint16))
 
 
-@pytest.mark.parametrize("name,ctx,steps", [("e4b", 2048, 3), ("g12b", 8192, 2)])
-def test_verify_steps_at_full_shape(lg, ob, gpu_required, model_path, name, ctx, steps):
+@pytest.mark.parametrize("name,ctx,steps,rows", [("e4b", 2048, 3, 5), ("g12b", 8192, 2, 5),
+                                                 ("e4b", 2048, 2, 4), ("g12b", 8192, 2, 4)])    # 4 rows: the reference's "block-4" (include/model.h:179-186)
+def test_verify_steps_at_full_shape(lg, ob, gpu_required, model_path, name, ctx, steps, rows):
     path, spec = model_path(name)
-    V, rows = spec["n_vocab"], 5
+    V = spec["n_vocab"]
     print(f"{name}: model written, loading", flush=True)
     o = ob.Oracle(path)
     gpu = lg.hiplib.HipBackend(path, ctx + 64, max_rows=rows)
