@@ -142,6 +142,12 @@ struct lg_hip_model {
     int device = 0;
     hipStream_t stream = nullptr;
     bool owns_stream = true;           // false for a draft head: it runs on its target's stream and never destroys it
+    // a second stream and two events for the one branch of a step that is off the critical chain: the per-layer
+    // inputs (per_layer_model_proj + lg_k_ipl), needed first by layer 0's per-layer gate, run beside layer 0's
+    // attention and feed-forward (the reference forks its decode graph the same way, src/cuda/model-cuda.cuh:917-935)
+    hipStream_t stream2 = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    int fork_ple = 0;                  // option: use it.  Off: replayed as a graph with a second branch the step takes 2.77 ms instead of 2.26
     // config
     int n_layer = 0, E = 0, H = 0, n_vocab = 0, window = 0, ple = 0, n_kv_start = 0, max_rows = 0;
     float eps = 0, base = 0, base_swa = 0, softcap = 0;
@@ -162,6 +168,7 @@ struct lg_hip_model {
     float *x[2] = { nullptr, nullptr }, *qkv = nullptr, *dout = nullptr, *pmp_raw = nullptr, *hidden_rows = nullptr,
           *g_hidden = nullptr, *logits = nullptr, *pval = nullptr, *q_rot = nullptr;
     int8_t *aq = nullptr, *gq = nullptr, *pq = nullptr, *hq = nullptr;     // q8 activation buffers (values + {scale,sum})
+    int8_t *eq = nullptr;              // q8 of the block's embedding rows: input of per_layer_model_proj (kept apart from hq, which layer 0 rewrites meanwhile)
     int *pidx = nullptr;
     StepCtl *ctl = nullptr;
     int32_t *sched = nullptr, *out = nullptr, *adv = nullptr;
@@ -228,7 +235,11 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
     if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&m->stream2, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&m->ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&m->ev_join, hipEventDisableTiming);
     if (e != hipSuccess) { delete m; return fail(-100 - (int)e, "hipStreamCreate: %s", hipGetErrorString(e)); }
+    if (getenv("LG_HIP_FORK")) m->fork_ple = atoi(getenv("LG_HIP_FORK")) != 0;   // the per-layer inputs as a second branch (comparison runs)
     *out = m;
     return 0;
 }
@@ -586,6 +597,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
         dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
+    if (m->ple && dev_alloc(m, &m->eq, R * E * 5 / 4 + (size_t)12 * E)) return -7;
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
         return -7;
     if (xffn) {
@@ -623,6 +635,9 @@ extern "C" void lg_hip_model_destroy(lg_hip_model *m) {
         for (size_t i = 0; i < v.size(); ++i) if (v[i] == m) { v.erase(v.begin() + i); break; }
     }
     if (m->owns_stream && m->stream) (void)hipStreamDestroy(m->stream);
+    if (m->stream2) (void)hipStreamDestroy(m->stream2);
+    if (m->ev_fork) (void)hipEventDestroy(m->ev_fork);
+    if (m->ev_join) (void)hipEventDestroy(m->ev_join);
     for (lg_hip_model *d : m->drafts) { d->target = nullptr; d->stream = nullptr; }        // orphaned heads refuse to run
     delete m;
 }
@@ -772,6 +787,8 @@ struct Launcher {
     lg_hip_model *m;
     bool dry;              // only raise LDS limits, launch nothing (done once before a capture)
     int rc = 0;
+    bool side = false;     // launches go to the model's second stream (the forked branch of a step)
+    hipStream_t stream() const { return side ? m->stream2 : m->stream; }
     // per-class timing: an event pair that the launch itself fills in (begin and end of the kernel's own execution,
     // what a kernel trace reports; a pair recorded around the launch also counts the packet handling, ~1.5 us)
     bool events(int cls, hipEvent_t *a, hipEvent_t *b) {
@@ -791,8 +808,8 @@ static void launch_timed(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds
 }
 
 #define LAUNCH(cls, kernel, grid, block, lds, ...) do { if (!lx.rc) { lx.rc = set_lds(kernel, lds); } if (!lx.rc && !lx.dry) { \
-    if (lx.m->prof.on) { hipEvent_t e0_, e1_; if (lx.events(cls, &e0_, &e1_)) launch_timed(kernel, grid, block, lds, lx.m->stream, e0_, e1_, __VA_ARGS__); } \
-    else hipLaunchKernelGGL(kernel, grid, block, lds, lx.m->stream, __VA_ARGS__); \
+    if (lx.m->prof.on) { hipEvent_t e0_, e1_; if (lx.events(cls, &e0_, &e1_)) launch_timed(kernel, grid, block, lds, lx.stream(), e0_, e1_, __VA_ARGS__); } \
+    else hipLaunchKernelGGL(kernel, grid, block, lds, lx.stream(), __VA_ARGS__); \
     lx.end(); } } while (0)
 
 // Compute units of the current device (asked once).
@@ -955,10 +972,10 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     }
 
     // rows kernel: fold the pending sub-layer output into the residual, norm with w_pre, quantize
-    auto rows = [&](const float *w_pre, float *h_out, int units = 0) {
+    auto rows = [&](const float *w_pre, float *h_out, int units = 0, int8_t *q_out = nullptr) {
         RowArgs s{};
         s.q_units = M <= LG_HIP_MAX_ROWS ? units : 0;
-        s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = m->hq;
+        s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = q_out ? q_out : m->hq;
         if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
         else s.x = m->x[cur];
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os; s.dparts = pend_parts;
@@ -1001,19 +1018,41 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         }
     };
 
+    bool join_ple = false;                         // the forked branch has to be waited for before its result is used
     if (m->ple) {
-        rows(nullptr, nullptr);
+        rows(nullptr, nullptr, 0, m->eq);
+        // the per-layer inputs are not needed before layer 0's per-layer gate: they run on the second stream, beside
+        // layer 0's attention and feed-forward (captured, the graph gets a second branch)
+        const bool fork = m->fork_ple && !dry && !m->prof.on && m->stream2 && !lx.rc;
+        if (fork) {
+            hipError_t e = hipEventRecord(m->ev_fork, m->stream);
+            if (e == hipSuccess) e = hipStreamWaitEvent(m->stream2, m->ev_fork, 0);
+            if (e != hipSuccess) lx.rc = fail(-100 - (int)e, "fork of the per-layer input branch: %s", hipGetErrorString(e));
+            lx.side = true;
+        }
         if (m->pmp_f) {                                       // kept in a float type: the f32 rows themselves are the input
             MmfArgs f{ m->pmp_f, E, m->ple * nl, m->x[cur], E, M, m->pmp_raw, m->ple * nl, nullptr, 0 };
             launch_mmf<M>(lx, KC_PMP, f);
         } else {
-        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->hq, nullptr };
+        MmArgs a{ m->pmp, E, m->ple * nl, m->pmp_raw, m->eq, nullptr };
         launch_mm<M, false>(lx, KC_PMP, a);
         }
         IplArgs i{ m->pmp_raw, m->ple, nl, M, m->proj_norm, m->pte, m->sched,
                    1.0f / sqrtf((float)E), sqrtf((float)m->ple), 1.0f / sqrtf(2.0f), m->eps };
         LAUNCH(KC_PMP, lg_k_ipl, dim3(nl, M), dim3(64), 0, i, m->ctl);
+        if (fork) {
+            lx.side = false;
+            hipError_t e = hipEventRecord(m->ev_join, m->stream2);
+            if (e != hipSuccess && !lx.rc) lx.rc = fail(-100 - (int)e, "fork of the per-layer input branch: %s", hipGetErrorString(e));
+            join_ple = true;
+        }
     }
+    auto join = [&]() {
+        if (!join_ple) return;
+        join_ple = false;
+        hipError_t e = hipStreamWaitEvent(m->stream, m->ev_join, 0);
+        if (e != hipSuccess && !lx.rc) lx.rc = fail(-100 - (int)e, "join of the per-layer input branch: %s", hipGetErrorString(e));
+    };
     // tiles a block of layer L can touch (a sliding layer needs only its window's, not the cache's), and whether the
     // layer takes the kernel that serves all rows of a block per (tile, kv head)
     auto layer_tiles = [&](int L) {
@@ -1122,6 +1161,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
             }
         }
+        if (m->ple) join();
         if (m->ple && y.winp_f) {   // per-layer embedding block, matrices kept in a float type: residual update, then the
             // gate on the f32 rows (gelu(.) * ipl in its epilogue), then the projection of the f32 gate rows
             rows(nullptr, nullptr);
@@ -1148,6 +1188,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             pend_dout = m->dout; pend_w = y.post_norm; pend_os = y.out_scale;
         }
     }
+    join();
     if constexpr (M > LG_HIP_MAX_ROWS) {
         if (with_head) return fail(-2, "a wide block has no head: verify blocks hold at most %d rows", LG_HIP_MAX_ROWS);
         if (!lx.rc && !dry) hipLaunchKernelGGL(lg_k_advance, dim3(1), dim3(1), 0, m->stream, m->ctl, M);
@@ -1194,7 +1235,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1233,6 +1274,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
+    else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
     else if (!strcmp(name, "xcd_ffn_delay")) m->xffn_delay = value < 0 ? 0 : value > 0x3FF ? 0x3FF : value;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
@@ -1348,7 +1390,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f");
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;

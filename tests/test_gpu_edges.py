@@ -141,7 +141,8 @@ def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
 def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, rows, name, over):
     """The options that pick between kernels for the same arithmetic (row work inside the q/k/v matmul, the
     attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay, ffn_down
-    cut by K quarter: the last case has the long FFN rows and no per-layer embeddings that kernel is for) change
+    cut by K quarter: the last case has the long FFN rows and no per-layer embeddings that kernel is for; the
+    per-layer inputs built on a second stream beside layer 0) change
     timing only: every combination leaves the same cache rows and the same logits rows of a verify block."""
     path, spec = model_path(name, **over)
     V = spec["n_vocab"]
@@ -164,9 +165,10 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, r
             gpu.close()
 
     base = run()
-    for opt in ("fuse_rows", "attn_rows", "head_mfma", "wide_prefill", "use_graph", "down_kq"):
-        print(f"rows={rows} option {opt}=0", flush=True)
-        got = run(**{opt: 0})
+    for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
+                     ("fork_ple", 1)):       # (the per-layer inputs as a second branch of the graph: off by default)
+        print(f"rows={rows} option {opt}={val}", flush=True)
+        got = run(**{opt: val})
         assert got[0] == base[0] and np.array_equal(got[1], base[1]), opt
         assert np.array_equal(got[2].view(np.uint32), base[2].view(np.uint32)), opt
         for a, b in zip(got[3], base[3]):
