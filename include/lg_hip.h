@@ -241,9 +241,14 @@ int  lg_hip_attention(const float *q, const uint16_t *kc, const uint16_t *vc, in
  * partials do not fit (rows * n_head * key tiles * hd * 4 bytes, plus small change) are refused with
  * -2.  The launches go to `stream` (a hipStream_t, NULL = the default stream) and the call returns
  * without waiting: out is valid once the stream has passed them.  All calls on one GPU share the
- * array, so two calls that overlap in time on one GPU race; calls on one stream are ordered. */
+ * array, so two calls that overlap in time on one GPU race; calls on one stream are ordered.
+ * The first call on a device asks the runtime for the array's address and raises the kernels' dynamic
+ * LDS limits, which a stream under capture does not allow: a caller that captures calls
+ * lg_hip_attention_noalloc_init() on that device beforehand (it allocates nothing either, does the same
+ * two things for every shape the entry point accepts, and is a no-op from then on). */
 int    lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, const uint16_t *d_vc, int rows, int n_head,
                                 int n_head_kv, int hd, int seq, int window, int pos, float *d_out, void *stream);
+int    lg_hip_attention_noalloc_init(void);
 size_t lg_hip_attention_noalloc_limit(void);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */

@@ -10,6 +10,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <map>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -769,17 +770,31 @@ static size_t attn_lds(int G, int hd, bool fused_post) {
     return fused_post ? ((b + 15) & ~(size_t)15) + (size_t)(LG_WG / 64) * hd * 4 : b;
 }
 
-// Kernels that want more than the default dynamic LDS limit have it raised once per (kernel, size).
+// Kernels that want more than the default dynamic LDS limit have it raised once per (device, kernel, size).  What
+// has been raised is kept in a fixed table (open addressing on the kernel's address; nothing is allocated, so a
+// look-up is safe on a path that promises not to allocate); a kernel that finds no free slot has its limit set on
+// every call, which costs time and nothing else.
+struct LdsRaised { const void *fn; int dev; size_t bytes; };
+static LdsRaised g_lds_raised[1024];
+static std::mutex g_lds_mu;
 template <typename K>
 static int set_lds(K kernel, size_t bytes) {
-    static std::map<const void *, size_t> raised;
     if (bytes <= 48 * 1024) return 0;
     if (bytes > 160 * 1024) return fail(-8, "kernel needs %zu bytes of LDS (160 KiB per workgroup)", bytes);
     const void *fn = reinterpret_cast<const void *>(kernel);
-    auto it = raised.find(fn);
-    if (it != raised.end() && it->second >= bytes) return 0;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_lds_mu);
+    const size_t n = sizeof(g_lds_raised) / sizeof(g_lds_raised[0]);
+    size_t at = ((uintptr_t)fn >> 4) * 0x9E3779B97F4A7C15ull >> 54;          // 10 bits
+    LdsRaised *slot = nullptr;
+    for (size_t probe = 0; probe < 32; ++probe, at = (at + 1) % n) {
+        LdsRaised &e = g_lds_raised[at];
+        if (!e.fn || (e.fn == fn && e.dev == dev)) { slot = &e; break; }
+    }
+    if (slot && slot->fn && slot->bytes >= bytes) return 0;
     HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
-    raised[fn] = bytes;
+    if (slot) { slot->fn = fn; slot->dev = dev; slot->bytes = bytes; }
     return 0;
 }
 
@@ -1934,6 +1949,38 @@ static size_t up256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 extern "C" size_t lg_hip_attention_noalloc_limit(void) { return LG_NOALLOC_BYTES; }
 
+// Everything the entry point needs from the runtime besides launches, for the current device: the array's address
+// and, for every kernel it may launch with more than the default dynamic LDS, the limit raised to the most any
+// accepted shape asks for.  Neither call is legal while a stream is being captured, so a capturing caller calls
+// this first; the entry point calls it by itself on its first use on a device.
+template <int M>
+static int noalloc_raise_rows() {
+    int rc = set_lds(lg_k_attn_rows<M, 256>, AttnRowsGeo<256>::bytes(M * 8));
+    if (!rc) rc = set_lds(lg_k_attn_rows<M, 128>, AttnRowsGeo<128>::bytes(M * 8));
+    if (!rc) rc = set_lds(lg_k_attn_rows<M, 64>, AttnRowsGeo<64>::bytes(M * 8));
+    return rc;
+}
+extern "C" int lg_hip_attention_noalloc_init(void) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= LG_NOALLOC_DEVICES) return fail(-3, "attention_noalloc: device %d (0..%d are served)", dev, LG_NOALLOC_DEVICES - 1);
+    if (g_noalloc_ptr[dev]) return 0;
+    int rc = set_lds(lg_k_attn<false, 1>, attn_lds(8, 512, false));
+    if (!rc) rc = noalloc_raise_rows<2>();
+    if (!rc) rc = noalloc_raise_rows<3>();
+    if (!rc) rc = noalloc_raise_rows<4>();
+    if (!rc) rc = noalloc_raise_rows<5>();
+    if (!rc) rc = noalloc_raise_rows<6>();
+    if (!rc) rc = noalloc_raise_rows<7>();
+    if (!rc) rc = noalloc_raise_rows<8>();
+    if (rc) return rc;
+    void *p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(lg_noalloc_scratch)));
+    if (!p) return fail(-3, "attention_noalloc: the working array has no address on device %d", dev);
+    g_noalloc_ptr[dev] = (unsigned char *)p;
+    return 0;
+}
+
 extern "C" int lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, const uint16_t *d_vc, int rows, int n_head,
                                         int n_head_kv, int hd, int seq, int window, int pos, float *d_out, void *stream) {
     if (!d_q || !d_kc || !d_vc || !d_out) return fail(-1, "attention_noalloc: null argument");
@@ -1955,10 +2002,8 @@ extern "C" int lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, 
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= LG_NOALLOC_DEVICES) return fail(-3, "attention_noalloc: device %d (0..%d are served)", dev, LG_NOALLOC_DEVICES - 1);
     if (!g_noalloc_ptr[dev]) {
-        void *p = nullptr;
-        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(lg_noalloc_scratch)));
-        if (!p) return fail(-3, "attention_noalloc: the working array has no address on device %d", dev);
-        g_noalloc_ptr[dev] = (unsigned char *)p;
+        const int irc = lg_hip_attention_noalloc_init();
+        if (irc) return irc;
     }
     unsigned char *base = g_noalloc_ptr[dev];
     StepCtl *ctl = (StepCtl *)base;
