@@ -26,6 +26,8 @@ sys.path.insert(0, ROOT)
 lg = importlib.import_module("little-gemma_amd")
 
 HBM_PEAK_GBS = 8000.0
+FLOOR_LAUNCH_US = 1.55          # a dependent kernel boundary inside a captured graph on this part (bench.py --launch-floor)
+FLOOR_STREAM_GBS = 6000.0       # what a plain streaming kernel sustains from HBM here
 i32a = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
 # HBM bytes per launch of the dominant kernel (gate/up + GeGLU at the E4B shape), from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in the file named below (scaled by the copy-kernel calibration given
@@ -64,8 +66,7 @@ def seed_cache(gpu, info, layers, ctx, seed):
         V = np.zeros((rows, width), np.float16)
         K[:n] = (rng.standard_normal((n, width), np.float32) * kstd).astype(np.float16)
         V[:n] = rng.standard_normal((n, width), np.float32).astype(np.float16)
-        if rows < ctx:      # ring: row r holds the latest position p < ctx with p % rows == r: any filled row is fine
-            pass
+        # (a ring of fewer rows than ctx: row r stands for the latest position p < ctx with p % rows == r; any filled row will do)
         gpu.kv_write(L, 0, K.view(np.uint16))
         gpu.kv_write(L, 1, V.view(np.uint16))
         filled[L] = (K, V)
@@ -292,11 +293,15 @@ def main():
     ok_adv = bool(np.array_equal(adv, expect_adv))
     # greedy successors must reproduce the plain-decode sequence wherever they are valid
     seq = [first_tok] + greedy
-    at, ok_tok = 0, True
-    for s in range(total):
-        for j in range(int(adv[s])):
-            ok_tok &= int(out[s, j]) == seq[at + j + 1]
-        at += int(adv[s])
+
+    def successors_follow_plain_decode(out, adv):
+        at, ok = 0, True
+        for s in range(len(adv)):
+            for j in range(int(adv[s])):
+                ok &= int(out[s, j]) == seq[at + j + 1]
+            at += int(adv[s])
+        return bool(ok)
+    ok_tok = successors_follow_plain_decode(out, adv)
     timed_tokens = int(adv[a.warmup:].sum())
     value = timed_tokens / (ms * 1e-3)
 
@@ -317,6 +322,13 @@ def main():
                 "bytes_per_launch": dom["bytes"] / max(dom["launches"], 1), "ms_per_launch": dom["ms"] / max(dom["launches"], 1),
                 "launches_per_step": dom["launches"]}
     step_gbs = step_bytes / (ms / a.steps * 1e-3) / 1e9
+    # what a class cannot go below as long as it keeps its launches: a kernel boundary per launch plus its bytes at the
+    # rate a streaming kernel reaches on this part; the ratio says how much of a class's time is neither of the two
+    for c in prof:
+        c["floor_us"] = c["launches"] * FLOOR_LAUNCH_US + c["bytes"] / (FLOOR_STREAM_GBS * 1e9) * 1e6
+        c["over_floor"] = (c["ms"] * 1e3 / c["floor_us"]) if c["floor_us"] > 0 else None
+    floor_ms = sum(c["floor_us"] for c in prof) * 1e-3
+    uncaptured_ms = sum(c["ms"] for c in prof)
     # matrix-core utilisation of the verify step's one MFMA GEMM (gate/up for blocks of 4..8 rows): the weights of a
     # launch (bytes / 0.5625 elements) times the block's rows are the useful MACs, the 8 row slots of the tiles the
     # issued ones.  It is a bandwidth-bound kernel: the figure says how far the matrix cores are from mattering.
@@ -339,6 +351,13 @@ def main():
         "roofline": roofline,
         "step_hbm": {"bytes_per_step": step_bytes, "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": step_gbs / HBM_PEAK_GBS},
+        "floor": {"launch_us": FLOOR_LAUNCH_US, "stream_GBs": FLOOR_STREAM_GBS, "step_floor_ms": floor_ms,
+                  "ms_per_step_over_floor": (ms / a.steps) / floor_ms,
+                  "launches_per_step": int(sum(c["launches"] for c in prof)),
+                  "uncaptured_class_sum_ms": uncaptured_ms, "uncaptured_over_graph_step": uncaptured_ms / (ms / a.steps),
+                  "note": "kernel_classes are timed un-captured, kernel begin to end; in the captured step the launch gaps "
+                          "overlap the tails of the kernels before them, so the class durations (each also carrying its event pair) add up to more than "
+                          "ms_per_step"},
         "verify_mfma": mfma,
         "kernel_classes": [{k: (round(v, 5) if isinstance(v, float) else v) for k, v in c.items()} for c in prof],
         "checks": {"accept_counts_as_scheduled": ok_adv, "tokens_equal_plain_decode": ok_tok, "final_pos": final_pos,
@@ -353,11 +372,14 @@ def main():
         if a.warmup:
             gpu.schedule_time(a.warmup)
         ms4 = gpu.schedule_time(a.steps)
-        _, adv4, _ = gpu.schedule_wait()
+        out4, adv4, _ = gpu.schedule_wait()
+        ok4 = bool(np.array_equal(adv4, expect4)) and successors_follow_plain_decode(out4, adv4)
         line["block4"] = {"verify_rows": 4, "drafts": 3, "ms_per_step": ms4 / a.steps,
                           "value": int(adv4[a.warmup:].sum()) / (ms4 * 1e-3), "unit": "verified tok/s",
                           "mean_accepted_per_step": float(adv4[a.warmup:].mean()),
-                          "accept_counts_as_scheduled": bool(np.array_equal(adv4, expect4))}
+                          "accept_counts_as_scheduled": bool(np.array_equal(adv4, expect4)),
+                          "tokens_equal_plain_decode": successors_follow_plain_decode(out4, adv4)}
+        ok_tok = ok_tok and ok4
     # the loop a draft head drives (the reference's run.c with -mtp): per step K = rows-1 chained drafts on the
     # device head (synthetic gemma4-assistant weights: its drafts are rarely accepted, the step cost does not
     # depend on that), then the verify step; host clock around synchronous calls, from the seeded cache

@@ -61,6 +61,14 @@ void lg_hip_model_destroy(lg_hip_model *m);
 int  lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out);
 void lg_hip_kv_destroy(lg_hip_kv *kv);
 int  lg_hip_ring_rows(int window, int max_seq);
+/* What lg_hip_kv_create asks for besides the rings (no counterpart in the reference, whose attention
+ * keeps its partials per launch): bytes of attention partials, one slot of (max, sum, max_hd
+ * accumulators) per (row of the cache's widest block, head, key tile a block can touch).  The widest
+ * PROMPT block of a cache (*wide_rows: 512, 128, 32, or 0 = verify-width blocks only) is the largest
+ * whose partials stay within 2 GiB; any_global = the model has a layer without a sliding window.
+ * Arithmetic only: callable without a device. */
+size_t lg_hip_kv_partials(int max_seq, int window, int any_global, int max_rows, int n_head, int max_hd,
+                          int *wide_rows, int *tiles_max);
 /* rows/width of an owning layer's K (== V) storage; *rows = 0 for a layer that shares. */
 int  lg_hip_kv_layout(const lg_hip_kv *kv, int layer, int *rows, int *width);
 /* Copy whole cache rows (binary16 bit patterns) from/to host memory: which = 0 K, 1 V. */

@@ -51,6 +51,31 @@ extern "C" int lg_hip_ring_rows(int window, int max_seq) {
     return r < max_seq ? r : max_seq;
 }
 
+// The attention partials of a cache: one (max, sum, hd accumulators) slot per (row of the widest block, head, key
+// tile any block can touch).  A global layer's block late in a long cache touches every tile, so at the widest
+// block the slots grow with rows x max_seq: the widest PROMPT block of a cache is stepped down (512, 128, 32 rows,
+// then verify-width blocks only) until the partials fit LG_PARTIALS_BUDGET.  Pure arithmetic, no device needed.
+#define LG_PARTIALS_BUDGET ((size_t)2 << 30)
+extern "C" size_t lg_hip_kv_partials(int max_seq, int window, int any_global, int max_rows, int n_head, int max_hd,
+                                     int *wide_rows, int *tiles_max) {
+    const int steps[4] = { wide_rows_for(max_seq), LG_WIDE_MID, LG_WIDE, 0 };
+    size_t bytes = 0;
+    int wide = 0, tiles = 1;
+    for (int i = 0; i < 4; ++i) {
+        wide = steps[i];
+        if (i > 0 && wide >= steps[i - 1]) continue;
+        const int ring_span = window > 0 ? window + (wide > max_rows ? wide : max_rows) : max_seq;
+        const int span = any_global || window <= 0 ? max_seq : ring_span;
+        tiles = (span < max_seq ? span : max_seq) / 32 + 2;
+        const size_t slots = (size_t)(max_rows > wide ? max_rows : wide) * n_head * tiles;
+        bytes = slots * ((size_t)max_hd * 4 + 8);
+        if (bytes <= LG_PARTIALS_BUDGET || wide == 0) break;
+    }
+    if (wide_rows) *wide_rows = wide;
+    if (tiles_max) *tiles_max = tiles;
+    return bytes;
+}
+
 // ---- weight layout ----------------------------------------------------------------------------
 extern "C" int lg_hip_segments(int k) { return lg_segments(k); }
 
@@ -591,12 +616,15 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (max_rows != 1) return fail(-2, "model_commit: a draft head runs one row at a time");
     }
     m->host.clear();
-    const size_t R = (size_t)(max_rows > LG_WIDE_ROWS ? max_rows : LG_WIDE_ROWS);      // prefill runs blocks of LG_WIDE_ROWS rows
+    // Layer scratch holds the widest block that can run: LG_WIDE_ROWS for a model that takes prompts, max_rows for a
+    // draft head (it is never prefilled).  What only the head touches (final-norm rows, per-workgroup maxima, logits)
+    // holds max_rows: a prompt block has no head.
+    const size_t R = (size_t)(m->target || max_rows > LG_WIDE_ROWS ? max_rows : LG_WIDE_ROWS), HR = (size_t)max_rows;
     if (dev_alloc(m, &m->x[0], R * E) || dev_alloc(m, &m->x[1], R * E) || dev_alloc(m, &m->qkv, R * max_qkv) ||
-        dev_alloc(m, &m->dout, 4 * R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, R * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
+        dev_alloc(m, &m->dout, 4 * R * E) || dev_alloc(m, &m->q_rot, R * max_qd) || dev_alloc(m, &m->hidden_rows, HR * E) || dev_alloc(m, &m->g_hidden, (size_t)E) ||
         dev_alloc(m, &m->aq, R * max_qd * 5 / 4) || dev_alloc(m, &m->gq, R * max_ff * 5 / 4) || dev_alloc(m, &m->hq, R * E * 5 / 4 + (size_t)12 * E) ||
-        dev_alloc(m, &m->pval, R * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, R * (m->n_vocab / 32)) ||
-        dev_alloc(m, &m->logits, R * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
+        dev_alloc(m, &m->pval, HR * (m->n_vocab / 32)) || dev_alloc(m, &m->pidx, HR * (m->n_vocab / 32)) ||
+        dev_alloc(m, &m->logits, HR * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
     if (m->ple && dev_alloc(m, &m->eq, R * E * 5 / 4 + (size_t)12 * E)) return -7;
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
@@ -649,28 +677,29 @@ extern "C" int lg_hip_kv_create(lg_hip_model *m, int max_seq, lg_hip_kv **out) {
     if (max_seq < 1) return fail(-2, "kv_create: max_seq %d", max_seq);
     HIP_TRY(hipSetDevice(m->device));
     lg_hip_kv *kv = new lg_hip_kv();
-    kv->m = m; kv->max_seq = max_seq; kv->id = ++g_kv_ids; kv->wide_rows = wide_rows_for(max_seq);
+    kv->m = m; kv->max_seq = max_seq; kv->id = ++g_kv_ids;
     const int nl = m->n_layer;
     kv->seq.assign(nl, 0); kv->kv_dim.assign(nl, 0);
     kv->k.assign(nl, nullptr); kv->v.assign(nl, nullptr); kv->px_k.assign(nl, nullptr); kv->px_v.assign(nl, nullptr);
-    int tiles = 1, max_hd = 0;
+    int max_hd = 0, any_global = 0;
+    for (int L = 0; L < nl; ++L) {
+        const Layer &y = m->L[L];
+        if (y.hd > max_hd) max_hd = y.hd;
+        if (!(y.is_local && m->window > 0)) any_global = 1;
+    }
+    const size_t pbytes = lg_hip_kv_partials(max_seq, m->window, any_global, m->max_rows, m->H, max_hd, &kv->wide_rows, &kv->tiles_max);
     for (int L = 0; L < nl; ++L) {
         const Layer &y = m->L[L];
         kv->kv_dim[L] = y.kd;
-        if (y.hd > max_hd) max_hd = y.hd;
-        const bool ring = y.is_local && m->window > 0;
-        const int span = ring ? m->window + kv->wide_rows : max_seq;                // keys any block can touch
-        int t = (span < max_seq ? span : max_seq) / 32 + 2;
-        if (t > tiles) tiles = t;
         if (!y.owns) continue;
+        const bool ring = y.is_local && m->window > 0;
         kv->seq[L] = ring ? lg_hip_ring_rows(m->window, max_seq) : max_seq;
         const size_t bytes = (size_t)kv->seq[L] * y.kd * 2;
         hipError_t e1 = hipMalloc((void **)&kv->k[L], bytes), e2 = hipMalloc((void **)&kv->v[L], bytes);
         if (e1 != hipSuccess || e2 != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory at layer %d", L); }
         (void)hipMemset(kv->k[L], 0, bytes); (void)hipMemset(kv->v[L], 0, bytes);
     }
-    kv->tiles_max = tiles;
-    const size_t slots = (size_t)(m->max_rows > kv->wide_rows ? m->max_rows : kv->wide_rows) * m->H * tiles;
+    const size_t slots = pbytes / ((size_t)max_hd * 4 + 8);
     if (hipMalloc((void **)&kv->pm, slots * 4) != hipSuccess || hipMalloc((void **)&kv->pl, slots * 4) != hipSuccess ||
         hipMalloc((void **)&kv->pacc, slots * max_hd * 4) != hipSuccess) { lg_hip_kv_destroy(kv); return fail(-7, "kv_create: out of device memory for attention partials"); }
     HIP_TRY(hipDeviceSynchronize());
@@ -1146,7 +1175,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         }
         {   // attention output projection
             MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, nullptr };
-            launch_mm<M, false>(lx, KC_O, a);
+            pend_parts = launch_mm<M, false>(lx, KC_O, a);      // (four slabs for a wide block when n_head * head_dim > 4096)
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
         }
         {   // feed-forward: gate/up + GeGLU, then down
@@ -1449,8 +1478,8 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
     for (int done = 0; done < n;) {
         int rows = n - done < m->max_rows ? n - done : m->max_rows;
         if (wide_ok && n - done >= LG_WIDE_ROWS && kv->wide_rows >= LG_WIDE_ROWS) rows = LG_WIDE_ROWS;     // matrix-core blocks while the prompt lasts,
-        else if (wide_ok && n - done >= LG_WIDE_MID) rows = LG_WIDE_MID;
-        else if (wide_ok && n - done >= LG_WIDE) rows = LG_WIDE;        // a single row tile, then verify-width blocks for the tail
+        else if (wide_ok && n - done >= LG_WIDE_MID && kv->wide_rows >= LG_WIDE_MID) rows = LG_WIDE_MID;
+        else if (wide_ok && n - done >= LG_WIDE && kv->wide_rows >= LG_WIDE) rows = LG_WIDE;        // a single row tile, then verify-width blocks for the tail
         int rc = check_block(m, kv, toks + done, rows, rows, pos0 + done, true);
         if (rc) return rc;
         if ((rc = load_block(m, toks + done, rows, pos0 + done))) return rc;
@@ -1517,6 +1546,9 @@ extern "C" int lg_hip_schedule_wait(lg_hip_model *m, int32_t *out, int32_t *adv,
     HIP_TRY(hipStreamSynchronize(m->stream));
     StepCtl c;
     HIP_TRY(hipMemcpy(&c, m->ctl, sizeof c, hipMemcpyDeviceToHost));
+    // the step counter is device state: never copy more than the schedule that was loaded holds
+    if (c.step < 0 || c.step > m->sched_loaded)
+        return fail(-6, "schedule_wait: the device reports %d steps done, %d were loaded", c.step, m->sched_loaded);
     if (out) HIP_TRY(hipMemcpy(out, m->out, (size_t)c.step * m->sched_rows * 4, hipMemcpyDeviceToHost));
     if (adv) HIP_TRY(hipMemcpy(adv, m->adv, (size_t)c.step * 4, hipMemcpyDeviceToHost));
     if (final_pos) *final_pos = c.pos;

@@ -484,8 +484,7 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(LG_GEGLU_FIELDS(LG_XP, _)
     // of the first weight tiles and nothing waits for them before the end (a wait here would also be one for the tiles).
     // (nunits <= 16: k <= 4096 and at most three rows.)  The load is written as an instruction of its own: a volatile
     // load is followed by a wait for every load in flight, a plain one with no use before the end is moved there.  Its
-    // register stays reserved until the use at the end of the kernel, by when the loop's own waits for the later
-    // weight loads have also covered this older one.
+    // register stays reserved until the wait at the end of the loop, which names it as an operand.
     int touch;
     {
         const int *tp = (const int *)a.q_in + ((size_t)s * nunits + (lane < nunits ? lane : nunits - 1)) * 32;
@@ -538,7 +537,8 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_t(LG_GEGLU_FIELDS(LG_XP, _)
             }
         }
     }
-    asm volatile("" :: "v"(touch));
+    // the explicit wait for that load (after the loop every load of this wavefront has long returned: it costs nothing)
+    asm volatile("s_waitcnt vmcnt(0)" :: "v"(touch) : "memory");
     #pragma unroll
     for (int j = 0; j < M; ++j) red[s][j][lane] = p[j];
     __syncthreads();

@@ -73,6 +73,32 @@ def test_ring_rows_agree_with_the_oracle(lg, ob):
         assert H.lg_hip_ring_rows(window, max_seq) == L.lgo_ring_rows(window, max_seq)
 
 
+def test_attention_partials_of_a_cache_stay_within_their_budget(lg):
+    """The byte count lg_hip_kv_create asks for beside the rings, at the E4B and 12B shapes (8 verify rows): the
+    widest prompt block steps down with the cache length so that rows x heads x key tiles x (head_dim + 2) floats
+    never pass 2 GiB; the closed form is recomputed here from the returned block width."""
+    import ctypes as C
+    H = lg.hiplib.load_hip()
+    H.lg_hip_kv_partials.restype = C.c_size_t
+    H.lg_hip_kv_partials.argtypes = [C.c_int] * 6 + [C.POINTER(C.c_int)] * 2
+    cases = {  # (heads, window) -> max_seq -> widest prompt block
+        (8, 512): {600: 128, 4136: 512, 8192: 512, 32768: 128, 131072: 32},
+        (16, 1024): {4136: 512, 32768: 32, 131072: 0},
+    }
+    for (heads, window), by_seq in cases.items():
+        for max_seq, want_wide in by_seq.items():
+            wide, tiles = C.c_int(-1), C.c_int(-1)
+            got = H.lg_hip_kv_partials(max_seq, window, 1, 8, heads, 256, C.byref(wide), C.byref(tiles))
+            assert wide.value == want_wide, (heads, max_seq, wide.value)
+            assert tiles.value == max_seq // 32 + 2
+            assert got == max(wide.value, 8) * heads * tiles.value * (256 * 4 + 8)
+            assert got <= 2 << 30
+    # sliding layers only: the tiles a block can touch are bounded by window + block
+    wide, tiles = C.c_int(), C.c_int()
+    H.lg_hip_kv_partials(131072, 512, 0, 8, 8, 256, C.byref(wide), C.byref(tiles))
+    assert wide.value == 512 and tiles.value == (512 + 512) // 32 + 2
+
+
 @pytest.mark.skipif(has_gpu(), reason="checks the behaviour of a machine without a GPU")
 def test_compute_calls_fail_loudly_without_a_device(lg, model_path):
     H = lg.hiplib.load_hip()

@@ -36,6 +36,17 @@ def test_wide_prefill_leaves_the_same_cache_and_logits(lg, ob, gpu_required, mod
     every cache row identical, the logits of the next position identical; and identical to the same
     prompt pushed through 8-row blocks only."""
     path, spec = model_path(name)
+    check_wide_prefill(lg, ob, path, spec, name, n_prompt)
+
+
+def test_wide_prefill_with_an_attention_output_of_32_segments(lg, ob, gpu_required, model_path):
+    """n_head * head_dim = 5120 > 4096: the attention output projection of a wide block is cut into four K quarters
+    whose slabs the next row kernel adds (as ffn_down's are at the larger shapes)."""
+    path, spec = model_path("tiny", n_head=80, n_head_kv=10)
+    check_wide_prefill(lg, ob, path, spec, "tiny with 80 heads", 200)
+
+
+def check_wide_prefill(lg, ob, path, spec, name, n_prompt):
     rng = np.random.default_rng(n_prompt)
     prompt = rng.integers(1, spec["n_vocab"], n_prompt).astype(np.int32)
     o = ob.Oracle(path)
