@@ -21,6 +21,7 @@
 #include "lg_fused.h"
 #include "lg_xcd.h"
 #include "lg_xffn.h"
+#include "lg_xtail.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
 #define LG_FUSE_ROWS_MAX 2         // widest block whose q/k/v matmul does the preceding row work itself
@@ -154,9 +155,9 @@ struct Layer {
 };
 
 enum KClass { KC_ROWS, KC_PMP, KC_QKV, KC_QKVPOST, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
-              KC_HEAD, KC_ACCEPT, KC_FFN, KC_COUNT };
+              KC_HEAD, KC_ACCEPT, KC_FFN, KC_TAIL, KC_COUNT };
 static const char *k_class_names[KC_COUNT] = { "rows_norm_quant", "ple_model_proj", "qkv", "qkv_post", "attn_tiles", "attn_merge",
-    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept", "ffn_xcd" };
+    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept", "ffn_xcd", "ple_tail" };
 
 struct Profile {
     bool on = false;
@@ -204,6 +205,11 @@ struct lg_hip_model {
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
+    // the per-layer-input block and the next row work as one launch on one XCD (lg_xtail.h)
+    int xcd_tail = 1;                        // option: 0 off, 1 for blocks that do not fold the row work into q/k/v, 2 for every verify block
+    XtailSync *tsync = nullptr;
+    unsigned long long *tstamps = nullptr;   // [LG_XTAIL_UNITS][8] phase stamps of the last such launch (option xcd_tail_stamps)
+    int tail_stamps = 0;
     bool xffn_built = false;                 // streams and working memory exist
     int xffn_cls = -1;                       // which instantiation serves the shape
     int xffn_delay = 0;                      // option: units of 64 clocks its compute wavefronts wait before they request their weights
@@ -627,6 +633,12 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         dev_alloc(m, &m->logits, HR * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
     if (m->ple && dev_alloc(m, &m->eq, R * E * 5 / 4 + (size_t)12 * E)) return -7;
+    if (m->ple) {
+        if (dev_alloc(m, &m->tsync, (size_t)1) || dev_alloc(m, &m->tstamps, (size_t)LG_XTAIL_UNITS * 8)) return -7;
+        HIP_TRY(hipMemset(m->tstamps, 0, (size_t)LG_XTAIL_UNITS * 8 * 8));
+        HIP_TRY(hipMemset(m->tsync, 0, sizeof(XtailSync)));
+        if (getenv("LG_HIP_XCD_TAIL")) m->xcd_tail = atoi(getenv("LG_HIP_XCD_TAIL"));
+    }
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
         return -7;
     if (xffn) {
@@ -987,6 +999,46 @@ static void launch_xffn(Launcher &lx, const XffnArgs &a, int cls) {
     }
 }
 
+// The per-layer-input block of a verify block of `rows` rows as the one-XCD launch lg_k_ple_tail: q4_0 matrices of the
+// 256-wide per-layer input, at most LG_XTAIL_UNITS (gate block, row) units, a chip whose workgroups are dealt over 8 XCDs
+static bool use_ple_tail(const lg_hip_model *m, int rows) {
+    if (!m->ple || !m->tsync || m->xcd_tail <= 0 || m->target || rows < 1 || rows > LG_HIP_MAX_ROWS) return false;
+    if (m->ple != 256 || (m->ple / 32) * rows > LG_XTAIL_UNITS || m->E % 256 || m->E > 4096 || (m->E + 1023) / 1024 > m->ple / 32) return false;
+    if (m->xcd_tail == 1 && rows <= LG_FUSE_ROWS_MAX && m->fuse_rows) return false;
+    return cu_count() == LG_XCDS * LG_XCD_WGS;
+}
+template <int M>
+static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
+    if constexpr (M <= LG_HIP_MAX_ROWS) {
+        lg_hip_model *m = lx.m;
+        const int E = a.r.g.k, U = (a.r.g.ple / 32) * M;
+        const int G = (E / 8 + 4 * U - 1) / (4 * U);
+        const size_t lds = (size_t)E * 5 / 4 + (size_t)M * a.r.g.ple * 5 / 4;
+        const dim3 grid(LG_XCDS * U);
+        // the U units wait for each other: all of them must be resident on the 32 CUs of one XCD at once
+        static int fits[5] = { 0, 0, 0, 0, 0 };              // per G: 0 unknown, 1 yes, -1 no (asked once, outside any capture)
+        if (G >= 1 && G <= 4 && !fits[G]) {
+            int per_cu = 0;
+            hipError_t e = hipErrorInvalidValue;
+            switch (G) {
+                case 1: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail<M, 1>, LG_WG, lds); break;
+                case 2: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail<M, 2>, LG_WG, lds); break;
+                case 3: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail<M, 3>, LG_WG, lds); break;
+                case 4: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail<M, 4>, LG_WG, lds); break;
+            }
+            fits[G] = (e == hipSuccess && per_cu * LG_XCD_WGS >= U) ? 1 : -1;
+        }
+        if (G < 1 || G > 4 || fits[G] < 0) { lx.rc = fail(-2, "ple_tail: %d units of %d row groups per wavefront do not fit one XCD", U, G); return; }
+        switch (G) {
+            case 1: LAUNCH(KC_TAIL, (lg_k_ple_tail<M, 1>), grid, dim3(LG_WG), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+            case 2: LAUNCH(KC_TAIL, (lg_k_ple_tail<M, 2>), grid, dim3(LG_WG), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+            case 3: LAUNCH(KC_TAIL, (lg_k_ple_tail<M, 3>), grid, dim3(LG_WG), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+            case 4: LAUNCH(KC_TAIL, (lg_k_ple_tail<M, 4>), grid, dim3(LG_WG), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+            default: lx.rc = fail(-2, "ple_tail: %d row groups per wavefront", G);
+        }
+    }
+}
+
 template <int M>
 static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry) {
     Launcher lx{ m, dry };
@@ -1062,6 +1114,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         }
     };
 
+    const bool tail = use_ple_tail(m, M);
+    bool rows_done = false;                        // the row work ahead of the next matmul has been done by the launch before it
     bool join_ple = false;                         // the forked branch has to be waited for before its result is used
     if (m->ple) {
         rows(nullptr, nullptr, 0, m->eq);
@@ -1116,7 +1170,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         bool fused_post = false;
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
-            if (can_fuse()) rows_mm(y.attn_norm, a, KC_QKV);
+            if (rows_done) { launch_mm<M, false>(lx, KC_QKV, a); rows_done = false; }      // (the previous layer's tail did this layer's row work)
+            else if (can_fuse()) rows_mm(y.attn_norm, a, KC_QKV);
             else { rows(y.attn_norm, nullptr); launch_mm<M, false>(lx, KC_QKV, a); }
             // blocks of the model itself, up to LG_HIP_MAX_ROWS rows: the attention kernel does this part as well
             fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
@@ -1220,6 +1275,22 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             if constexpr (M > LG_HIP_MAX_ROWS) {
                 rows(nullptr, nullptr);
                 LAUNCH(KC_PLEGATE, (lg_k_mm_plegate_wide<M>), dim3(m->ple / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
+            } else if (tail && (L + 1 < nl || with_head) && pend_dout && have_x && !pend_os) {
+                // the whole block and the row work that follows it (the next layer's, or the head's) in one launch on one XCD
+                const bool last = L + 1 == nl;
+                const bool head_m = M >= 4 && m->emb_rb && m->head_mfma;
+                XtailArgs f{};
+                f.r = RowsPleGateArgs{ a, m->x[cur], pend_dout, pend_w, nullptr, m->eps, pend_parts };
+                f.pw = y.wproj; f.pout = m->dout; f.w_post2 = y.post_norm; f.os = y.out_scale;
+                f.w_pre = last ? m->output_norm : m->L[L + 1].attn_norm;
+                f.x_out = m->x[cur ^ 1]; f.h_out = last ? m->hidden_rows : nullptr;
+                f.q = m->hq; f.q_units = last && head_m ? 2 : 0;
+                f.sync = m->tsync; f.spin_limit = 1 << 16; f.stamps = m->tail_stamps ? m->tstamps : nullptr;
+                launch_ple_tail<M>(lx, f);
+                cur ^= 1;
+                pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+                rows_done = true;
+                continue;
             } else {
                 // the residual update after ffn_down and its q8 happen inside the gate kernel (no rows kernel here)
                 RowsPleGateArgs r{ a, m->x[cur], pend_dout, pend_w, m->x[cur ^ 1], m->eps, pend_parts };
@@ -1240,7 +1311,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     } else
     if (with_head && !lx.rc) {
         const bool head_m = M >= 4 && m->emb_rb && m->head_mfma;
-        rows(m->output_norm, m->hidden_rows, head_m ? 2 : 0);
+        if (!rows_done) rows(m->output_norm, m->hidden_rows, head_m ? 2 : 0);
         int grid = 512;                                  // two workgroups per CU, each walks `passes` blocks of 64 rows
         int passes = (m->n_vocab / 64 + grid - 1) / grid;
         if (passes < 1) passes = 1;
@@ -1279,7 +1350,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "");
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1319,9 +1390,20 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
+    else if (!strcmp(name, "xcd_tail")) m->xcd_tail = value < 0 ? 0 : value > 2 ? 2 : value;
+    else if (!strcmp(name, "xcd_tail_stamps")) m->tail_stamps = value != 0;
     else if (!strcmp(name, "xcd_ffn_delay")) m->xffn_delay = value < 0 ? 0 : value > 0x3FF ? 0x3FF : value;
     else return fail(-2, "set_option: unknown option %s", name);
     return 0;
+}
+
+// What a kernel of a step left in StepCtl.err (a hand-over inside an XCD that was given up, or whose workgroups were not
+// on one XCD): the step's results are not to be used.
+static int step_err(const char *who, int err) {
+    if (!err) return 0;
+    return fail(-9, "%s: a kernel of the step reported %s%s(err 0x%x); its results are void", who,
+                (err & LG_XFFN_ERR_PLACE) ? "workgroups of one group on different XCDs " : "",
+                (err & LG_XFFN_ERR_WAIT) ? "a hand-over that was given up " : "", err);
 }
 
 static int load_block(lg_hip_model *m, const int32_t *toks, int rows, int pos) {
@@ -1343,7 +1425,9 @@ extern "C" int lg_hip_forward_spec(lg_hip_model *m, lg_hip_kv *kv, const int32_t
     if ((rc = launch_step(m, kv, rows, true))) return rc;
     HIP_TRY(hipMemcpyAsync(m->pin + 32, m->out, (size_t)rows * 4, hipMemcpyDeviceToHost, m->stream));
     HIP_TRY(hipMemcpyAsync(m->pin + 48, m->adv, 4, hipMemcpyDeviceToHost, m->stream));
+    HIP_TRY(hipMemcpyAsync(m->pin + 56, m->ctl, sizeof(StepCtl), hipMemcpyDeviceToHost, m->stream));
     HIP_TRY(hipStreamSynchronize(m->stream));
+    if ((rc = step_err("forward_spec", m->pin[58]))) return rc;
     memcpy(out, m->pin + 32, (size_t)rows * 4);
     *adv = m->pin[48];
     m->last_rows = rows; m->last_adv = *adv;
@@ -1434,7 +1518,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f");
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -1456,6 +1540,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     StepCtl c;
     HIP_TRY(hipMemcpy(&c, t->ctl, sizeof c, hipMemcpyDeviceToHost));
     if (c.step != n_rounds) return fail(-9, "mtp_rounds: %d of %d rounds ran", c.step, n_rounds);
+    { const int erc = step_err("mtp_rounds", c.err); if (erc) return erc; }
     HIP_TRY(hipMemcpy(blocks, t->sched, (size_t)n_rounds * rows * 4, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(out, t->out, (size_t)n_rounds * rows * 4, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(adv, t->adv, (size_t)n_rounds * 4, hipMemcpyDeviceToHost));
@@ -1488,6 +1573,15 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
         done += rows;
     }
     return 0;
+}
+
+extern "C" int lg_hip_tail_stamps(lg_hip_model *m, unsigned long long *dst, int cap) {
+    if (!m || !dst || !m->tstamps) return fail(-1, "tail_stamps: the model has no one-XCD tail");
+    if (cap < LG_XTAIL_UNITS * 8) return fail(-2, "tail_stamps: room for %d values needed", LG_XTAIL_UNITS * 8);
+    HIP_TRY(hipSetDevice(m->device));
+    HIP_TRY(hipStreamSynchronize(m->stream));
+    HIP_TRY(hipMemcpy(dst, m->tstamps, (size_t)LG_XTAIL_UNITS * 8 * 8, hipMemcpyDeviceToHost));
+    return LG_XTAIL_UNITS;
 }
 
 extern "C" int lg_hip_get_hidden(lg_hip_model *m, float *dst) {
@@ -1546,6 +1640,7 @@ extern "C" int lg_hip_schedule_wait(lg_hip_model *m, int32_t *out, int32_t *adv,
     HIP_TRY(hipStreamSynchronize(m->stream));
     StepCtl c;
     HIP_TRY(hipMemcpy(&c, m->ctl, sizeof c, hipMemcpyDeviceToHost));
+    { const int erc = step_err("schedule_wait", c.err); if (erc) return erc; }
     // the step counter is device state: never copy more than the schedule that was loaded holds
     if (c.step < 0 || c.step > m->sched_loaded)
         return fail(-6, "schedule_wait: the device reports %d steps done, %d were loaded", c.step, m->sched_loaded);
@@ -1583,7 +1678,8 @@ static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int
         b[KC_O] += (double)y.qd * m->E * q;
         if (m->xffn_built && m->xcd_ffn && rows >= 4) b[KC_FFN] += 3.0 * m->E * y.nff * q;
         else { b[KC_GATEUP] += 2.0 * m->E * y.nff * q; b[KC_DOWN] += (double)y.nff * m->E * q; }
-        if (m->ple) { const double pq = y.winp_f ? 4.0 : q; b[KC_PLEGATE] += (double)m->E * m->ple * pq; b[KC_PLEPROJ] += (double)m->ple * m->E * pq; }
+        if (m->ple && !y.winp_f && use_ple_tail(m, rows)) b[KC_TAIL] += 2.0 * m->E * m->ple * q;
+        else if (m->ple) { const double pq = y.winp_f ? 4.0 : q; b[KC_PLEGATE] += (double)m->E * m->ple * pq; b[KC_PLEPROJ] += (double)m->ple * m->E * pq; }
         const int window = (y.is_local && m->window > 0) ? m->window : 0;
         const int last = pos + rows - 1, start = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
         b[KC_ATTN] += 2.0 * (last - start + 1) * y.kd * 2.0;          // K and V rows, f16

@@ -729,16 +729,17 @@ struct RowsPleGateArgs {
     int            dparts;              // 8: dout is eight [M][E] slabs of partial sums (one per XCD), added here in tree order; else 1
 };
 #define LG_RPG_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const uint8_t *, gw, g.w, v) X(int, gk, g.k, v) X(int, gple, g.ple, v) X(int, dparts, dparts, v) X(const float *, gipl, g.ipl, v) X(int, glayer, g.layer, v) X(int, gnl, g.n_layer, v) X(int8_t *, gpq, g.pq, v) X(const int8_t *, gq_in, g.q_in, v) X(float *, x_out, x_out, v) X(float, eps, eps, v)
-template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, _) int p_end_) {
-    RowsPleGateArgs a; LG_RPG_FIELDS(LG_XI, a)
-    extern __shared__ __align__(16) unsigned char smem[];
+// The body for gate block gb and draft row j (a device function: the kernel below runs it per workgroup of its grid,
+// lg_k_ple_tail as the first phase of a longer kernel).  xnew receives the lane's float4s of the updated residual;
+// after_requests runs once every load of the body has been requested (a caller's own loads go there: loads return
+// in the order they were requested, and the row's must not wait behind them).
+template <int M, typename Hook>
+__device__ __forceinline__ void lg_rows_plegate_body(const RowsPleGateArgs &a, int gb, int j, unsigned char *smem, float *gbuf, float *red,
+                                                     float4 (&xnew)[LG_ROWV], bool write_x, Hook &&after_requests) {
     int8_t *lq = (int8_t *)smem;                              // one row: [E] int8, then [E/32] {scale, sum}
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.g.k, nit = E >> 8, ple = a.g.ple;
     float2 *lds = (float2 *)(smem + (size_t)E);
-    __shared__ float gbuf[32], red[4];
-    const int j = blockIdx.y;
-    const uint8_t *wg[1] = { a.g.w + (size_t)(blockIdx.x * 4 + wave) * nit * LG_TILE };
+    const uint8_t *wg[1] = { a.g.w + (size_t)(gb * 4 + wave) * nit * LG_TILE };
     // Every load of the kernel is requested up front, the row's first (loads return in order: the row work then starts
     // while the tiles are still arriving), then the whole row group (nit <= 16 tiles: with this few workgroups the
     // kernel is a chain of memory round trips, and fetching the tiles two at a time adds one per pair), then the
@@ -769,7 +770,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, 
         wq[u] = *(const uint4 *)(wg[0] + (size_t)it * LG_TILE + lane * 16);
         wsc[u] = *(const uint16_t *)(wg[0] + (size_t)it * LG_TILE + 1024 + lane * 2);
     }
-    const float iplv = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + blockIdx.x * 32 + wave * 8 + (lane >> 3)];   // of this lane's gate column
+    const float iplv = a.g.ipl[(size_t)j * a.g.n_layer * ple + (size_t)a.g.layer * ple + gb * 32 + wave * 8 + (lane >> 3)];   // of this lane's gate column
+    after_requests();
     {
         float ss = 0.0f;
         #pragma unroll
@@ -783,7 +785,8 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, 
                 float4 x = xv[v];
                 x.x = x.x + d.x * sc * w.x;  x.y = x.y + d.y * sc * w.y;
                 x.z = x.z + d.z * sc * w.z;  x.w = x.w + d.w * sc * w.w;
-                if (blockIdx.x == 0) ((float4 *)(a.x_out + (size_t)j * E))[t + 256 * v] = x;
+                if (write_x) ((float4 *)(a.x_out + (size_t)j * E))[t + 256 * v] = x;
+                xnew[v] = x;
                 float dq; int sum;
                 const uint32_t packed = lg_quant4_8lanes(x, &dq, &sum);
                 const int quad = t + 256 * v;
@@ -814,9 +817,17 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, 
         float d; int sum;
         const int q = lg_quant1_32lanes(gbuf[i], &d, &sum);
         const ActLayout lay = lg_act_layout(ple);
-        a.g.pq[(size_t)j * ple + lg_act_unit(lay, blockIdx.x * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
-        if (i == 0) lg_q8_ds<M>(a.g.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, blockIdx.x)] = make_float2(d, __int_as_float(sum));
+        a.g.pq[(size_t)j * ple + lg_act_unit(lay, gb * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
+        if (i == 0) lg_q8_ds<M>(a.g.pq, ple)[(size_t)j * (ple >> 5) + lg_act_block(lay, gb)] = make_float2(d, __int_as_float(sum));
     }
+}
+template <int M>
+__global__ __launch_bounds__(LG_WG) void lg_k_rows_plegate(LG_RPG_FIELDS(LG_XP, _) int p_end_) {
+    RowsPleGateArgs a; LG_RPG_FIELDS(LG_XI, a)
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float gbuf[32], red[4];
+    float4 xnew[LG_ROWV];
+    lg_rows_plegate_body<M>(a, (int)blockIdx.x, (int)blockIdx.y, smem, gbuf, red, xnew, blockIdx.x == 0, [] {});
 }
 
 // lm_head: each workgroup walks `passes` blocks of 64 vocabulary rows (4 wavefronts x 2 groups

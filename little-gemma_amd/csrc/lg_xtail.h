@@ -1,0 +1,213 @@
+// lg_xtail.h — the narrow end of a layer as ONE launch that runs on ONE XCD (verify blocks, models with per-layer inputs).
+//
+// After ffn_down a layer with per-layer inputs still has three dependent steps, each of them a handful of workgroups
+// and a kernel of its own when launched separately:
+//   1  rows + PLE gate   x += rmsnorm(ffn_down) * w ; q8(x) ; gelu(inp_gate . q8(x)) * per-layer input ; q8    (ple/32 x M workgroups)
+//   2  PLE projection    proj . that q8 row: [E] outputs of K = ple                                              (E x ple weights: 0.37 MB)
+//   3  rows              x = (x + rmsnorm(2) * w) * out_scale ; q8(rmsnorm(x) * next norm weight)               (M rows)
+// None of them can use the chip: what they cost is a kernel boundary each (the gap to the predecessor's end plus the
+// first trip of the predecessor's data through the memory-side cache).  The workgroups of one XCD share an L2, and a
+// hand-over through it costs a fraction of a boundary (lg_xcd.h).  So the three run as the phases of one kernel on the
+// U = ple/32 x M workgroups i of the launch with i % 8 == 0 (the dispatcher deals workgroups to the XCDs in turn: one
+// XCD gets them all; the other 7U workgroups of the launch leave at once):
+//   phase 1 is lg_k_rows_plegate's body for unit (gate block, row); the unit keeps the updated residual row in registers;
+//   hand-over (the M x ple q8 values: 1.6 KB) ;
+//   phase 2: the E/8 row groups of the projection dealt over the 4U wavefronts, weights requested at kernel start
+//   (they depend on nothing and are in registers long before the hand-over);
+//   hand-over (the [M][E] f32 outputs) ;
+//   phase 3: lg_k_rows' work for row j, by the units (v, j) of the row's first E/1024 gate blocks: each forms the row's
+//   sums and stores and quantizes the float4s t + 256 v of every lane (the slices of lg_k_rows).
+// Sums and quantization are the ones of the separate kernels, lane for lane: the results are bit-identical.
+// The flags carry the writer's XCD id; a unit that sees another id, or gives up a bounded wait, reports it in
+// StepCtl.err and goes on, so the kernel always ends and the host refuses the step.
+#pragma once
+#include "lg_kernels.h"
+#include "lg_xcd.h"
+#include "lg_xffn.h"
+
+#define LG_XTAIL_UNITS 64           // most units of a launch (lane i of a wavefront polls flag i)
+struct XtailSync {
+    uint32_t gen;                   // launches so far (advanced by unit 0 at the end of a launch); epochs 2 gen + 1, + 2
+    uint32_t pad[31];
+    uint32_t flags[2][LG_XTAIL_UNITS];
+};
+
+struct XtailArgs {
+    RowsPleGateArgs r;              // phase 1 (x_out is not written: the row stays in registers)
+    const uint8_t *pw;              // phase 2: tiled projection weights [E][ple]
+    float         *pout;            // [M][E] its output (the XCD's L2 hands it from phase 2 to phase 3)
+    const float   *w_post2, *os;    // phase 3: norm weight for pout, layer output scale (or nullptr)
+    const float   *w_pre;           // norm weight applied before quantization
+    float         *x_out, *h_out;   // [M][E] new residual; normed rows before quantization, or nullptr
+    int8_t        *q;               // q8 activation buffer of the result
+    int            q_units;         // 0: rows in the order of lg_act_layout; 2: the 80-dword blocks of lg_k_geglu_m
+    XtailSync     *sync;
+    int            spin_limit;
+    unsigned long long *stamps;     // nullptr, or [LG_XTAIL_UNITS][8] device wall-clock ticks at the phase boundaries of every unit (measurement runs)
+};
+#define LG_XTAIL_FIELDS(X, v) X(const float *, x, r.x, v) X(const float *, dout, r.dout, v) X(const float *, w_post, r.w_post, v) X(const uint8_t *, gw, r.g.w, v) \
+    X(int, gk, r.g.k, v) X(int, gple, r.g.ple, v) X(int, dparts, r.dparts, v) X(XtailSync *, sync, sync, v) X(const float *, gipl, r.g.ipl, v) X(int, glayer, r.g.layer, v) \
+    X(int, gnl, r.g.n_layer, v) X(int8_t *, gpq, r.g.pq, v) X(const uint8_t *, pw, pw, v) X(const float *, w_post2, w_post2, v) X(const float *, w_pre, w_pre, v) \
+    X(const float *, os, os, v) X(float *, pout, pout, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) \
+    X(float, eps, r.eps, v) X(int, spin_limit, spin_limit, v) X(unsigned long long *, stamps, stamps, v)
+
+__device__ __forceinline__ void lg_ld4_wait1(lg_x4u &a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a) :: "memory"); }
+
+// G: most projection row groups per wavefront (E/8 groups over 4U wavefronts).
+template <int M, int G>
+__global__ __launch_bounds__(LG_WG) void lg_k_ple_tail(StepCtl *ctl, LG_XTAIL_FIELDS(LG_XP, _) int p_end_) {
+    if (blockIdx.x & (LG_XCDS - 1)) return;
+    XtailArgs a; LG_XTAIL_FIELDS(LG_XI, a)
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float gbuf[32], red[3][4];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int E = a.r.g.k, ple = a.r.g.ple, nblk = ple >> 5, U = nblk * M, nq = E >> 2;
+    const int u = blockIdx.x >> 3, gb = u % nblk, j = u / nblk;
+    const uint32_t gen = a.sync->gen;
+    auto stamp = [&](int i) { if (a.stamps && t == 0) a.stamps[(size_t)u * 8 + i] = wall_clock64(); };
+    stamp(0);
+    const int xcc = lg_xcc_id();
+    // ---- phase 1, with this kernel's later loads requested behind its own ----
+    const int groups = E >> 3, waves = 4 * U, gw = u * 4 + wave;
+    const uint8_t *wgp[G];
+    int row[G];
+    bool live[G];
+    #pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int gi = gw + g * waves;
+        live[g] = gi < groups;
+        const int gc = live[g] ? gi : groups - 1;
+        wgp[g] = a.pw + (size_t)gc * LG_TILE;                  // K = ple = 256: one tile per group of 8 rows
+        row[g] = gc * 8 + (lane >> 3);
+    }
+    WChunk<G, 1> pwt;
+    float4 wpost2[LG_ROWV], wpre[LG_ROWV];
+    float osv = 1.0f;
+    float4 xv[LG_ROWV];
+    lg_rows_plegate_body<M>(a.r, gb, j, smem, gbuf, red[0], xv, false, [&] {
+        lg_mm_fetch<G, 1>(pwt, wgp, 0, 1, lane);
+        const float4 *w2 = (const float4 *)a.w_post2, *w3 = (const float4 *)a.w_pre;
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { wpost2[v] = w2[t + 256 * v]; wpre[v] = w3[t + 256 * v]; }
+        if (a.os) osv = a.os[0];
+    });
+    stamp(1);
+    // ---- hand-over: every unit's 32 gated values of its row are in the XCD's L2 ----
+    int8_t *lq2 = (int8_t *)(smem + (size_t)E * 5 / 4);       // [M][ple] int8, [M][ple/32] {scale, sum}
+    lg_wait_vm();
+    __syncthreads();
+    if (wave == 0) {
+        const int err = lg_xcd_arrive_wait(a.sync->flags[0], u, true, U, 2 * gen + 1, xcc, a.spin_limit);
+        if (err && lane == 0) atomicOr(&ctl->err, err);
+    }
+    __syncthreads();
+    stamp(2);
+    {
+        const int n16 = M * ple * 5 / 64;                      // 16-byte units of the q8 rows
+        for (int i = t; i < n16; i += LG_WG) {
+            lg_x4u v = lg_ld4_sc_issue<2>(a.r.g.pq + (size_t)i * 16);
+            lg_ld4_wait1(v);
+            *(lg_x4u *)(lq2 + (size_t)i * 16) = v;
+        }
+    }
+    __syncthreads();
+    stamp(3);
+    // ---- phase 2: this wavefront's row groups of the projection ----
+    {
+        float acc[G][M];
+        lg_mm_groups<M, 8, G, false, 1>(wgp, pwt, 1, lq2, lg_q8_ds<M>(lq2, ple), ple, acc, lane, nullptr, E, row);
+        const int c = lane & 7;
+        if (c < M) {
+            #pragma unroll
+            for (int g = 0; g < G; ++g) if (live[g]) a.pout[(size_t)c * E + row[g]] = lg_pick<M>(acc[g], c);
+        }
+    }
+    // ---- hand-over: the projection's [M][E] is in the XCD's L2 ----
+    const int slices = (E + 1023) >> 10;
+    stamp(4);
+    lg_wait_vm();
+    __syncthreads();
+    if (gb >= slices) {                                        // this unit has no share of the row work: it arrives and leaves
+        if (t == 0) lg_st_sc<0>(a.sync->flags[1] + u, ((2 * gen + 2) << 4) | (uint32_t)xcc);
+        return;
+    }
+    if (wave == 0) {
+        const int err = lg_xcd_arrive_wait(a.sync->flags[1], u, true, U, 2 * gen + 2, xcc, a.spin_limit);
+        if (err && lane == 0) atomicOr(&ctl->err, err);
+    }
+    __syncthreads();
+    stamp(5);
+    // ---- phase 3: the row work of row j, this unit storing and quantizing slice gb ----
+    float4 dv[LG_ROWV];
+    {
+        lg_x4u d0 = lg_x4u{ 0, 0, 0, 0 }, d1 = d0, d2 = d0, d3 = d0;
+        const float *pr = a.pout + (size_t)j * E;
+        const int last = nq - 1;
+        d0 = lg_ld4_sc_issue<2>(pr + 4 * min(t, last));
+        d1 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 256, last));
+        d2 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 512, last));
+        d3 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 768, last));
+        lg_ld4_wait(d0, d1, d2, d3);
+        const lg_x4u d[4] = { d0, d1, d2, d3 };
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) dv[v] = make_float4(__uint_as_float(d[v].x), __uint_as_float(d[v].y), __uint_as_float(d[v].z), __uint_as_float(d[v].w));
+    }
+    stamp(6);
+    {
+        float ss = 0.0f;
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
+        ss = lg_block_sum256(ss, red[1]);
+        const float sc = 1.0f / sqrtf(ss / (float)E + a.r.eps);
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+            const float4 w = wpost2[v];
+            float4 r;
+            r.x = xv[v].x + dv[v].x * sc * w.x;  r.y = xv[v].y + dv[v].y * sc * w.y;
+            r.z = xv[v].z + dv[v].z * sc * w.z;  r.w = xv[v].w + dv[v].w * sc * w.w;
+            if (a.os) { r.x = r.x * osv; r.y = r.y * osv; r.z = r.z * osv; r.w = r.w * osv; }
+            xv[v] = r;
+        }
+    }
+    {
+        float4 *xo = (float4 *)(a.x_out + (size_t)j * E);
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq && v == gb) xo[t + 256 * v] = xv[v];
+    }
+    {
+        float ss = 0.0f;
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(xv[v], ss);
+        ss = lg_block_sum256(ss, red[2]);
+        const float sc = 1.0f / sqrtf(ss / (float)E + a.r.eps);
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+            const float4 w = wpre[v];
+            xv[v] = make_float4(xv[v].x * sc * w.x, xv[v].y * sc * w.y, xv[v].z * sc * w.z, xv[v].w * sc * w.w);
+        }
+    }
+    if (a.h_out) {
+        float4 *ho = (float4 *)(a.h_out + (size_t)j * E);
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq && v == gb) ho[t + 256 * v] = xv[v];
+    }
+    float2 *dsb = lg_q8_ds<M>(a.q, E);
+    #pragma unroll
+    for (int v = 0; v < LG_ROWV; ++v) {
+        if (t + 256 * v >= nq || v != gb) continue;
+        float d; int sum;
+        const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
+        const int quad = t + 256 * v;
+        if (a.q_units == 2) {
+            uint32_t *blk = (uint32_t *)a.q + (size_t)(quad >> 3) * LG_MU_DWORDS;
+            const int dw = quad & 7;
+            blk[j * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))] = packed;
+            if ((t & 7) == 0) *(float2 *)(blk + 64 + 2 * j) = make_float2(d, 12582912.0f + (float)(8 * sum));
+        } else {
+            *(uint32_t *)(a.q + lg_q8_off<M>(E, j, quad >> 2, (quad & 3) * 4)) = packed;
+            if ((t & 7) == 0) dsb[lg_q8_ds_idx<M>(E, j, quad >> 3)] = make_float2(d, __int_as_float(sum));
+        }
+    }
+    stamp(7);
+    if (u == 0 && t == 0) a.sync->gen = gen + 1;
+}

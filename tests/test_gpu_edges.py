@@ -166,7 +166,8 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, r
 
     base = run()
     for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
-                     ("fork_ple", 1)):       # (the per-layer inputs as a second branch of the graph: off by default)
+                     ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
+                     ("xcd_tail", 0), ("xcd_tail", 2)):   # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
         print(f"rows={rows} option {opt}={val}", flush=True)
         got = run(**{opt: val})
         assert got[0] == base[0] and np.array_equal(got[1], base[1]), opt
