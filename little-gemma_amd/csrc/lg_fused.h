@@ -946,3 +946,68 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge_split(const StepCtl *ct
     if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));
     if (a.xf) a.xf[(size_t)j * qd + e] = r;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Attention merge + output projection in one launch, with no hand-over between workgroups.
+// With 8 query heads the 8 K segments of the output projection ARE the heads (K = n_head * head_dim, a segment =
+// head_dim elements): the serial chain of segment c only reads head c of the attention output, and the row's result is
+// the adjacent-pair tree over the 8 chains.  So the workgroup that merges (head, row j) can run that head's chain
+// for a slice of the E output rows straight from LDS, and slab `head` of 8 receives the chain sums: the consumer (the
+// row kernel, dparts = 8) adds the slabs in the tree's order, bit for bit what lg_k_mm computes from the q8 row.
+// Unit = (row j, head, slice s of the output rows in chunks of 64); the merge is repeated by the slices of a (head, row),
+// which costs less than the kernel boundary it replaces.  Workgroup id = j * (8 * slices) + head * slices + s: the units
+// that read the same weights differ by a multiple of 8 and run on one XCD (one trip from HBM, the others hit its L2).
+// Weights: the projection tiled by row blocks (tile (64-row chunk, K block): lane r = row 64 * chunk + r), where the
+// tiles of a head are consecutive.  Lane r of wavefront w runs the chains of the rows r of the unit's chunks w, w + 4, ...
+// NIT = head_dim / 32 blocks per chain; RPL = most chunks per wavefront.
+struct MergeOArgs {
+    MergeArgs      g;           // g.xq unused; g.xf optional
+    const uint8_t *w;           // row-block tiles of attn_output [E][n_head * head_dim]
+    float         *slabs;       // [8][M][E]
+    int            E, slices, rows;
+};
+#define LG_MERGEO_FIELDS(X, v) X(const float *, pm, g.pm, v) X(const float *, pl, g.pl, v) X(const float *, pacc, g.pacc, v) X(int, tiles_max, g.tiles_max, v) \
+    X(int, H, g.H, v) X(int, hd, g.hd, v) X(int, window, g.window, v) X(int, pos_off, g.pos_off, v) X(const uint8_t *, w, w, v) X(int, E, E, v) X(int, slices, slices, v) \
+    X(int, rows, rows, v) X(float *, slabs, slabs, v) X(float *, xf, g.xf, v)
+template <int NIT, int RPL>
+__global__ __launch_bounds__(LG_WG) void lg_k_merge_o(const StepCtl *ctl, LG_MERGEO_FIELDS(LG_XP, _) int p_end_) {
+    MergeOArgs a; LG_MERGEO_FIELDS(LG_XI, a)
+    a.g.xq = nullptr;
+    __shared__ float wts[512], pls[512], wmx[LG_WG / 64];
+    __shared__ __align__(16) int8_t hq[NIT * 32];             // the merged head as q8, natural order
+    __shared__ float2 hds[NIT];
+    const int W = a.g.H * a.slices, id = blockIdx.x;
+    const int j = id / W, wi = id - j * W, head = wi / a.slices, s = wi - head * a.slices;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = a.g.H * NIT, n64 = (a.E >> 6) / a.slices, chunk0 = s * n64;
+    uint4 wq[RPL][NIT];
+    uint16_t wsc[RPL][NIT];
+    const int qd = a.g.H * a.g.hd;
+    lg_attn_merge_body(ctl, a.g, head, j, wts, pls, wmx, [&] {
+        #pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int c = wave + 4 * r < n64 ? wave + 4 * r : n64 - 1;     // past the unit's chunks: its last one again, unused
+            const uint8_t *tb = a.w + ((size_t)(chunk0 + c) * nb + (size_t)head * NIT) * LG_TILE;
+            #pragma unroll
+            for (int it = 0; it < NIT; ++it) { wq[r][it] = lg_ldt16(tb, it, lane); wsc[r][it] = lg_ldt2(tb, it, lane); }
+        }
+    }, [&](int d, float r, int q, float dq, int sum) {
+        hq[d] = (int8_t)q;
+        if ((d & 31) == 0) hds[d >> 5] = make_float2(dq, __int_as_float(sum));
+        if (a.g.xf && s == 0) a.g.xf[(size_t)j * qd + head * a.g.hd + d] = r;
+    });
+    __syncthreads();
+    #pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+        if (wave + 4 * r >= n64) break;
+        float acc = 0.0f;
+        #pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const float2 ds = hds[it];
+            const int4 a0 = *(const int4 *)(hq + it * 32), a1 = *(const int4 *)(hq + it * 32 + 16);
+            const int dot = lg_block_dot(wq[r][it], a0, a1, __float_as_int(ds.y));
+            acc = lg_fmaf(ds.x * lg_h2f(wsc[r][it]), (float)dot, acc);
+        }
+        a.slabs[((size_t)head * a.rows + j) * a.E + (size_t)(chunk0 + wave + 4 * r) * 64 + lane] = acc;
+    }
+}

@@ -147,6 +147,7 @@ struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; }
 struct Layer {
     uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
     float *winp_f = nullptr, *wproj_f = nullptr;   // inp_gate / proj when the file keeps them in a float type (then winp / wproj are null)
+    uint8_t *wo_rb = nullptr;                      // attn_output again as row-block tiles: the chains of lg_k_merge_o
     uint8_t *xgu = nullptr, *xdn = nullptr;        // gate/up and ffn_down again as per-workgroup streams of the XCD-partitioned kernel (lg_xffn.h)
     float *attn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *post_attn = nullptr, *ffn_norm = nullptr,
           *post_ffw = nullptr, *post_norm = nullptr, *out_scale = nullptr;
@@ -205,6 +206,10 @@ struct lg_hip_model {
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
+    int merge_o = 0;                         // option: attention merge and output projection as one launch (lg_k_merge_o): 0 off (as measured it loses
+                                             // as much in the row kernel that adds its 8 slabs as it gains), 1 from three rows up, 2 always; the second
+                                             // copy of the weights it reads is only built when LG_HIP_MERGE_O is set at commit
+    int merge_o_slices = 0;                  // option: slices of the output rows per (head, row), 0 = chosen by the launcher
     // the per-layer-input block and the next row work as one launch on one XCD (lg_xtail.h)
     int xcd_tail = 1;                        // option: 0 off, 1 for blocks that do not fold the row work into q/k/v, 2 for every verify block
     XtailSync *tsync = nullptr;
@@ -551,6 +556,9 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if ((rc = check_mat(o, lname(L, "attn_output.weight"), y.qd, E))) return rc;
         push_rows(rows, o, 0, E);
         if ((rc = upload_tiled(m, rows, y.qd, &y.wo, stage))) return rc;
+        // (8 query heads: the K segments of this projection are the heads, and the merge can run their chains itself)
+        if (getenv("LG_HIP_MERGE_O") && atoi(getenv("LG_HIP_MERGE_O")) > 0 && !m->target && m->H == 8 && lg_segments(y.qd) == 8 && E % 64 == 0 && y.hd % 32 == 0 && y.hd <= 512 &&
+            (rc = upload_tiled(m, rows, y.qd, &y.wo_rb, stage, true))) return rc;
         rows.clear();
         const HostTensor *g = find(m, lname(L, "ffn_gate.weight")), *u = find(m, lname(L, "ffn_up.weight")),
                          *d = find(m, lname(L, "ffn_down.weight"));
@@ -639,6 +647,8 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         HIP_TRY(hipMemset(m->tsync, 0, sizeof(XtailSync)));
         if (getenv("LG_HIP_XCD_TAIL")) m->xcd_tail = atoi(getenv("LG_HIP_XCD_TAIL"));
     }
+    if (getenv("LG_HIP_MERGE_O")) m->merge_o = atoi(getenv("LG_HIP_MERGE_O"));
+    if (getenv("LG_HIP_MERGE_O_SLICES")) m->merge_o_slices = atoi(getenv("LG_HIP_MERGE_O_SLICES"));
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
         return -7;
     if (xffn) {
@@ -1005,8 +1015,37 @@ static bool use_ple_tail(const lg_hip_model *m, int rows) {
     if (!m->ple || !m->tsync || m->xcd_tail <= 0 || m->target || rows < 1 || rows > LG_HIP_MAX_ROWS) return false;
     if (m->ple != 256 || (m->ple / 32) * rows > LG_XTAIL_UNITS || m->E % 256 || m->E > 4096 || (m->E + 1023) / 1024 > m->ple / 32) return false;
     if (m->xcd_tail == 1 && rows <= LG_FUSE_ROWS_MAX && m->fuse_rows) return false;
+    const int U = (m->ple / 32) * rows;
+    if ((m->E / 8 + 4 * U - 1) / (4 * U) > 4) return false;       // (few rows of a wide model: too few wavefronts for the projection)
     return cu_count() == LG_XCDS * LG_XCD_WGS;
 }
+// Slices of the E output rows per (head, row) of lg_k_merge_o: a divisor of the E/64 chunks that leaves at most two
+// chunks per wavefront, the largest that keeps the launch within one workgroup per CU (else the smallest)
+static int merge_o_slices(const lg_hip_model *m, int rows) {
+    const int chunks = m->E / 64;
+    int best = 0, least = 0;
+    for (int d = 1; d <= chunks; ++d) {
+        if (chunks % d || (chunks / d + 3) / 4 > 2) continue;
+        if (!least) least = d;
+        if (8 * rows * d <= cu_count()) best = d;
+    }
+    const int pick = best ? best : least;
+    if (m->merge_o_slices > 0 && chunks % m->merge_o_slices == 0 && (chunks / m->merge_o_slices + 3) / 4 <= 2) return m->merge_o_slices;
+    return pick;
+}
+static bool use_merge_o(const lg_hip_model *m, const Layer &y, int rows, int tiles) {
+    if (!y.wo_rb || m->merge_o <= 0 || rows > LG_HIP_MAX_ROWS || (m->merge_o == 1 && rows < 3)) return false;
+    return tiles < 128 && merge_o_slices(m, rows) > 0;
+}
+static void launch_merge_o(Launcher &lx, const MergeOArgs &a) {
+    const int nit = a.g.hd / 32, rpl = ((a.E / 64) / a.slices + 3) / 4;
+    const dim3 grid(a.rows * a.g.H * a.slices);
+#define CASE(N, R) if (nit == N && rpl == R) { LAUNCH(KC_MERGE, (lg_k_merge_o<N, R>), grid, dim3(LG_WG), 0, lx.m->ctl, LG_MERGEO_FIELDS(LG_XA, a) 0); return; }
+    CASE(2, 1) CASE(2, 2) CASE(4, 1) CASE(4, 2) CASE(8, 1) CASE(8, 2) CASE(16, 1) CASE(16, 2)
+#undef CASE
+    lx.rc = fail(-2, "merge_o: no instantiation for head_dim %d with %d chunks per wavefront", a.g.hd, rpl);
+}
+
 template <int M>
 static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
     if constexpr (M <= LG_HIP_MAX_ROWS) {
@@ -1167,7 +1206,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
-        bool fused_post = false;
+        bool fused_post = false, merged_o = false;
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
             if (rows_done) { launch_mm<M, false>(lx, KC_QKV, a); rows_done = false; }      // (the previous layer's tail did this layer's row work)
@@ -1225,10 +1264,17 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 LAUNCH(KC_ATTN, (lg_k_attn<false, 1>), dim3(tiles, y.nkv, M), dim3(LG_WG), attn_lds(G, y.hd, false), m->ctl, LG_ATTN_FIELDS(LG_XA, a) 0);
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
+            merged_o = pos_off == 0 && use_merge_o(m, y, M, tiles);
+            if (merged_o) {
+                // the merge of (head, row) runs that head's chain of the output projection itself: eight slabs for the row kernel
+                MergeOArgs f{ g, y.wo_rb, m->dout, E, merge_o_slices(m, M), M };
+                launch_merge_o(lx, f);
+                pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr; pend_parts = 8;
+            } else
             if (M <= LG_HIP_MAX_ROWS && tiles >= 128 && y.hd % 64 == 0) LAUNCH(KC_MERGE, (lg_k_attn_merge_split<M>), dim3(H, M, y.hd / 64), dim3(LG_WG), 0, m->ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
             else LAUNCH(KC_MERGE, (lg_k_attn_merge<M>), dim3(H, M), dim3(LG_WG), 0, m->ctl, LG_MERGE_FIELDS(LG_XA, g) 0);
         }
-        {   // attention output projection
+        if (!merged_o) {   // attention output projection
             MmArgs a{ y.wo, y.qd, E, m->dout, m->aq, nullptr };
             pend_parts = launch_mm<M, false>(lx, KC_O, a);      // (four slabs for a wide block when n_head * head_dim > 4096)
             pend_dout = m->dout; pend_w = y.post_attn; pend_os = nullptr;
@@ -1350,7 +1396,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "");
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1390,6 +1436,8 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
+    else if (!strcmp(name, "merge_o")) m->merge_o = value < 0 ? 0 : value > 2 ? 2 : value;
+    else if (!strcmp(name, "merge_o_slices")) m->merge_o_slices = value < 0 ? 0 : value;
     else if (!strcmp(name, "xcd_tail")) m->xcd_tail = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "xcd_tail_stamps")) m->tail_stamps = value != 0;
     else if (!strcmp(name, "xcd_ffn_delay")) m->xffn_delay = value < 0 ? 0 : value > 0x3FF ? 0x3FF : value;
@@ -1518,7 +1566,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -1675,7 +1723,11 @@ static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int
     for (int L = 0; L < m->n_layer; ++L) {
         const Layer &y = m->L[L];
         b[KC_QKV] += (double)m->E * y.qkv_m * q;
-        b[KC_O] += (double)y.qd * m->E * q;
+        {
+            const int w = (y.is_local && m->window > 0) ? m->window : 0, st = (w > 0 && pos - w + 1 > 0) ? pos - w + 1 : 0;
+            const int tiles = ((pos + rows - 1) >> 5) - (st >> 5) + 1;
+            b[use_merge_o(m, y, rows, tiles) ? KC_MERGE : KC_O] += (double)y.qd * m->E * q;
+        }
         if (m->xffn_built && m->xcd_ffn && rows >= 4) b[KC_FFN] += 3.0 * m->E * y.nff * q;
         else { b[KC_GATEUP] += 2.0 * m->E * y.nff * q; b[KC_DOWN] += (double)y.nff * m->E * q; }
         if (m->ple && !y.winp_f && use_ple_tail(m, rows)) b[KC_TAIL] += 2.0 * m->E * m->ple * q;

@@ -1398,11 +1398,14 @@ struct MergeArgs {
     float *xf;                 // optional f32 copy [M][H*hd]
 };
 #define LG_MERGE_FIELDS(X, v) X(const float *, pm, pm, v) X(const float *, pl, pl, v) X(const float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(int, H, H, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int8_t *, xq, xq, v) X(float *, xf, xf, v)
-template <int M>
-__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_MERGE_FIELDS(LG_XP, _) int p_end_) {
-    MergeArgs a; LG_MERGE_FIELDS(LG_XI, a)
-    __shared__ float wts[512], pls[512];                      // exp(m_tile - M) and the sums of up to 512 tiles at a time
-    const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
+// The body for (head, row j) as a device function (the kernel below runs it per workgroup of its grid, lg_k_merge_o as
+// its first phase).  wts, pls: 512 floats of LDS each (exp(m_tile - M) and the sums of up to 512 tiles at a time), wmx: 4.
+// after_first_fetch runs once the first batch of partials has been requested (a caller's own loads go behind it);
+// sink(d, r, q, dq, sum) receives dim d's result, its q8 value and its block's scale and sum.
+template <typename Hook, typename Sink>
+__device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const MergeArgs &a, int head, int j, float *wts, float *pls, float *wmx,
+                                                   Hook &&after_first_fetch, Sink &&sink) {
+    const int hd = a.hd;
     const int pos = ctl->pos + a.pos_off, pj = pos + j;
     const int first = lg_win_start(pos, a.window) >> 5;
     const int lo = (lg_win_start(pj, a.window) >> 5) - first, hi = (pj >> 5) - first;
@@ -1437,10 +1440,10 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_
         }
     };
     fetch(lo, hi - lo + 1 < 512 ? hi - lo + 1 : 512, 0);
+    after_first_fetch();
     float mx = pm1;
     for (int n = lo + (int)threadIdx.x + LG_WG; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
     mx = lg_max_n(mx, 64);
-    __shared__ float wmx[LG_WG / 64];
     if ((threadIdx.x & 63) == 0) wmx[threadIdx.x >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
@@ -1475,11 +1478,18 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_
         const float r = d < hd ? o[h2] / L : 0.0f;
         float dq; int sum;
         const int q = lg_quant1_32lanes(r, &dq, &sum);
-        if (d < hd) {
-            const int e = head * hd + d;                       // element of the row, natural order
-            a.xq[lg_q8_off<M>(qd, j, e >> 4, e & 15)] = (int8_t)q;      // order the attn_output matmul reads
-            if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));
-            if (a.xf) a.xf[(size_t)j * qd + e] = r;
-        }
+        if (d < hd) sink(d, r, q, dq, sum);
     }
+}
+template <int M>
+__global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_MERGE_FIELDS(LG_XP, _) int p_end_) {
+    MergeArgs a; LG_MERGE_FIELDS(LG_XI, a)
+    __shared__ float wts[512], pls[512], wmx[LG_WG / 64];
+    const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
+    lg_attn_merge_body(ctl, a, head, j, wts, pls, wmx, [] {}, [&](int d, float r, int q, float dq, int sum) {
+        const int e = head * hd + d;                           // element of the row, natural order
+        a.xq[lg_q8_off<M>(qd, j, e >> 4, e & 15)] = (int8_t)q;          // order the attn_output matmul reads
+        if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));
+        if (a.xf) a.xf[(size_t)j * qd + e] = r;
+    });
 }

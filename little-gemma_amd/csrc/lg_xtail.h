@@ -211,3 +211,10 @@ __global__ __launch_bounds__(LG_WG) void lg_k_ple_tail(StepCtl *ctl, LG_XTAIL_FI
     stamp(7);
     if (u == 0 && t == 0) a.sync->gen = gen + 1;
 }
+
+// A second form was built and measured, and is not kept: 32 units of 8 gate rows and 8 wavefronts whatever the block
+// width (so that no CU holds two units from 5 rows up), the row update as a phase of its own ahead of the gate (units
+// (slice, row), q8 rows handed over), the gated rows handed over as floats and quantized by every unit.  Bit-identical,
+// three hand-overs instead of two, and slower at every width: E4B shape, 5 rows 11.2 against 10.6 us per launch (step
+// 2.231 against 2.210 ms), 6 rows 2.326 against 2.303 ms, 8 rows 2.494 against 2.477 ms.  A hand-over costs about 1 us
+// once the wait for the stores and the load of what was handed over are counted, more than the lighter phases save.

@@ -138,12 +138,13 @@ def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
 
 
 @pytest.mark.parametrize("rows,name,over", [(2, "tiny_full", {}), (5, "tiny_full", {}), (6, "tiny", {"n_ff": 5120})])
-def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, rows, name, over):
+def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, monkeypatch, rows, name, over):
     """The options that pick between kernels for the same arithmetic (row work inside the q/k/v matmul, the
     attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay, ffn_down
     cut by K quarter: the last case has the long FFN rows and no per-layer embeddings that kernel is for; the
     per-layer inputs built on a second stream beside layer 0) change
     timing only: every combination leaves the same cache rows and the same logits rows of a verify block."""
+    monkeypatch.setenv("LG_HIP_MERGE_O", "1")          # (builds the second copy of attn_output that the merge_o option needs)
     path, spec = model_path(name, **over)
     V = spec["n_vocab"]
     rng = np.random.default_rng(rows)
@@ -167,7 +168,8 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, r
     base = run()
     for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
                      ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
-                     ("xcd_tail", 0), ("xcd_tail", 2)):   # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
+                     ("xcd_tail", 0), ("xcd_tail", 2),    # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
+                     ("merge_o", 0), ("merge_o", 2), ("merge_o_slices", 8)):   # (attention merge + output projection: separate / one launch for every width / another cut of the rows)
         print(f"rows={rows} option {opt}={val}", flush=True)
         got = run(**{opt: val})
         assert got[0] == base[0] and np.array_equal(got[1], base[1]), opt
