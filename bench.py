@@ -205,6 +205,34 @@ def xcd_handover():
                       "placement": placement, "handover": rows}), flush=True)
 
 
+def tail_stamps(rows, model_dir):
+    """Phase boundaries of the one-XCD layer tail (lg_k_ple_tail) at the E4B shape: device wall-clock stamps of every
+    unit of the last layer's launch, over four verify steps from a 600-position cache."""
+    path = os.path.join(model_dir, f"lg_bench_e4b_seed{lg.synth.E4B['seed']}.gguf")
+    if not os.path.exists(path):
+        lg.synth.write_model(path + ".tmp", **lg.synth.E4B)
+        os.replace(path + ".tmp", path)
+    gpu = lg.hiplib.HipBackend(path, 2400, max_rows=8)
+    gpu.set_option("xcd_tail_stamps", 1)
+    rng = np.random.default_rng(1)
+    gpu.prefill(rng.integers(1, 262144, 600).astype(np.int32), 0)
+    pos, steps = 600, []
+    names = ["start", "rows + per-layer gate done", "hand-over 1 done", "gated rows copied", "projection done", "hand-over 2 done",
+             "projected row loaded", "row work done"]
+    for _ in range(4):
+        adv, _ = gpu.forward_spec(rng.integers(1, 262144, rows).astype(np.int32), pos)
+        pos += adv
+        st = gpu.tail_stamps().astype(np.int64)
+        s = st[st[:, 0] >= st[:, 0].max() - 1000]          # the units of the latest launch (older launches of other widths left theirs: > 10 us back)
+        rel = (s - s[:, 0].min()) * 10                     # ns (100 MHz clock)
+        steps.append({n: {"first_unit_ns": int(rel[:, i][s[:, i] != 0].min()), "last_unit_ns": int(rel[:, i][s[:, i] != 0].max())}
+                      for i, n in enumerate(names)})
+        units = int(s.shape[0])
+    gpu.close()
+    print(json.dumps({"metric": "phase boundaries of lg_k_ple_tail, ns since the first unit's start", "rows": rows, "units": units,
+                      "steps": steps}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -223,7 +251,12 @@ def main():
     ap.add_argument("--xcd-handover", action="store_true",
                     help="measure only where workgroups run (XCD of every workgroup) and what a flag hand-over among the "
                          "workgroups of one XCD costs next to one spread over all XCDs, and exit")
+    ap.add_argument("--tail-stamps", action="store_true",
+                    help="print the phase boundaries of the one-XCD layer tail at --rows rows instead of the benchmark line")
     a = ap.parse_args()
+    if a.tail_stamps:
+        tail_stamps(a.rows, a.model_dir)
+        return
     if a.xcd_handover:
         xcd_handover()
         return
