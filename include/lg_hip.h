@@ -107,9 +107,10 @@ int  lg_hip_get_logits(lg_hip_model *m, int row, float *dst);
  * default 1: 0 sends the whole prompt through verify-width blocks). */
 int  lg_hip_set_option(lg_hip_model *m, const char *name, int value);
 /* Measurement aid (no reference counterpart): with the option "xcd_tail_stamps" on, every unit of the
- * one-XCD launch that ends a layer (lg_k_ple_tail) writes the device wall clock (100 MHz) at its 8 phase
- * boundaries; this copies the stamps of the latest such launch, [64 units][8], and returns 64. */
-int  lg_hip_tail_stamps(lg_hip_model *m, unsigned long long *dst, int cap);
+ * one-XCD launches of a layer writes the device wall clock (100 MHz) at its 8 phase boundaries; this
+ * copies the stamps of the latest such launch, [64 units][8], and returns 64.  which = 0: the launch that
+ * ends the layer (lg_k_ple_tail), 1: the one that ends its attention half (lg_k_attn_tail). */
+int  lg_hip_tail_stamps(lg_hip_model *m, int which, unsigned long long *dst, int cap);
 
 /* ---- draft head: the gemma4-assistant network on the device (mtp_draft_device,
  * mtp_draft_chain_device, mtp_free_device: src/mtp-internal.h:33-37, src/cuda/mtp-kernel.cuh:272-402).

@@ -983,7 +983,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_merge_o(const StepCtl *ctl, LG_MER
     uint4 wq[RPL][NIT];
     uint16_t wsc[RPL][NIT];
     const int qd = a.g.H * a.g.hd;
-    lg_attn_merge_body(ctl, a.g, head, j, wts, pls, wmx, [&] {
+    lg_attn_merge_body(ctl, a.g, head, j, (int)threadIdx.x, wts, pls, wmx, [&] {
         #pragma unroll
         for (int r = 0; r < RPL; ++r) {
             const int c = wave + 4 * r < n64 ? wave + 4 * r : n64 - 1;     // past the unit's chunks: its last one again, unused

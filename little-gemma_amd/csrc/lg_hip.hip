@@ -147,6 +147,7 @@ struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; }
 struct Layer {
     uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
     float *winp_f = nullptr, *wproj_f = nullptr;   // inp_gate / proj when the file keeps them in a float type (then winp / wproj are null)
+    uint8_t *wo_ch = nullptr;                      // attn_output again as matrix-core chains [row block][segment]: lg_k_attn_tail
     uint8_t *wo_rb = nullptr;                      // attn_output again as row-block tiles: the chains of lg_k_merge_o
     uint8_t *xgu = nullptr, *xdn = nullptr;        // gate/up and ffn_down again as per-workgroup streams of the XCD-partitioned kernel (lg_xffn.h)
     float *attn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr, *post_attn = nullptr, *ffn_norm = nullptr,
@@ -156,9 +157,9 @@ struct Layer {
 };
 
 enum KClass { KC_ROWS, KC_PMP, KC_QKV, KC_QKVPOST, KC_ATTN, KC_MERGE, KC_O, KC_GATEUP, KC_DOWN, KC_PLEGATE, KC_PLEPROJ,
-              KC_HEAD, KC_ACCEPT, KC_FFN, KC_TAIL, KC_COUNT };
+              KC_HEAD, KC_ACCEPT, KC_FFN, KC_TAIL, KC_ATAIL, KC_COUNT };
 static const char *k_class_names[KC_COUNT] = { "rows_norm_quant", "ple_model_proj", "qkv", "qkv_post", "attn_tiles", "attn_merge",
-    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept", "ffn_xcd", "ple_tail" };
+    "attn_output", "gate_up_geglu", "ffn_down", "ple_gate", "ple_proj", "lm_head", "accept", "ffn_xcd", "ple_tail", "attn_tail" };
 
 struct Profile {
     bool on = false;
@@ -206,6 +207,9 @@ struct lg_hip_model {
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
+    int xcd_attn_tail = 0;                   // option: attention merge, output projection and the row work after it as one launch on one XCD
+                                             // (lg_k_attn_tail): 0 off (as measured it gains nothing), 1 from three rows up, 2 for every verify block;
+                                             // the copy of the weights it reads is only built when LG_HIP_XCD_ATTN_TAIL is set at commit
     int merge_o = 0;                         // option: attention merge and output projection as one launch (lg_k_merge_o): 0 off (as measured it loses
                                              // as much in the row kernel that adds its 8 slabs as it gains), 1 from three rows up, 2 always; the second
                                              // copy of the weights it reads is only built when LG_HIP_MERGE_O is set at commit
@@ -442,6 +446,31 @@ static void xffn_pack_dn(const uint8_t *down, const XffnGeo &g, uint8_t *dst) {
     });
 }
 
+// attn_output as the chains of lg_k_attn_tail: chain (row block rb of 32 rows, K segment c of 8) = the segment's nit blocks
+// of the 32 rows in the pair layout of the streams above; chains ordered [rb][c], nit * 576 bytes each
+static void pack_o_chains(const uint8_t *const *rows, int k, int m, uint8_t *dst) {
+    const int nit = k / 32 / 8;
+    const size_t cb = (size_t)nit * 576;
+    for (int rb = 0; rb < m / 32; ++rb)
+        for (int c = 0; c < 8; ++c) {
+            uint8_t *ub = dst + ((size_t)rb * 8 + c) * cb;
+            for (int n = 0; n < 32; ++n)
+                for (int it = 0; it < nit; ++it) {
+                    const uint8_t *blk = rows[rb * 32 + n] + (size_t)(c * nit + it) * 18;
+                    for (int h = 0; h < 2; ++h) memcpy(ub + (size_t)(((it >> 1) * 2 + h) * 32 + n) * 16 + (it & 1) * 8, blk + 2 + 8 * h, 8);
+                    memcpy(ub + (size_t)nit * 512 + (size_t)((it >> 1) * 32 + n) * 4 + (it & 1) * 2, blk, 2);
+                }
+        }
+}
+// shapes lg_k_attn_tail is instantiated for: pairs of blocks per chain, row blocks per unit
+static bool attn_tail_shape(int qd, int E, int *np, int *rbs) {
+    if (qd % 512 || lg_segments(qd) != 8 || E % 256 || E > 4096) return false;
+    const int p = qd / 512, r = (E / 32 + LG_XCD_WGS - 1) / LG_XCD_WGS;
+    if (np) *np = p;
+    if (rbs) *rbs = r;
+    return (p == 1 && r == 1) || (p == 2 && r == 1) || (p == 4 && r == 3);
+}
+
 static const float *rope_table(lg_hip_model *m, int is_local, int hd, int *rc) {
     auto key = std::make_pair(is_local, hd);
     auto it = m->rope_tabs.find(key);
@@ -557,6 +586,14 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         push_rows(rows, o, 0, E);
         if ((rc = upload_tiled(m, rows, y.qd, &y.wo, stage))) return rc;
         // (8 query heads: the K segments of this projection are the heads, and the merge can run their chains itself)
+        if (getenv("LG_HIP_XCD_ATTN_TAIL") && atoi(getenv("LG_HIP_XCD_ATTN_TAIL")) > 0 && !m->target && attn_tail_shape(y.qd, E, nullptr, nullptr) &&
+            cu_count() == LG_XCDS * LG_XCD_WGS) {
+            stage.resize((size_t)E * (y.qd / 32) * 18);
+            pack_o_chains(rows.data(), y.qd, E, stage.data());
+            if (dev_alloc(m, &y.wo_ch, stage.size())) return -7;
+            HIP_TRY(hipMemcpy(y.wo_ch, stage.data(), stage.size(), hipMemcpyHostToDevice));
+            m->weight_bytes += stage.size();
+        }
         if (getenv("LG_HIP_MERGE_O") && atoi(getenv("LG_HIP_MERGE_O")) > 0 && !m->target && m->H == 8 && lg_segments(y.qd) == 8 && E % 64 == 0 && y.hd % 32 == 0 && y.hd <= 512 &&
             (rc = upload_tiled(m, rows, y.qd, &y.wo_rb, stage, true))) return rc;
         rows.clear();
@@ -641,12 +678,14 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         dev_alloc(m, &m->logits, HR * m->n_vocab) || dev_alloc(m, &m->ctl, (size_t)1))
         return -7;
     if (m->ple && dev_alloc(m, &m->eq, R * E * 5 / 4 + (size_t)12 * E)) return -7;
-    if (m->ple) {
-        if (dev_alloc(m, &m->tsync, (size_t)1) || dev_alloc(m, &m->tstamps, (size_t)LG_XTAIL_UNITS * 8)) return -7;
-        HIP_TRY(hipMemset(m->tstamps, 0, (size_t)LG_XTAIL_UNITS * 8 * 8));
+    if (!m->target) {                        // hand-over state of the one-XCD kernels (lg_xtail.h)
+        if (dev_alloc(m, &m->tsync, (size_t)1) || dev_alloc(m, &m->tstamps, (size_t)2 * LG_XTAIL_UNITS * 8)) return -7;
+        HIP_TRY(hipMemset(m->tstamps, 0, (size_t)2 * LG_XTAIL_UNITS * 8 * 8));
         HIP_TRY(hipMemset(m->tsync, 0, sizeof(XtailSync)));
+        HIP_TRY(hipMemset(m->aq, 0, R * max_qd * 5 / 4));       // (row slots past the block are read as operand rows of the matrix cores)
         if (getenv("LG_HIP_XCD_TAIL")) m->xcd_tail = atoi(getenv("LG_HIP_XCD_TAIL"));
     }
+    if (getenv("LG_HIP_XCD_ATTN_TAIL")) m->xcd_attn_tail = atoi(getenv("LG_HIP_XCD_ATTN_TAIL"));
     if (getenv("LG_HIP_MERGE_O")) m->merge_o = atoi(getenv("LG_HIP_MERGE_O"));
     if (getenv("LG_HIP_MERGE_O_SLICES")) m->merge_o_slices = atoi(getenv("LG_HIP_MERGE_O_SLICES"));
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
@@ -1046,6 +1085,25 @@ static void launch_merge_o(Launcher &lx, const MergeOArgs &a) {
     lx.rc = fail(-2, "merge_o: no instantiation for head_dim %d with %d chunks per wavefront", a.g.hd, rpl);
 }
 
+static bool use_attn_tail(const lg_hip_model *m, const Layer &y, int rows, int tiles) {
+    if (!y.wo_ch || !m->tsync || m->xcd_attn_tail <= 0 || rows > LG_HIP_MAX_ROWS || (m->xcd_attn_tail == 1 && rows < 3)) return false;
+    const int slices = (m->E + 1023) / 1024;
+    return tiles < 128 && m->H * rows <= 2 * LG_XCD_WGS && slices * rows <= LG_XCD_WGS && y.hd % 32 == 0 && y.hd <= 256;
+}
+template <int M>
+static void launch_attn_tail(Launcher &lx, const XattnTailArgs &a) {
+    if constexpr (M <= LG_HIP_MAX_ROWS) {
+        lg_hip_model *m = lx.m;
+        int np = 0, rb = 0;
+        if (!attn_tail_shape(a.g.H * a.g.hd, a.E, &np, &rb)) { lx.rc = fail(-2, "attn_tail: no instantiation for this shape"); return; }
+        const size_t lds = (size_t)(16 * np) * LG_MU_DWORDS * 4 + (size_t)8 * rb * 8 * 32 * 4;
+        const dim3 grid(LG_XCDS * LG_XCD_WGS);
+        if (np == 1 && rb == 1) LAUNCH(KC_ATAIL, (lg_k_attn_tail<M, 1, 1>), grid, dim3(512), lds, m->ctl, LG_XATTN_FIELDS(LG_XA, a) 0);
+        else if (np == 2 && rb == 1) LAUNCH(KC_ATAIL, (lg_k_attn_tail<M, 2, 1>), grid, dim3(512), lds, m->ctl, LG_XATTN_FIELDS(LG_XA, a) 0);
+        else LAUNCH(KC_ATAIL, (lg_k_attn_tail<M, 4, 3>), grid, dim3(512), lds, m->ctl, LG_XATTN_FIELDS(LG_XA, a) 0);
+    }
+}
+
 template <int M>
 static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
     if constexpr (M <= LG_HIP_MAX_ROWS) {
@@ -1206,7 +1264,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
     for (int L = 0; L < nl && !lx.rc; ++L) {
         const Layer &y = m->L[L];
         const int window = (y.is_local && m->window > 0) ? m->window + pos_off : 0;
-        bool fused_post = false, merged_o = false;
+        bool fused_post = false, merged_o = false, ffn_rows_done = false;
         {   // q/k/v projections, then per-head norm, rotary and the K/V rows of this block
             MmArgs a{ y.wqkv, E, y.qkv_m, m->qkv, m->hq, nullptr };
             if (rows_done) { launch_mm<M, false>(lx, KC_QKV, a); rows_done = false; }      // (the previous layer's tail did this layer's row work)
@@ -1265,6 +1323,18 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             }
             MergeArgs g{ kv->pm, kv->pl, kv->pacc, kv->tiles_max, H, y.hd, window, pos_off, m->aq, nullptr };
             merged_o = pos_off == 0 && use_merge_o(m, y, M, tiles);
+            if (pos_off == 0 && have_x && use_attn_tail(m, y, M, tiles)) {
+                // merge, output projection and the row work ahead of gate/up as one launch on one XCD
+                XattnTailArgs f{};
+                f.g = g; f.wo = y.wo_ch; f.aq = (uint32_t *)m->aq; f.pout = m->dout;
+                f.x = m->x[cur]; f.w_post = y.post_attn; f.w_pre = y.ffn_norm; f.x_out = m->x[cur ^ 1];
+                f.q = m->hq; f.q_units = (M >= 4) ? 2 : 1; f.E = E; f.eps = m->eps;
+                f.sync = m->tsync; f.spin_limit = 1 << 16; f.stamps = m->tail_stamps ? m->tstamps + LG_XTAIL_UNITS * 8 : nullptr;
+                launch_attn_tail<M>(lx, f);
+                cur ^= 1;
+                pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+                merged_o = true; ffn_rows_done = true;
+            } else
             if (merged_o) {
                 // the merge of (head, row) runs that head's chain of the output projection itself: eight slabs for the row kernel
                 MergeOArgs f{ g, y.wo_rb, m->dout, E, merge_o_slices(m, M), M };
@@ -1293,7 +1363,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 pend_dout = m->slabs; pend_parts = LG_XCDS; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
             } else {
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
-            rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
+            if (!ffn_rows_done) rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
             else if constexpr (mfma)
@@ -1396,7 +1466,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1436,6 +1506,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
+    else if (!strcmp(name, "xcd_attn_tail")) m->xcd_attn_tail = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "merge_o")) m->merge_o = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "merge_o_slices")) m->merge_o_slices = value < 0 ? 0 : value;
     else if (!strcmp(name, "xcd_tail")) m->xcd_tail = value < 0 ? 0 : value > 2 ? 2 : value;
@@ -1566,7 +1637,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -1623,12 +1694,12 @@ extern "C" int lg_hip_prefill(lg_hip_model *m, lg_hip_kv *kv, const int32_t *tok
     return 0;
 }
 
-extern "C" int lg_hip_tail_stamps(lg_hip_model *m, unsigned long long *dst, int cap) {
-    if (!m || !dst || !m->tstamps) return fail(-1, "tail_stamps: the model has no one-XCD tail");
+extern "C" int lg_hip_tail_stamps(lg_hip_model *m, int which, unsigned long long *dst, int cap) {
+    if (!m || !dst || !m->tstamps || which < 0 || which > 1) return fail(-1, "tail_stamps: the model has no one-XCD tail");
     if (cap < LG_XTAIL_UNITS * 8) return fail(-2, "tail_stamps: room for %d values needed", LG_XTAIL_UNITS * 8);
     HIP_TRY(hipSetDevice(m->device));
     HIP_TRY(hipStreamSynchronize(m->stream));
-    HIP_TRY(hipMemcpy(dst, m->tstamps, (size_t)LG_XTAIL_UNITS * 8 * 8, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(dst, m->tstamps + (size_t)which * LG_XTAIL_UNITS * 8, (size_t)LG_XTAIL_UNITS * 8 * 8, hipMemcpyDeviceToHost));
     return LG_XTAIL_UNITS;
 }
 
@@ -1726,7 +1797,7 @@ static void class_bytes(const lg_hip_model *m, const lg_hip_kv *kv, int pos, int
         {
             const int w = (y.is_local && m->window > 0) ? m->window : 0, st = (w > 0 && pos - w + 1 > 0) ? pos - w + 1 : 0;
             const int tiles = ((pos + rows - 1) >> 5) - (st >> 5) + 1;
-            b[use_merge_o(m, y, rows, tiles) ? KC_MERGE : KC_O] += (double)y.qd * m->E * q;
+            b[use_attn_tail(m, y, rows, tiles) ? KC_ATAIL : use_merge_o(m, y, rows, tiles) ? KC_MERGE : KC_O] += (double)y.qd * m->E * q;
         }
         if (m->xffn_built && m->xcd_ffn && rows >= 4) b[KC_FFN] += 3.0 * m->E * y.nff * q;
         else { b[KC_GATEUP] += 2.0 * m->E * y.nff * q; b[KC_DOWN] += (double)y.nff * m->E * q; }

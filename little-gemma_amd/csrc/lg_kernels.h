@@ -1398,12 +1398,13 @@ struct MergeArgs {
     float *xf;                 // optional f32 copy [M][H*hd]
 };
 #define LG_MERGE_FIELDS(X, v) X(const float *, pm, pm, v) X(const float *, pl, pl, v) X(const float *, pacc, pacc, v) X(int, tiles_max, tiles_max, v) X(int, H, H, v) X(int, hd, hd, v) X(int, window, window, v) X(int, pos_off, pos_off, v) X(int8_t *, xq, xq, v) X(float *, xf, xf, v)
-// The body for (head, row j) as a device function (the kernel below runs it per workgroup of its grid, lg_k_merge_o as
-// its first phase).  wts, pls: 512 floats of LDS each (exp(m_tile - M) and the sums of up to 512 tiles at a time), wmx: 4.
+// The body for (head, row j) as a device function run by 256 threads numbered tid (the kernel below runs it per workgroup
+// of its grid, lg_k_merge_o and lg_k_attn_tail as their first phase; a workgroup of 512 threads runs two at once, and
+// every thread of the workgroup has to be inside one of them: the body synchronises the workgroup).  wts, pls: 512 floats of LDS each (exp(m_tile - M) and the sums of up to 512 tiles at a time), wmx: 4.
 // after_first_fetch runs once the first batch of partials has been requested (a caller's own loads go behind it);
-// sink(d, r, q, dq, sum) receives dim d's result, its q8 value and its block's scale and sum.
-template <typename Hook, typename Sink>
-__device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const MergeArgs &a, int head, int j, float *wts, float *pls, float *wmx,
+// sink(d, r, q, dq, sum) receives dim d's result, its q8 value and its block's scale and sum.  WIDE_OK = false: heads of at most 256 dims.
+template <bool WIDE_OK = true, typename Hook, typename Sink>
+__device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const MergeArgs &a, int head, int j, int tid, float *wts, float *pls, float *wmx,
                                                    Hook &&after_first_fetch, Sink &&sink) {
     const int hd = a.hd;
     const int pos = ctl->pos + a.pos_off, pj = pos + j;
@@ -1413,7 +1414,7 @@ __device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const Mer
     // rows with at most one tile per thread (every sliding layer, global layers up to 8192 keys) read each tile's
     // maximum and sum once, with the pass that finds the row's maximum
     const bool once = hi - lo < LG_WG;
-    const int mine = lo + (int)threadIdx.x <= hi ? lo + (int)threadIdx.x : hi;
+    const int mine = lo + tid <= hi ? lo + tid : hi;
     const float pm1 = a.pm[base + mine], pl1 = a.pl[base + mine];
     // a batch of partials is one memory round trip (they were written by other CUs a moment ago), so the batch is
     // made large enough to hold all the tiles of a sliding layer.  Buffer loads: the row's partials as the base in
@@ -1422,8 +1423,8 @@ __device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const Mer
     // the weights and is requested here, with the maxima.
     constexpr int U = 24;
     float pau[U], pbu[U];                                     // dims 0..255, dims 256..511 (hd = 512 only)
-    const bool wide = hd > LG_WG;
-    const int tl = (int)threadIdx.x < hd ? (int)threadIdx.x : hd - 1;   // (lanes past a short head repeat its last dim; their sums are never used)
+    const bool wide = WIDE_OK && hd > LG_WG;                  // (a caller that never sees heads wider than 256 saves the second batch's registers)
+    const int tl = tid < hd ? tid : hd - 1;   // (lanes past a short head repeat its last dim; their sums are never used)
     auto fetch = [&](int c0, int cn, int n0) {
         const __amdgpu_buffer_rsrc_t rp = lg_buffer_rsrc(a.pacc + (base + c0) * hd);
         #pragma unroll
@@ -1435,26 +1436,26 @@ __device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const Mer
             #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int n = __builtin_amdgcn_readfirstlane(n0 + u < cn ? n0 + u : cn - 1);
-                pbu[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, (LG_WG + (int)threadIdx.x) * 4, n * hd * 4, 0));
+                pbu[u] = __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(rp, (LG_WG + tid) * 4, n * hd * 4, 0));
             }
         }
     };
     fetch(lo, hi - lo + 1 < 512 ? hi - lo + 1 : 512, 0);
     after_first_fetch();
     float mx = pm1;
-    for (int n = lo + (int)threadIdx.x + LG_WG; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
+    for (int n = lo + tid + LG_WG; n <= hi; n += LG_WG) mx = fmaxf(mx, a.pm[base + n]);
     mx = lg_max_n(mx, 64);
-    if ((threadIdx.x & 63) == 0) wmx[threadIdx.x >> 6] = mx;
+    if ((tid & 63) == 0) wmx[tid >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
     float L = 0.0f, o[2] = { 0.0f, 0.0f };
     for (int c0 = lo; c0 <= hi; c0 += 512) {
         const int cn = hi - c0 + 1 < 512 ? hi - c0 + 1 : 512;
         if (once) {
-            if ((int)threadIdx.x < cn) { wts[threadIdx.x] = lg_expf(pm1 - mx); pls[threadIdx.x] = pl1; }
+            if (tid < cn) { wts[tid] = lg_expf(pm1 - mx); pls[tid] = pl1; }
         } else {
             __syncthreads();
-            for (int n = threadIdx.x; n < cn; n += LG_WG) { wts[n] = lg_expf(a.pm[base + c0 + n] - mx); pls[n] = a.pl[base + c0 + n]; }
+            for (int n = tid; n < cn; n += LG_WG) { wts[n] = lg_expf(a.pm[base + c0 + n] - mx); pls[n] = a.pl[base + c0 + n]; }
         }
         __syncthreads();
         for (int n0 = 0; n0 < cn; n0 += U) {                  // fma in tile order
@@ -1473,7 +1474,7 @@ __device__ __forceinline__ void lg_attn_merge_body(const StepCtl *ctl, const Mer
     }
     #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
-        const int d = h2 * LG_WG + threadIdx.x;
+        const int d = h2 * LG_WG + tid;
         if (h2 * LG_WG >= hd) break;
         const float r = d < hd ? o[h2] / L : 0.0f;
         float dq; int sum;
@@ -1486,7 +1487,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_merge(const StepCtl *ctl, LG_
     MergeArgs a; LG_MERGE_FIELDS(LG_XI, a)
     __shared__ float wts[512], pls[512], wmx[LG_WG / 64];
     const int head = blockIdx.x, j = blockIdx.y, hd = a.hd, qd = a.H * hd;
-    lg_attn_merge_body(ctl, a, head, j, wts, pls, wmx, [] {}, [&](int d, float r, int q, float dq, int sum) {
+    lg_attn_merge_body(ctl, a, head, j, (int)threadIdx.x, wts, pls, wmx, [] {}, [&](int d, float r, int q, float dq, int sum) {
         const int e = head * hd + d;                           // element of the row, natural order
         a.xq[lg_q8_off<M>(qd, j, e >> 4, e & 15)] = (int8_t)q;          // order the attn_output matmul reads
         if ((d & 31) == 0) lg_q8_ds<M>(a.xq, qd)[lg_q8_ds_idx<M>(qd, j, e >> 5)] = make_float2(dq, __int_as_float(sum));

@@ -218,3 +218,278 @@ __global__ __launch_bounds__(LG_WG) void lg_k_ple_tail(StepCtl *ctl, LG_XTAIL_FI
 // three hand-overs instead of two, and slower at every width: E4B shape, 5 rows 11.2 against 10.6 us per launch (step
 // 2.231 against 2.210 ms), 6 rows 2.326 against 2.303 ms, 8 rows 2.494 against 2.477 ms.  A hand-over costs about 1 us
 // once the wait for the stores and the load of what was handed over are counted, more than the lighter phases save.
+
+// the sum over the 256 lanes of wavefronts 0..3 (order of lg_block_sum256) in a workgroup of 8 wavefronts that all call it
+__device__ __forceinline__ float lg_block_sum256_of512(float v, float *scratch8) {
+    v = lg_wave_sum64(v);
+    if ((threadIdx.x & 63) == 0) scratch8[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (scratch8[0] + scratch8[1]) + (scratch8[2] + scratch8[3]);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Measured at the E4B shape (5 rows): 12.3 us per launch against 4.3 + 4.1 + 4.5 for the three kernels it replaces, and the
+// step 2.219 against 2.203 ms: not a gain, so the option is off by default.  By the stamps: merges 4.3-4.8 us (the same chain of
+// round trips as the separate kernel: the partials come from other XCDs), hand-over 0.45, copy of the merged rows 0.5, the
+// projection 2.1 (bound by the vector instructions around the MFMA: 640 chains x 8 steps x ~20 instructions on one XCD's
+// 128 SIMDs), hand-over 0.55, row work 1.7; the three separate kernels hide their launch gaps under each other's tails, the
+// phases of one launch cannot.
+// The narrow end of the attention half the same way: merge -> output projection -> row work, one launch on one XCD.
+//   1  merge of the tile partials of every (head, row), two of them at a time per unit (a unit is 8 wavefronts, a merge
+//      takes 4); the q8 of the merged head goes to the XCD's L2 in the matrix-core block order (80 dwords per block of 32:
+//      8 row slots of 32 bytes, then 8 x {scale, 12582912 + 8 * sum});
+//      hand-over;
+//   2  the output projection on the matrix cores: a chain = (block of 32 output rows, K segment); wavefront w of unit u
+//      runs segment w of the row blocks u, u + 32, ...: per block of the segment one v_mfma_i32_32x32x32_i8 (A = the
+//      block's activations in 8 row slots, B = the 32 rows' nibbles) and four fma per lane, p = fma(xd * dw, (float)dot, p),
+//      the chain of lg_k_mm; the 8 segment sums of a row meet in LDS in the adjacent-pair tree.  The weights (E x K / 32
+//      units = 92 KB per unit at the E4B shape) are requested at kernel start and arrive under the merge: a lone XCD pulls
+//      3 MB from HBM in about 2 us.  On v_dot4 the same projection would keep the XCD's 128 SIMDs busy for 4.5 us;
+//      hand-over;
+//   3  the row work ahead of gate/up (residual update, ffn norm, q8 in the order the gate/up kernel reads) by units (slice, row).
+// Weights: per chain the stream layout of lg_xffn.h (pairs of blocks: [pair][half h][row n] 8 + 8 nibble bytes, then
+// [pair][row n] the two f16 scales), chains ordered [row block][segment].
+struct XattnTailArgs {
+    MergeArgs      g;            // g.xq, g.xf unused
+    const uint8_t *wo;           // chains of attn_output
+    uint32_t      *aq;           // [K / 32][80] the merged rows as matrix-core blocks
+    float         *pout;         // [M][E]
+    const float   *x, *w_post, *w_pre;
+    float         *x_out;
+    int8_t        *q;
+    int            q_units;      // 2: blocks of lg_k_geglu_m (4..8 rows), 1: units of lg_k_geglu_t (up to 3 rows)
+    int            E;
+    float          eps;
+    XtailSync     *sync;
+    int            spin_limit;
+    unsigned long long *stamps;
+};
+#define LG_XATTN_FIELDS(X, v) X(const float *, pm, g.pm, v) X(const float *, pl, g.pl, v) X(const float *, pacc, g.pacc, v) X(int, tiles_max, g.tiles_max, v) \
+    X(int, H, g.H, v) X(int, hd, g.hd, v) X(int, window, g.window, v) X(int, pos_off, g.pos_off, v) X(const uint8_t *, wo, wo, v) X(XtailSync *, sync, sync, v) \
+    X(const float *, x, x, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(uint32_t *, aq, aq, v) X(float *, pout, pout, v) \
+    X(float *, x_out, x_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(int, E, E, v) X(float, eps, eps, v) X(int, spin_limit, spin_limit, v) \
+    X(unsigned long long *, stamps, stamps, v)
+
+// Row blocks of a unit whose weights are requested with the merge's partials; the rest after the merge.  All of them early
+// is the faster choice: requested after the merge they delay the first hand-over, whose store wait also waits for them
+// (the merge phase 4.3-4.8 us either way, the whole launch 10.1 against 11.0 us).
+#ifndef LG_XATTN_EARLY
+#define LG_XATTN_EARLY 8
+#endif
+// M: rows; NP: pairs of blocks per chain (K / 32 / 8 / 2); RB: most row blocks per unit (E / 32 over 32 units).
+template <int M, int NP, int RB>
+__global__ __launch_bounds__(512) void lg_k_attn_tail(StepCtl *ctl, LG_XATTN_FIELDS(LG_XP, _) int p_end_) {
+    if (blockIdx.x & (LG_XCDS - 1)) return;
+    XattnTailArgs a; LG_XATTN_FIELDS(LG_XI, a)
+    a.g.xq = nullptr; a.g.xf = nullptr;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float wts[2][512], pls[2][512], wmx[2][4], red3[2][8];
+    __shared__ __align__(16) int8_t hq[2][512];
+    __shared__ float2 hds[2][16];
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), half = wave >> 2, tid = t & 255;
+    const int n = lane & 31, h = lane >> 5;
+    const int E = a.E, nq = E >> 2, hd = a.g.hd, nbh = hd >> 5, nit = 2 * NP, nb = 8 * nit;
+    const int U = LG_XCD_WGS, u = blockIdx.x >> 3;
+    const int slices = (E + 1023) >> 10, nrow = slices * M;
+    const bool rowunit = u < nrow, rowlane = t < LG_WG;
+    const int v_ = u / M, jr = u - v_ * M;
+    const uint32_t gen = a.sync->gen;
+    const int xcc = lg_xcc_id();
+    auto stamp = [&](int i) { if (a.stamps && t == 0) a.stamps[(size_t)u * 8 + i] = wall_clock64(); };
+    stamp(0);
+    lg_v16i magic;
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;
+    asm volatile("" : "+v"(magic));
+    // ---- phase 1: the merges (tasks u and u + 32), with everything else this unit reads requested behind their partials ----
+    const int ntasks = a.g.H * M, task = u + U * half;
+    const bool on = task < ntasks;
+    const int tk = on ? task : ntasks - 1, head = tk % a.g.H, j = tk / a.g.H;
+    struct Pair { lg_x4u q; uint32_t sw; };
+    Pair wq[RB][NP];
+    bool live[RB];
+    float4 xv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
+    const int nrb = E >> 5;
+    auto fetch_w = [&](int k0, int k1) {
+        #pragma unroll
+        for (int k = 0; k < RB; ++k) {
+            if (k < k0 || k >= k1) continue;
+            const int rb = u + U * k;
+            live[k] = rb < nrb;
+            const uint8_t *cb = a.wo + ((size_t)(live[k] ? rb : 0) * 8 + wave) * ((size_t)nit * 576);    // (no such row block: the first one's weights, never stored)
+            #pragma unroll
+            for (int jp = 0; jp < NP; ++jp) {
+                wq[k][jp].q = __builtin_nontemporal_load((const lg_x4u *)(cb + (size_t)((jp * 2 + h) * 32 + n) * 16));
+                wq[k][jp].sw = __builtin_nontemporal_load((const uint32_t *)(cb + (size_t)nit * 512 + (size_t)(jp * 32 + n) * 4));
+            }
+        }
+    };
+    lg_attn_merge_body<false>(ctl, a.g, head, j, tid, wts[half], pls[half], wmx[half], [&] { fetch_w(0, LG_XATTN_EARLY); }, [&](int d, float r, int q, float dq, int sum) {
+        hq[half][d] = (int8_t)q;
+        if ((d & 31) == 0) hds[half][d >> 5] = make_float2(dq, 12582912.0f + (float)(8 * sum));
+    });
+    fetch_w(LG_XATTN_EARLY, RB);
+    __syncthreads();
+    if (on && tid < (hd >> 2)) {                               // dword tid of the merged head: block tid / 8, dword tid % 8 of it
+        const int b = tid >> 3, dw = tid & 7;
+        uint32_t *blk = a.aq + (size_t)(head * nbh + b) * LG_MU_DWORDS;
+        blk[j * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))] = *(const uint32_t *)(hq[half] + 4 * tid);
+        if (dw == 0) *(float2 *)(blk + 64 + 2 * j) = hds[half][b];
+    }
+    stamp(1);
+    // ---- hand-over: the merged rows are in the XCD's L2 ----
+    const int nmerge = ntasks < U ? ntasks : U;                 // units that ran a merge
+    lg_wait_vm();
+    __syncthreads();
+    if (wave == 0) {
+        const int err = lg_xcd_arrive_wait(a.sync->flags[0], u, u < nmerge, nmerge, 2 * gen + 1, xcc, a.spin_limit);
+        if (err && lane == 0) atomicOr(&ctl->err, err);
+    }
+    __syncthreads();
+    stamp(2);
+    unsigned char *la = smem;                                  // [nb][320]
+    float *red = (float *)(smem + (size_t)nb * LG_MU_DWORDS * 4);          // [8 segments][RB][8 row slots][32]
+    {
+        const int n16 = nb * LG_MU_DWORDS / 4;                 // 16-byte units
+        for (int i0 = t; i0 < n16; i0 += 4 * 512) {
+            const int i1 = min(i0 + 512, n16 - 1), i2 = min(i0 + 1024, n16 - 1), i3 = min(i0 + 1536, n16 - 1);
+            lg_x4u v0 = lg_ld4_sc_issue<2>((const unsigned char *)a.aq + (size_t)i0 * 16), v1 = lg_ld4_sc_issue<2>((const unsigned char *)a.aq + (size_t)i1 * 16);
+            lg_x4u v2 = lg_ld4_sc_issue<2>((const unsigned char *)a.aq + (size_t)i2 * 16), v3 = lg_ld4_sc_issue<2>((const unsigned char *)a.aq + (size_t)i3 * 16);
+            lg_ld4_wait(v0, v1, v2, v3);
+            *(lg_x4u *)(la + (size_t)i0 * 16) = v0; *(lg_x4u *)(la + (size_t)i1 * 16) = v1;
+            *(lg_x4u *)(la + (size_t)i2 * 16) = v2; *(lg_x4u *)(la + (size_t)i3 * 16) = v3;
+        }
+    }
+    __syncthreads();
+    stamp(3);
+    // (what phase 3 needs besides the projection is requested here: behind the loads this phase waits for, with a phase's
+    // time to arrive, and not occupying registers during the merge)
+    if (rowunit && rowlane) {
+        const float4 *xr = (const float4 *)(a.x + (size_t)jr * E), *w1 = (const float4 *)a.w_post, *w2 = (const float4 *)a.w_pre;
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; wpost[v] = w1[t + 256 * v]; wpre[v] = w2[t + 256 * v]; }
+    }
+    // ---- phase 2: segment `wave` of the unit's row blocks ----
+    {
+        const int arow = n < 8 ? n : 7;
+        float p[RB][4];
+        #pragma unroll
+        for (int k = 0; k < RB; ++k)
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) p[k][i] = 0.0f;
+        #pragma unroll
+        for (int jp = 0; jp < NP; ++jp) {
+            #pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const XffnAct ac = lg_xffn_act(la + (size_t)(wave * nit + 2 * jp + e) * (LG_MU_DWORDS * 4), arow, h);
+                #pragma unroll
+                for (int k = 0; k < RB; ++k) {
+                    lg_v2u q; q.x = e ? wq[k][jp].q.z : wq[k][jp].q.x; q.y = e ? wq[k][jp].q.w : wq[k][jp].q.y;
+                    lg_xffn_step(ac.av, ac.xd, ac.cf, q, lg_h2f((uint16_t)(e ? wq[k][jp].sw >> 16 : wq[k][jp].sw)), magic, p[k]);
+                }
+            }
+        }
+        #pragma unroll
+        for (int k = 0; k < RB; ++k)
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) red[((size_t)(wave * RB + k) * 8 + 4 * h + i) * 32 + n] = p[k][i];      // (all 8 row slots: the tree reads the first M)
+    }
+    __syncthreads();
+    for (int idx = t; idx < RB * M * 32; idx += 512) {         // the adjacent-pair tree over the 8 segments
+        const int k = idx / (M * 32), rem = idx - k * (M * 32), jj = rem >> 5, nn = rem & 31, rb = u + U * k;
+        if (rb < nrb) {
+            const float *b = red + ((size_t)k * 8 + jj) * 32 + nn;
+            const size_t sg = (size_t)RB * 8 * 32;
+            a.pout[(size_t)jj * E + rb * 32 + nn] = ((b[0] + b[sg]) + (b[2 * sg] + b[3 * sg])) + ((b[4 * sg] + b[5 * sg]) + (b[6 * sg] + b[7 * sg]));
+        }
+    }
+    stamp(4);
+    // ---- hand-over: the projection's [M][E] is in the XCD's L2 ----
+    lg_wait_vm();
+    __syncthreads();
+    if (!rowunit) {
+        if (t == 0) lg_st_sc<0>(a.sync->flags[1] + u, ((2 * gen + 2) << 4) | (uint32_t)xcc);
+        return;
+    }
+    if (wave == 0) {
+        const int err = lg_xcd_arrive_wait(a.sync->flags[1], u, true, U, 2 * gen + 2, xcc, a.spin_limit);
+        if (err && lane == 0) atomicOr(&ctl->err, err);
+    }
+    __syncthreads();
+    stamp(5);
+    // ---- phase 3: the row work of row jr, this unit storing and quantizing slice v_ ----
+    float4 dv[LG_ROWV];
+    if (rowlane) {
+        lg_x4u d0, d1, d2, d3;
+        const float *pr = a.pout + (size_t)jr * E;
+        const int last = nq - 1;
+        d0 = lg_ld4_sc_issue<2>(pr + 4 * min(t, last));
+        d1 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 256, last));
+        d2 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 512, last));
+        d3 = lg_ld4_sc_issue<2>(pr + 4 * min(t + 768, last));
+        lg_ld4_wait(d0, d1, d2, d3);
+        const lg_x4u d[4] = { d0, d1, d2, d3 };
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) dv[v] = make_float4(__uint_as_float(d[v].x), __uint_as_float(d[v].y), __uint_as_float(d[v].z), __uint_as_float(d[v].w));
+    }
+    stamp(6);
+    {
+        float ss = 0.0f;
+        if (rowlane) {
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(dv[v], ss);
+        }
+        ss = lg_block_sum256_of512(ss, red3[0]);
+        if (rowlane) {
+            const float sc = 1.0f / sqrtf(ss / (float)E + a.eps);
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 w = wpost[v];
+                float4 r;
+                r.x = xv[v].x + dv[v].x * sc * w.x;  r.y = xv[v].y + dv[v].y * sc * w.y;
+                r.z = xv[v].z + dv[v].z * sc * w.z;  r.w = xv[v].w + dv[v].w * sc * w.w;
+                xv[v] = r;
+            }
+            float4 *xo = (float4 *)(a.x_out + (size_t)jr * E);
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq && v == v_) xo[t + 256 * v] = xv[v];
+        }
+    }
+    {
+        float ss = 0.0f;
+        if (rowlane) {
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) ss = lg_sumsq4(xv[v], ss);
+        }
+        ss = lg_block_sum256_of512(ss, red3[1]);
+        if (rowlane) {
+            const float sc = 1.0f / sqrtf(ss / (float)E + a.eps);
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 w = wpre[v];
+                xv[v] = make_float4(xv[v].x * sc * w.x, xv[v].y * sc * w.y, xv[v].z * sc * w.z, xv[v].w * sc * w.w);
+            }
+        }
+    }
+    if (rowlane) {
+        #pragma unroll
+        for (int v = 0; v < LG_ROWV; ++v) {
+            if (t + 256 * v >= nq || v != v_) continue;
+            float d; int sum;
+            const uint32_t packed = lg_quant4_8lanes(xv[v], &d, &sum);
+            const int quad = t + 256 * v;
+            if (a.q_units == 2) {
+                uint32_t *blk = (uint32_t *)a.q + (size_t)(quad >> 3) * LG_MU_DWORDS;
+                const int dw = quad & 7;
+                blk[jr * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))] = packed;
+                if ((t & 7) == 0) *(float2 *)(blk + 64 + 2 * jr) = make_float2(d, 12582912.0f + (float)(8 * sum));
+            } else {
+                uint32_t *unit = (uint32_t *)a.q + ((size_t)(quad >> 3) * ((M + 2) / 3) + jr / 3) * 32;
+                unit[(jr % 3) * 8 + (quad & 7)] = packed;
+                if ((t & 7) == 0) *(float2 *)(unit + 24 + 2 * (jr % 3)) = make_float2(d, __int_as_float(sum));
+            }
+        }
+    }
+    stamp(7);
+    if (u == 0 && t == 0) a.sync->gen = gen + 1;
+}

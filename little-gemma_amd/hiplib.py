@@ -74,7 +74,7 @@ def load_hip():
     L.lg_hip_get_hidden.argtypes = [C.c_void_p, f32p]
     L.lg_hip_get_logits.argtypes = [C.c_void_p, C.c_int, f32p]
     L.lg_hip_set_option.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
-    L.lg_hip_tail_stamps.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+    L.lg_hip_tail_stamps.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int]
     L.lg_hip_mtp_rounds.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, i32p, i32p, i32p, C.POINTER(C.c_int32)]
     L.lg_hip_schedule_load.argtypes = [C.c_void_p, i32p, C.c_int, C.c_int, C.c_int]
     L.lg_hip_schedule_run.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
@@ -274,10 +274,11 @@ class HipBackend:
     def set_option(self, name, value):
         hip_check(self.H.lg_hip_set_option(self.dev, name.encode(), int(value)), "set_option")
 
-    def tail_stamps(self):
-        """[64 units][8] wall-clock stamps (100 MHz ticks) of the latest one-XCD layer tail (option xcd_tail_stamps)."""
+    def tail_stamps(self, which=0):
+        """[64 units][8] wall-clock stamps (100 MHz ticks) of the latest one-XCD launch (option xcd_tail_stamps):
+        which = 0 the layer's tail, 1 the attention half's."""
         out = np.zeros((64, 8), np.uint64)
-        hip_check(self.H.lg_hip_tail_stamps(self.dev,
+        hip_check(self.H.lg_hip_tail_stamps(self.dev, which,
                                             out.ctypes.data_as(C.c_void_p), out.size), "tail_stamps")
         return out
 

@@ -145,6 +145,7 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
     per-layer inputs built on a second stream beside layer 0) change
     timing only: every combination leaves the same cache rows and the same logits rows of a verify block."""
     monkeypatch.setenv("LG_HIP_MERGE_O", "1")          # (builds the second copy of attn_output that the merge_o option needs)
+    monkeypatch.setenv("LG_HIP_XCD_ATTN_TAIL", "1")    # (... and the one the xcd_attn_tail option needs)
     path, spec = model_path(name, **over)
     V = spec["n_vocab"]
     rng = np.random.default_rng(rows)
@@ -169,6 +170,7 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
     for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
                      ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
                      ("xcd_tail", 0), ("xcd_tail", 2),    # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
+                     ("xcd_attn_tail", 0), ("xcd_attn_tail", 2),   # (attention merge + output projection + row work: separate kernels / one launch on one XCD for every width)
                      ("merge_o", 0), ("merge_o", 2), ("merge_o_slices", 8)):   # (attention merge + output projection: separate / one launch for every width / another cut of the rows)
         print(f"rows={rows} option {opt}={val}", flush=True)
         got = run(**{opt: val})

@@ -149,3 +149,49 @@ def test_verify_steps_with_the_one_xcd_tail_match_the_oracle(lg, ob, gpu_require
             pos += adv; tok = int(out[adv - 1])
     finally:
         gpu.close(); o.close()
+
+
+@pytest.mark.parametrize("name", ["tiny", "tiny_full"])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_verify_steps_with_the_one_xcd_attention_tail_match_the_oracle(lg, ob, gpu_required, model_path, monkeypatch, name, rows):
+    """Whole verify steps with attention merge, output projection (on the matrix cores) and the row work after it as
+    one launch on one XCD (lg_k_attn_tail, option xcd_attn_tail = 2: every block width): accept counts, successors,
+    every row's logits and the kept hidden state are the oracle's, bit for bit, over several steps, and the same as
+    with the separate kernels.  tiny has 64-wide heads everywhere, tiny_full 128-wide ones in its global layers (two
+    chain lengths), sliding windows that start inside the cache and per-layer inputs (so both one-XCD launches run)."""
+    monkeypatch.setenv("LG_HIP_XCD_ATTN_TAIL", "2")     # (builds the copy of attn_output that the kernel reads)
+    path, spec = model_path(name)
+    V = spec["n_vocab"]
+    rng = np.random.default_rng(rows + 160)
+    prompt = rng.integers(0, V, 150).astype(np.int32)
+    o = ob.Oracle(path)
+    gpu = lg.hiplib.HipBackend(path, 400, max_rows=8)
+    try:
+        gpu.set_option("xcd_attn_tail", 2)
+        gpu.prefill(prompt[:-1], 0)
+        gpu.set_option("store_logits", 1)
+        okv = o.kv_new(400, ob.I8)
+        o.prefill(okv, prompt[:-1], 0, ob.I8)
+        lg.hiplib.hip_check(gpu.H.lg_hip_kv_save_prefix(gpu.dkv, 149), "save")
+        pos = 149
+        tok = int(prompt[-1])
+        for step in range(5):
+            blk = np.array([tok] + rng.integers(0, V, rows - 1).tolist(), np.int32)
+            print(f"xcd attention tail {name} rows={rows} step={step} pos={pos}", flush=True)
+            adv, out = gpu.forward_spec(blk, pos)
+            hid = gpu.last_hidden(spec["n_embd"])
+            logits = np.stack([gpu.logits_row(j, V) for j in range(rows)])
+            oadv, oout, ohid = o.forward_spec_all(okv, blk, pos, ob.I8, want_hidden=True)
+            assert adv == oadv and out[:adv].tolist() == oout[:adv].tolist()
+            assert np.array_equal(hid.view(np.uint32), ohid.view(np.uint32))
+            if step == 0:
+                lg.hiplib.hip_check(gpu.H.lg_hip_kv_restore_prefix(gpu.dkv, 149), "restore")
+                gpu.set_option("xcd_attn_tail", 0)
+                adv0, out0 = gpu.forward_spec(blk, pos)
+                logits0 = np.stack([gpu.logits_row(j, V) for j in range(rows)])
+                assert adv0 == adv and np.array_equal(out0, out)
+                assert np.array_equal(logits0.view(np.uint32), logits.view(np.uint32))
+                gpu.set_option("xcd_attn_tail", 2)
+            pos += adv; tok = int(out[adv - 1])
+    finally:
+        gpu.close(); o.close()
