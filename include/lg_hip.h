@@ -263,6 +263,12 @@ int    lg_hip_attention_noalloc(const float *d_q, const uint16_t *d_kc, const ui
                                 int n_head_kv, int hd, int seq, int window, int pos, float *d_out, void *stream);
 int    lg_hip_attention_noalloc_init(void);
 size_t lg_hip_attention_noalloc_limit(void);
+/* ffn_down of a verify block of 4..8 rows on the matrix cores (lg_k_down_m), in isolation: act = rows x FF floats (quantized
+ * to q8 on the device, as the gate/up kernel's epilogue does), down = FF-wide q4_0 rows of the E outputs; out = rows x E,
+ * the four K-quarter slabs added by the four workgroups of a row group themselves (join = 1: a hand-over inside their XCD)
+ * or here as the consumer kernel adds them (join = 0).  The model path is ffn_down of
+ * src/cuda/model-cuda-i8.cu's q4_0 x q8 matmul; this entry exists for parity tests and timing. */
+int    lg_hip_down_m(const float *act, const void *down_q4_0, int rows, int E, int FF, int join, float *out, int repeats, float *kernel_ms);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
 int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 */

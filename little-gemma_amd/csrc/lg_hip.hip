@@ -147,6 +147,7 @@ struct HostTensor { uint32_t type, n_dims; uint64_t dims[4]; const void *data; }
 struct Layer {
     uint8_t *wqkv = nullptr, *wo = nullptr, *wgu = nullptr, *wdown = nullptr, *winp = nullptr, *wproj = nullptr;
     float *winp_f = nullptr, *wproj_f = nullptr;   // inp_gate / proj when the file keeps them in a float type (then winp / wproj are null)
+    uint8_t *wdn_m = nullptr;                      // ffn_down again as the per-workgroup streams of lg_k_down_m
     uint8_t *wo_ch = nullptr;                      // attn_output again as matrix-core chains [row block][segment]: lg_k_attn_tail
     uint8_t *wo_rb = nullptr;                      // attn_output again as row-block tiles: the chains of lg_k_merge_o
     uint8_t *xgu = nullptr, *xdn = nullptr;        // gate/up and ffn_down again as per-workgroup streams of the XCD-partitioned kernel (lg_xffn.h)
@@ -207,6 +208,10 @@ struct lg_hip_model {
     int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
+    int down_m = 1;                          // option: ffn_down of 4..8-row blocks on the matrix cores (lg_k_down_m): 1 = the row group's four workgroups add
+                                             // their slabs themselves, 2 = four slabs for the consumer, 0 = the v_dot4 kernels; its streams are built
+                                             // at commit unless LG_HIP_DOWN_M=0
+    DownMSync *dmsync = nullptr;
     int xcd_attn_tail = 0;                   // option: attention merge, output projection and the row work after it as one launch on one XCD
                                              // (lg_k_attn_tail): 0 off (as measured it gains nothing), 1 from three rows up, 2 for every verify block;
                                              // the copy of the weights it reads is only built when LG_HIP_XCD_ATTN_TAIL is set at commit
@@ -446,6 +451,33 @@ static void xffn_pack_dn(const uint8_t *down, const XffnGeo &g, uint8_t *dst) {
     });
 }
 
+// ffn_down as the streams of lg_k_down_m: workgroup (row group r of 64, K quarter q), per segment 8q + s and operand of up to
+// 32 rows the pair layout of the streams above
+static void pack_down_m(const uint8_t *down, const DownMGeo &g, uint8_t *dst) {
+    const size_t rowb = (size_t)(g.FF >> 5) * 18;
+    memset(dst, 0, 256 * g.wg_bytes);
+    for_workgroups([&](int wg) {
+        const int r = wg >> 2, q = wg & 3;
+        for (int s = 0; s < 8; ++s)
+            for (int o = 0; o < g.ops; ++o) {
+                const int vr = g.RW - 32 * o < 32 ? g.RW - 32 * o : 32;
+                uint8_t *ob = dst + (size_t)wg * g.wg_bytes + (size_t)s * g.seg_bytes + (size_t)32 * o * g.nitdp * 18;
+                for (int n = 0; n < vr; ++n) {
+                    const uint8_t *row = down + (size_t)(r * g.RW + 32 * o + n) * rowb;
+                    for (int it = 0; it < g.nitd; ++it) {
+                        const uint8_t *blk = row + (size_t)((8 * q + s) * g.nitd + it) * 18;
+                        for (int h = 0; h < 2; ++h) memcpy(ob + (size_t)(((it >> 1) * 2 + h) * vr + n) * 16 + (it & 1) * 8, blk + 2 + 8 * h, 8);
+                        memcpy(ob + (size_t)g.nitdp * vr * 16 + (size_t)((it >> 1) * vr + n) * 4 + (it & 1) * 2, blk, 2);
+                    }
+                }
+            }
+    });
+}
+// shapes lg_k_down_m is instantiated for: operands per workgroup, pairs of blocks per segment
+static bool down_m_shape(const DownMGeo &g) {
+    return g.ok && ((g.ops == 1 && g.npairs <= 3) || (g.ops == 2 && g.npairs <= 5) || (g.ops == 2 && g.npairs <= 8));
+}
+
 // attn_output as the chains of lg_k_attn_tail: chain (row block rb of 32 rows, K segment c of 8) = the segment's nit blocks
 // of the 32 rows in the pair layout of the streams above; chains ordered [rb][c], nit * 576 bytes each
 static void pack_o_chains(const uint8_t *const *rows, int k, int m, uint8_t *dst) {
@@ -608,6 +640,19 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         push_rows(rows, d, 0, E);
         if ((rc = upload_tiled(m, rows, y.nff, &y.wdown, stage))) return rc;
         rows.clear();
+        if (!(getenv("LG_HIP_DOWN_M") && atoi(getenv("LG_HIP_DOWN_M")) <= 0) && !m->target && max_rows >= 4 && cu_count() == LG_XCDS * LG_XCD_WGS) {
+            const DownMGeo dg = lg_down_m_geo(E, y.nff);
+            if (down_m_shape(dg)) {
+                xstage.resize(256 * dg.wg_bytes);
+                pack_down_m((const uint8_t *)d->data, dg, xstage.data());
+                if (dev_alloc(m, &y.wdn_m, 256 * dg.wg_bytes)) return -7;
+                HIP_TRY(hipMemcpy(y.wdn_m, xstage.data(), 256 * dg.wg_bytes, hipMemcpyHostToDevice));
+                if (!m->dmsync) {
+                    if (dev_alloc(m, &m->dmsync, (size_t)1)) return -7;
+                    HIP_TRY(hipMemset(m->dmsync, 0, sizeof(DownMSync)));
+                }
+            }
+        }
         if (xffn) {                                               // (second copies: not counted into weight_bytes, which says what a step streams)
             xstage.resize(256 * (xg.gu_bytes > xg.dn_bytes ? xg.gu_bytes : xg.dn_bytes));
             xffn_pack_gu((const uint8_t *)g->data, (const uint8_t *)u->data, xg, xstage.data());
@@ -686,6 +731,7 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         if (getenv("LG_HIP_XCD_TAIL")) m->xcd_tail = atoi(getenv("LG_HIP_XCD_TAIL"));
     }
     if (getenv("LG_HIP_XCD_ATTN_TAIL")) m->xcd_attn_tail = atoi(getenv("LG_HIP_XCD_ATTN_TAIL"));
+    if (getenv("LG_HIP_DOWN_M")) m->down_m = atoi(getenv("LG_HIP_DOWN_M"));
     if (getenv("LG_HIP_MERGE_O")) m->merge_o = atoi(getenv("LG_HIP_MERGE_O"));
     if (getenv("LG_HIP_MERGE_O_SLICES")) m->merge_o_slices = atoi(getenv("LG_HIP_MERGE_O_SLICES"));
     if (m->ple && (dev_alloc(m, &m->pmp_raw, R * m->ple * nl) || dev_alloc(m, &m->pq, R * m->ple * 5 / 4) || dev_alloc(m, &m->pgf, R * m->ple)))
@@ -1085,6 +1131,17 @@ static void launch_merge_o(Launcher &lx, const MergeOArgs &a) {
     lx.rc = fail(-2, "merge_o: no instantiation for head_dim %d with %d chunks per wavefront", a.g.hd, rpl);
 }
 
+template <int M>
+static void launch_down_m(Launcher &lx, const DownMArgs &a) {
+    if constexpr (M >= 4 && M <= LG_HIP_MAX_ROWS) {
+        const DownMGeo g = lg_down_m_geo(a.E, a.FF);
+        const size_t lds = (size_t)8 * g.nitd * (LG_MU_DWORDS * 4) + (size_t)8 * g.ops * 8 * 32 * 4;
+        if (g.ops == 1 && g.npairs <= 3) LAUNCH(KC_DOWN, (lg_k_down_m<M, 1, 3>), dim3(256), dim3(512), lds, LG_DOWNM_FIELDS(LG_XA, a) 0);
+        else if (g.ops == 2 && g.npairs <= 5) LAUNCH(KC_DOWN, (lg_k_down_m<M, 2, 5>), dim3(256), dim3(512), lds, LG_DOWNM_FIELDS(LG_XA, a) 0);
+        else if (g.ops == 2 && g.npairs <= 8) LAUNCH(KC_DOWN, (lg_k_down_m<M, 2, 8>), dim3(256), dim3(512), lds, LG_DOWNM_FIELDS(LG_XA, a) 0);
+        else lx.rc = fail(-2, "down_m: no instantiation for this shape");
+    }
+}
 static bool use_attn_tail(const lg_hip_model *m, const Layer &y, int rows, int tiles) {
     if (!y.wo_ch || !m->tsync || m->xcd_attn_tail <= 0 || rows > LG_HIP_MAX_ROWS || (m->xcd_attn_tail == 1 && rows < 3)) return false;
     const int slices = (m->E + 1023) / 1024;
@@ -1362,7 +1419,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 cur ^= 1;
                 pend_dout = m->slabs; pend_parts = LG_XCDS; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
             } else {
-            GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq };
+            const bool dn_m = mfma && m->down_m && y.wdn_m;       // ffn_down on the matrix cores: the activations as 80-dword blocks
+            GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq, dn_m ? 2 : 0 };
             if (!ffn_rows_done) rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
@@ -1371,6 +1429,11 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             else
                 LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, LG_GEGLU_FIELDS(LG_XA, a) 0);
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
+            if (dn_m) {
+                DownMArgs dm{ y.wdn_m, (const uint32_t *)m->gq, m->dout, E, y.nff, m->down_m == 1 ? m->dmsync : nullptr, m->ctl, 1 << 16 };
+                launch_down_m<M>(lx, dm);
+                pend_parts = dm.sync ? 1 : 4;
+            } else
             // (the rows kernel adds four slabs; the fused rows + PLE gate kernel of verify blocks takes whole sums)
             pend_parts = launch_mm<M, false>(lx, KC_DOWN, d, !m->ple && m->down_kq);
             pend_dout = m->dout; pend_w = y.post_ffw; pend_os = m->ple ? nullptr : y.out_scale;
@@ -1466,7 +1529,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1506,6 +1569,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
+    else if (!strcmp(name, "down_m")) m->down_m = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "xcd_attn_tail")) m->xcd_attn_tail = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "merge_o")) m->merge_o = value < 0 ? 0 : value > 2 ? 2 : value;
     else if (!strcmp(name, "merge_o_slices")) m->merge_o_slices = value < 0 ? 0 : value;
@@ -1637,7 +1701,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
@@ -2394,6 +2458,64 @@ extern "C" int lg_hip_xcd_handover(int set_mode, int sel, int n, int store_scope
 // ---- the XCD-partitioned feed-forward half on its own (tests, timing) ------------------------------
 // x_out = x + rmsnorm(dout) * w_post; h = rmsnorm(x_out) * w_pre; act = gelu(gate . q8(h)) * (up . q8(h));
 // out = down . q8(act): lg_k_ffn_xcd on host data, the 8 slabs added here in tree order.
+extern "C" int lg_hip_down_m(const float *act, const void *down, int rows, int E, int FF, int join, float *out, int repeats, float *kernel_ms) {
+    if (!act || !down || !out) return fail(-1, "down_m: null argument");
+    const DownMGeo g = lg_down_m_geo(E, FF);
+    if (rows < 4 || rows > LG_HIP_MAX_ROWS || !down_m_shape(g)) return fail(-2, "down_m: rows %d (4..%d), E %d, FF %d: no instantiation for this shape", rows, LG_HIP_MAX_ROWS, E, FF);
+    if (lg_hip_device_count() < 1) return fail(-3, "down_m: no HIP device");
+    Scratch sc;
+    std::vector<uint8_t> stage(256 * g.wg_bytes);
+    uint8_t *dw; float *dx, *dslabs; uint32_t *dq; DownMSync *dsync; StepCtl *ctl;
+    const size_t n = (size_t)rows * E;
+    if (sc.get(&dw, 256 * g.wg_bytes) || sc.get(&dx, (size_t)rows * FF) || sc.get(&dslabs, 4 * n) || sc.get(&dq, (size_t)(FF / 32) * LG_MU_DWORDS) ||
+        sc.get(&dsync, (size_t)1) || sc.get(&ctl, (size_t)1)) return -7;
+    HIP_TRY(hipMemset(dsync, 0, sizeof(DownMSync)));
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    pack_down_m((const uint8_t *)down, g, stage.data());
+    HIP_TRY(hipMemcpy(dw, stage.data(), 256 * g.wg_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dx, act, (size_t)rows * FF * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(dq, 0, (size_t)(FF / 32) * LG_MU_DWORDS * 4));
+    hipStream_t st;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    lg_hip_model shim;
+    shim.stream = st;
+    Launcher lx{ &shim, false };
+    DownMArgs a{ dw, dq, dslabs, E, FF, join ? dsync : nullptr, ctl, 1 << 16 };
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        hipLaunchKernelGGL(lg_k_quant_mu, dim3((rows * (FF / 32) * 8 + LG_WG - 1) / LG_WG), dim3(LG_WG), 0, st, dx, rows, FF, dq);
+        for (int r = 0; r < repeats + 1 && !lx.rc; ++r) {
+            if (r == 1) HIP_TRY(hipEventRecord(e0, st));
+            switch (rows) {
+#define CASE(M) case M: launch_down_m<M>(lx, a); break;
+                CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+            }
+        }
+        if (lx.rc) return lx.rc;
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipGetLastError());
+        float t = 0;
+        if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+        if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+        return 0;
+    };
+    int rc = body();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipStreamDestroy(st);
+    if (rc) return rc;
+    std::vector<float> slabs(4 * n);
+    HIP_TRY(hipMemcpy(slabs.data(), dslabs, 4 * n * 4, hipMemcpyDeviceToHost));
+    StepCtl c;
+    HIP_TRY(hipMemcpy(&c, ctl, sizeof c, hipMemcpyDeviceToHost));
+    { const int erc = step_err("down_m", c.err); if (erc) return erc; }
+    for (size_t i = 0; i < n; ++i) out[i] = join ? slabs[i] : (slabs[i] + slabs[n + i]) + (slabs[2 * n + i] + slabs[3 * n + i]);    // (what the consumer kernel does)
+    return 0;
+}
+
 extern "C" int lg_hip_ffn_xcd(const float *x, const float *dout, const float *w_post, const float *w_pre,
                               const void *gate, const void *up, const void *down, int rows, int E, int FF, float eps,
                               float *x_out, float *act, float *out, int repeats, float *kernel_ms, int flush_mb, int delay_w, int64_t *stamps) {

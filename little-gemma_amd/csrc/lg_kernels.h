@@ -444,8 +444,9 @@ struct GegluArgs {
     int            k, n_ff;
     const int8_t  *q_in;     // verify blocks: unit order (below); wide blocks: lg_q8_off
     int8_t        *gq;       // q8 activation buffer of the result, width n_ff
+    int            gq_units; // lg_k_geglu_m only: 2 = write the 80-dword blocks of the matrix-core kernels (what lg_k_down_m reads) instead of rows
 };
-#define LG_GEGLU_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, n_ff, n_ff, v) X(int8_t *, gq, gq, v)
+#define LG_GEGLU_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const int8_t *, q_in, q_in, v) X(int, k, k, v) X(int, n_ff, n_ff, v) X(int8_t *, gq, gq, v) X(int, gq_units, gq_units, v)
 // Gate/up + GeGLU for verify blocks (M <= 8): a wavefront is 64 weight rows x one of
 // the 8 K segments, so every lane of it multiplies its own weight block with the SAME activation
 // block.  The activations then travel through the scalar cache into SGPRs (loads from the constant
@@ -668,6 +669,13 @@ __global__ __launch_bounds__(512, 2) void lg_k_geglu_m(LG_GEGLU_FIELDS(LG_XP, _)
         const float up = ((u[0] + u[1]) + (u[2] + u[3])) + ((u[4] + u[5]) + (u[6] + u[7]));
         float d; int sum;
         const int q = lg_quant1_32lanes(lg_gelu(gate) * up, &d, &sum);
+        if (a.gq_units == 2) {                                // block t of 80 dwords: row slot j's 32 bytes, dwords in the order 0 1 4 5 2 3 6 7
+            int8_t *blk = a.gq + (size_t)t * (LG_MU_DWORDS * 4);
+            const int dw = i >> 2;
+            blk[(j * 8 + ((dw & 1) | ((dw & 2) << 1) | ((dw & 4) >> 1))) * 4 + (i & 3)] = (int8_t)q;
+            if (i == 0) *(float2 *)(blk + 256 + 8 * j) = make_float2(d, 12582912.0f + (float)(8 * sum));
+            continue;
+        }
         const ActLayout lay = lg_act_layout(a.n_ff);          // order the ffn_down matmul reads
         a.gq[(size_t)j * a.n_ff + lg_act_unit(lay, t * 2 + (i >> 4)) * 16 + (i & 15)] = (int8_t)q;
         if (i == 0) lg_q8_ds<M>(a.gq, a.n_ff)[(size_t)j * (a.n_ff >> 5) + lg_act_block(lay, t)] = make_float2(d, __int_as_float(sum));
@@ -751,6 +759,15 @@ __device__ __forceinline__ void lg_rows_plegate_body(const RowsPleGateArgs &a, i
         const float4 *wr = (const float4 *)a.w_post, *xr = (const float4 *)(a.x + (size_t)j * E), *dr = (const float4 *)(a.dout + (size_t)j * E);
         #pragma unroll
         for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) { xv[v] = xr[t + 256 * v]; dv[v] = dr[t + 256 * v]; wp[v] = wr[t + 256 * v]; }
+        if (a.dparts == 4) {                                  // the top two levels of the tree of an ffn_down cut by K quarter
+            const size_t slab = (size_t)M * nq;
+            #pragma unroll
+            for (int v = 0; v < LG_ROWV; ++v) if (t + 256 * v < nq) {
+                const float4 p1 = dr[slab + t + 256 * v], p2 = dr[2 * slab + t + 256 * v], p3 = dr[3 * slab + t + 256 * v], p0 = dv[v];
+                dv[v] = make_float4((p0.x + p1.x) + (p2.x + p3.x), (p0.y + p1.y) + (p2.y + p3.y),
+                                    (p0.z + p1.z) + (p2.z + p3.z), (p0.w + p1.w) + (p2.w + p3.w));
+            }
+        }
         if (a.dparts == 8) {                                  // the top three levels of the K-segment tree of an ffn_down cut over the 8 XCDs
             const size_t slab = (size_t)M * nq;
             #pragma unroll

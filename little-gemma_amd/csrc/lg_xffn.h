@@ -475,3 +475,177 @@ __global__ __launch_bounds__(LG_XFFN_THREADS) void lg_k_ffn_xcd(LG_XFFN_FIELDS(L
     }
     stamp(10);
 }
+
+// ---------------------------------------------------------------------------------------------------------
+// ffn_down of verify blocks (4..8 rows) on the matrix cores, as a kernel of its own: exactly 256 workgroups whatever the
+// shape.  Workgroup (row group r of 64, K quarter q of 4): its E/64 output rows (one or two operands of up to 32 rows)
+// against the 8 K segments 8q .. 8q+7 of the 32, one segment per wavefront: the serial chain of the segment's blocks,
+// p = fma(xd * dw, (float)dot, p), one v_mfma_i32_32x32x32_i8 per block and operand (A = the block's activations in 8 row
+// slots, B = the rows' nibbles); the 8 chain sums of a row meet in LDS in the adjacent-pair tree (the bottom three
+// levels of the 32-segment tree) and go to slab q of four; the consumer adds (p0 + p1) + (p2 + p3), the top two.
+// Every CU streams the same E * FF * 18 / 32 / 256 bytes of weights (the v_dot4 kernel's cut, 10 rows x all of K per CU,
+// has the same balance but stages all FF activations per workgroup, 64 KB at 5 x 10240, and spends a third of its time
+// on vector instructions); a wavefront reads only its own segment's activation blocks.
+// Weights: per workgroup, segment and operand the stream layout of the kernels above (pairs of blocks: [pair][half h][row n]
+// 8 + 8 nibble bytes, then [pair][row n] the two f16 scales; rows past the operand's count are not stored: their lanes
+// read the last row again).  Activations: the 80-dword blocks that lg_k_geglu_m writes when asked to (gq_units = 2).
+struct DownMGeo {
+    int E, FF, RW, ops, nitd, nitdp, npairs;
+    size_t seg_bytes, wg_bytes;        // stream bytes of a (workgroup, segment): all operands; of a workgroup
+    bool ok;
+};
+__host__ __device__ static inline DownMGeo lg_down_m_geo(int E, int FF) {
+    DownMGeo g{};
+    g.E = E; g.FF = FF;
+    g.ok = E >= 64 && E % 64 == 0 && E <= 4096 && FF % 1024 == 0 && lg_segments(FF) == 32;
+    if (!g.ok) return g;
+    g.RW = E >> 6; g.ops = (g.RW + 31) >> 5;
+    g.nitd = (FF >> 5) >> 5; g.nitdp = (g.nitd + 1) & ~1; g.npairs = g.nitdp >> 1;
+    g.seg_bytes = (size_t)g.RW * g.nitdp * 18;
+    g.wg_bytes = 8 * g.seg_bytes;
+    g.ok = g.ops <= 2;
+    return g;
+}
+// The four workgroups of a row group can also add their slabs themselves: workgroup id = 64 q + r puts them on one XCD
+// (ids that differ by a multiple of 8), quarters 1..3 store their slab, wait for the stores and raise a flag, quarter 0
+// polls the three flags, reads the three slabs from the XCD's L2 and stores (p0 + p1) + (p2 + p3) over its own: slab 0
+// then holds the whole sums and the consumer reads a quarter of the bytes.  Only quarter 0 waits, for workgroups that
+// wait for nobody, so no residency is assumed; the wait is bounded and a flag from another XCD is reported (StepCtl.err).
+struct DownMSync {
+    uint32_t gen[64];            // per row group: launches so far (advanced by its quarter 0 once it has seen the flags)
+    uint32_t flags[64][4];       // (epoch << 4 | XCD id) of the quarter's last arrival, epoch = gen + 1
+};
+struct DownMArgs {
+    const uint8_t *w;        // [256][wg_bytes]
+    const uint32_t *act;     // [FF / 32][80]
+    float *slabs;            // [4][M][E]
+    int E, FF;
+    DownMSync *sync;         // nullptr: leave four slabs to the consumer
+    StepCtl *ctl;
+    int spin_limit;
+};
+#define LG_DOWNM_FIELDS(X, v) X(const uint8_t *, w, w, v) X(const uint32_t *, act, act, v) X(int, E, E, v) X(int, FF, FF, v) X(float *, slabs, slabs, v) \
+    X(DownMSync *, sync, sync, v) X(StepCtl *, ctl, ctl, v) X(int, spin_limit, spin_limit, v)
+// M: rows of the block; OPS: operands of 32 rows per workgroup; NDP: capacity in pairs of blocks of a segment.
+template <int M, int OPS, int NDP>
+__global__ __launch_bounds__(512) void lg_k_down_m(LG_DOWNM_FIELDS(LG_XP, _) int p_end_) {
+    DownMArgs a; LG_DOWNM_FIELDS(LG_XI, a)
+    extern __shared__ __align__(16) unsigned char smem[];
+    const DownMGeo g = lg_down_m_geo(a.E, a.FF);
+    const int wg = blockIdx.x, r = wg & 63, q = wg >> 6;
+    const int t = threadIdx.x, lane = t & 63, n = lane & 31, h = lane >> 5;
+    const int s = __builtin_amdgcn_readfirstlane(t >> 6);             // segment 8q + s
+    const uint32_t gen = a.sync ? a.sync->gen[r] : 0u;
+    unsigned char *la = smem + (size_t)s * g.nitd * (LG_MU_DWORDS * 4);                          // this wavefront's blocks
+    float *red = (float *)(smem + (size_t)8 * g.nitd * (LG_MU_DWORDS * 4));                      // [8 segments][OPS][8 row slots][32]
+    // the activation blocks of the segment first (they come from nearer), then the whole chain's weights
+    const uint4 *src = (const uint4 *)(a.act + (size_t)(8 * q + s) * g.nitd * LG_MU_DWORDS);
+    const int nu = g.nitd * (LG_MU_DWORDS / 4);
+    const int i0 = min(lane, nu - 1), i1 = min(lane + 64, nu - 1), i2 = min(lane + 128, nu - 1), i3 = min(lane + 192, nu - 1), i4 = min(lane + 256, nu - 1);
+    const uint4 t0 = src[i0], t1 = src[i1], t2 = src[i2], t3 = src[i3], t4 = src[i4];                // (up to 16 blocks per segment)
+    __builtin_amdgcn_sched_barrier(0);
+    struct Pair { lg_x4u q; uint32_t sw; };
+    Pair w[OPS][NDP];
+    const uint8_t *sb = a.w + (size_t)(4 * r + q) * g.wg_bytes + (size_t)s * g.seg_bytes;
+    #pragma unroll
+    for (int o = 0; o < OPS; ++o) {
+        const int vr = g.RW - 32 * o < 32 ? g.RW - 32 * o : 32, vc = vr > 0 ? vr : 1, nn = n < vc ? n : vc - 1;
+        const uint8_t *ob = sb + (size_t)32 * o * g.nitdp * 18;
+        #pragma unroll
+        for (int jp = 0; jp < NDP; ++jp) {
+            const int jc = jp < g.npairs ? jp : g.npairs - 1;
+            w[o][jp].q = __builtin_nontemporal_load((const lg_x4u *)(ob + (size_t)((jc * 2 + h) * vc + nn) * 16));
+            w[o][jp].sw = __builtin_nontemporal_load((const uint32_t *)(ob + (size_t)g.nitdp * vc * 16 + (size_t)(jc * vc + nn) * 4));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    ((uint4 *)la)[i0] = t0; ((uint4 *)la)[i1] = t1; ((uint4 *)la)[i2] = t2; ((uint4 *)la)[i3] = t3; ((uint4 *)la)[i4] = t4;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    lg_v16i magic;
+    #pragma unroll
+    for (int i = 0; i < 16; ++i) magic[i] = 0x4B400000;
+    asm volatile("" : "+v"(magic));
+    const int arow = n < 8 ? n : 7;
+    float p[OPS][4];
+    #pragma unroll
+    for (int o = 0; o < OPS; ++o)
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) p[o][i] = 0.0f;
+    #pragma unroll
+    for (int jp = 0; jp < NDP; ++jp) {
+        #pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            if (2 * jp + e < g.nitd) {
+                const XffnAct ac = lg_xffn_act(la + (size_t)(2 * jp + e) * (LG_MU_DWORDS * 4), arow, h);
+                #pragma unroll
+                for (int o = 0; o < OPS; ++o) {
+                    lg_v2u qq; qq.x = e ? w[o][jp].q.z : w[o][jp].q.x; qq.y = e ? w[o][jp].q.w : w[o][jp].q.y;
+                    lg_xffn_step(ac.av, ac.xd, ac.cf, qq, lg_h2f((uint16_t)(e ? w[o][jp].sw >> 16 : w[o][jp].sw)), magic, p[o]);
+                }
+            }
+        }
+    }
+    #pragma unroll
+    for (int o = 0; o < OPS; ++o)
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) red[((size_t)(s * OPS + o) * 8 + 4 * h + i) * 32 + n] = p[o][i];
+    __syncthreads();
+    // the quarter's three levels of the segment tree: one output per thread (M * RW <= 8 * 64)
+    const bool on = t < M * g.RW;
+    const int j = on ? t / g.RW : 0, rr = on ? t - j * g.RW : 0;
+    float *p0 = a.slabs + (size_t)j * a.E + (size_t)r * g.RW + rr;    // this output in slab 0
+    const size_t slab = (size_t)M * a.E;
+    float mine = 0.0f;
+    if (on) {
+        const float *b = red + ((size_t)(rr >> 5) * 8 + j) * 32 + (rr & 31);
+        const size_t sg = (size_t)OPS * 8 * 32;
+        mine = ((b[0] + b[sg]) + (b[2 * sg] + b[3 * sg])) + ((b[4 * sg] + b[5 * sg]) + (b[6 * sg] + b[7 * sg]));
+        p0[q * slab] = mine;
+    }
+    if (!a.sync) return;
+    // ---- the row group's four slabs added here ----
+    const int xcc = lg_xcc_id();
+    const uint32_t epoch = gen + 1;
+    if (q != 0) {
+        lg_wait_vm();
+        __syncthreads();
+        if (t == 0) lg_st_sc<0>(&a.sync->flags[r][q], (epoch << 4) | (uint32_t)xcc);
+        return;
+    }
+    if (s == 0) {
+        int err = LG_XFFN_ERR_WAIT;
+        for (int spins = 0; spins < a.spin_limit; ++spins) {
+            const uint32_t f = (lane >= 1 && lane < 4) ? lg_ld_sc<2>(&a.sync->flags[r][lane]) : ((epoch << 4) | (uint32_t)xcc);
+            const bool there = (int)(((f >> 4) - epoch) << 4) >= 0;
+            if (__all(there)) { err = __any((int)(f & 15) != xcc) ? LG_XFFN_ERR_PLACE : 0; break; }
+        }
+        if (err && lane == 0) atomicOr(&a.ctl->err, err);
+        if (lane == 0) a.sync->gen[r] = epoch;
+    }
+    __syncthreads();
+    if (on) {
+        uint32_t v1, v2, v3;                                          // one round trip for the three
+        asm volatile("global_load_dword %0, %1, off sc1" : "=v"(v1) : "v"(p0 + slab) : "memory");
+        asm volatile("global_load_dword %0, %1, off sc1" : "=v"(v2) : "v"(p0 + 2 * slab) : "memory");
+        asm volatile("global_load_dword %0, %1, off sc1" : "=v"(v3) : "v"(p0 + 3 * slab) : "memory");
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(v1), "+v"(v2), "+v"(v3) :: "memory");
+        *p0 = (mine + __uint_as_float(v1)) + (__uint_as_float(v2) + __uint_as_float(v3));
+    }
+}
+
+// q8 of rows x k floats into the 80-dword blocks (8 lanes per block of 32, one float4 each): what lg_k_geglu_m writes
+// in its epilogue, as a kernel of its own for the isolated entry point of lg_k_down_m.
+__global__ __launch_bounds__(LG_WG) void lg_k_quant_mu(const float *x, int rows, int k, uint32_t *q) {
+    const int g = (blockIdx.x * LG_WG + threadIdx.x) >> 3, l = threadIdx.x & 7, nb = k >> 5;
+    const bool live = g < rows * nb;
+    const float4 h = live ? ((const float4 *)x)[(size_t)g * 8 + l] : make_float4(0, 0, 0, 0);
+    float d; int sum;
+    const uint32_t packed = lg_quant4_8lanes(h, &d, &sum);
+    if (!live) return;
+    const int j = g / nb, b = g - j * nb;
+    uint32_t *blk = q + (size_t)b * LG_MU_DWORDS;
+    blk[j * 8 + ((l & 1) | ((l & 2) << 1) | ((l & 4) >> 1))] = packed;
+    if (l == 0) *(float2 *)(blk + 64 + 2 * j) = make_float2(d, 12582912.0f + (float)(8 * sum));
+}

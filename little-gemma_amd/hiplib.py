@@ -384,6 +384,17 @@ def rows_ple_gate(x, dout, w_post, w_gate_q4_0, ipl, eps=1e-6):
     return dict(x_out=x_out, pq=pq, pd=pd, psum=psum)
 
 
+def down_m(act, down_q4_0, E, repeats=0, join=1):
+    """lg_k_down_m in isolation: act [rows][FF] f32, down_q4_0 raw q4_0 rows [E][FF]; returns out [rows][E], kernel ms."""
+    H = load_hip()
+    rows, FF = act.shape
+    H.lg_hip_down_m.argtypes = [f32p, u8p, C.c_int, C.c_int, C.c_int, C.c_int, f32p, C.c_int, C.POINTER(C.c_float)]
+    out = np.zeros((rows, E), np.float32)
+    ms = C.c_float(0)
+    hip_check(H.lg_hip_down_m(np.ascontiguousarray(act, np.float32), down_q4_0, rows, E, FF, int(join), out, repeats, C.byref(ms)), "down_m")
+    return out, ms.value
+
+
 def ffn_xcd(x, dout, w_post, w_pre, gate_q4_0, up_q4_0, down_q4_0, FF, eps=1e-6, repeats=0, flush_mb=0, want_stamps=False, delay_w=0):
     """The XCD-partitioned feed-forward half of a layer through the C ABI.  x, dout: [rows, E] (rows 4..8); gate / up:
     FF q4_0 rows of E, down: E q4_0 rows of FF.  Returns dict(x_out, act [rows, FF], out [rows, E], kernel_ms)."""

@@ -137,7 +137,7 @@ def test_sampling_hook_replaces_the_argmax(lg, ob, gpu_required, model_path):
         gpu.close(); o.close()
 
 
-@pytest.mark.parametrize("rows,name,over", [(2, "tiny_full", {}), (5, "tiny_full", {}), (6, "tiny", {"n_ff": 5120})])
+@pytest.mark.parametrize("rows,name,over", [(2, "tiny_full", {}), (5, "tiny_full", {}), (6, "tiny", {"n_ff": 5120}), (5, "tiny_full", {"n_ff": 5120})])
 def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, monkeypatch, rows, name, over):
     """The options that pick between kernels for the same arithmetic (row work inside the q/k/v matmul, the
     attention kernels that share a staged tile, the matrix-core lm_head, wide prompt blocks, graph replay, ffn_down
@@ -167,9 +167,11 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
             gpu.close()
 
     base = run()
+    assert np.isfinite(base[2]).all()                  # (a bitwise comparison would call two rows of NaN equal)
     for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
                      ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
                      ("xcd_tail", 0), ("xcd_tail", 2),    # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
+                     ("down_m", 0), ("down_m", 2),                      # (ffn_down of 4..8-row blocks on v_dot4 instead of the matrix cores; the last two cases have the long FFN rows)
                      ("xcd_attn_tail", 0), ("xcd_attn_tail", 2),   # (attention merge + output projection + row work: separate kernels / one launch on one XCD for every width)
                      ("merge_o", 0), ("merge_o", 2), ("merge_o_slices", 8)):   # (attention merge + output projection: separate / one launch for every width / another cut of the rows)
         print(f"rows={rows} option {opt}={val}", flush=True)

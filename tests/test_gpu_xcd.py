@@ -195,3 +195,20 @@ def test_verify_steps_with_the_one_xcd_attention_tail_match_the_oracle(lg, ob, g
             pos += adv; tok = int(out[adv - 1])
     finally:
         gpu.close(); o.close()
+
+
+@pytest.mark.parametrize("rows,E,FF", [(4, 512, 5120), (6, 512, 5120), (5, 2560, 10240), (8, 2560, 10240), (4, 2560, 10240), (5, 3840, 15360), (7, 3840, 15360)])
+def test_down_m_matches_oracle(lg, ob, gpu_required, rows, E, FF):
+    """ffn_down of a verify block on the matrix cores (lg_k_down_m: 64 row groups x 4 K quarters, one K segment per
+    wavefront, four slabs) against the oracle's q4_0 x q8 matmul of the same rows: 8, 40 and 60 output rows per
+    workgroup (one operand, 32 + 8, 32 + 28), segments of 5, 10 and 15 blocks (odd counts are padded)."""
+    rng = np.random.default_rng(rows * 17 + E + FF)
+    act = (rng.normal(0, 1, (rows, FF)) * rng.uniform(0.2, 3.0, (rows, 1))).astype(np.float32)
+    act[0, :96] = 0.0
+    w = random_q4_0(rng, E, FF)
+    print(f"down_m rows={rows} E={E} FF={FF}", flush=True)
+    _, _, _, want, _ = oracle_matmul(ob, w, FF, E, act)
+    for join in (1, 0):       # the row group's workgroups add their slabs themselves (several launches in a row: the flags go on from launch to launch) / the caller does
+        got, ms = lg.hiplib.down_m(act, w, E, repeats=3, join=join)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), join
+        print(f"  join={join}: kernel {1e3 * ms:.2f} us", flush=True)
