@@ -33,7 +33,7 @@ i32a = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
 # WRITE_SIZE counter runs summarised in the file named below (scaled by the copy-kernel calibration given
 # there): reads 29.40 MB for M = 5 (29.27 MB for M = 1), writes 0.15 MB (0.03 MB).  Counters cannot be read
 # from inside this process, so the figure is quoted with its source; shapes without a counter run report null.
-MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.40e6 + 0.15e6, ("e4b", "gate_up_geglu", 1): 29.27e6 + 0.03e6}
+MEASURED_TRAFFIC = {("e4b", "gate_up_geglu", 5): 29.41e6 + 0.07e6, ("e4b", "gate_up_geglu", 1): 29.27e6 + 0.03e6}
 TRAFFIC_SOURCE = "profiles/verify_step_e4b_rows5_hbm_counters.md"
 CTX = 2048
 WORKLOADS = {

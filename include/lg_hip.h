@@ -271,7 +271,7 @@ size_t lg_hip_attention_noalloc_limit(void);
 int    lg_hip_down_m(const float *act, const void *down_q4_0, int rows, int E, int FF, int join, float *out, int repeats, float *kernel_ms);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
-int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 */
+int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 and a multiple of 32 */
 size_t lg_hip_repacked_bytes(int k, int m);
 int    lg_hip_repack_q4_0(const void *src, int k, int m, void *dst);
 

@@ -64,7 +64,9 @@ __device__ __forceinline__ uint16_t lg_ldt2b(__amdgpu_buffer_rsrc_t r, int it, i
 // blocks); the m x k matrix is cut into groups of 64/S rows; tile (group, it) holds, for
 // lane = r*S + c, the 16 nibble bytes and the f16 scale of block c*nit + it of row r of the group.
 // A wavefront reads one tile with one 16-byte load and one 2-byte load per lane.
-__host__ __device__ static inline int lg_segments(int k) { return (k >> 5) > 128 ? 32 : 8; }
+// (a long row whose block count is no multiple of 32, like the 2 x 3840 inputs of a draft head's pre-projection on a 3840-wide
+// backbone, keeps 8 segments)
+__host__ __device__ static inline int lg_segments(int k) { return ((k >> 5) > 128 && ((k >> 5) & 31) == 0) ? 32 : 8; }
 
 // Order of a q8 activation row in memory.  A matmul lane (row r, segment c) needs, at step `it`,
 // block c*nit + it of the row; lanes c = 0..S-1 therefore want blocks that lie nit apart.  Rows are

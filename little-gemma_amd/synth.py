@@ -63,7 +63,10 @@ def assistant_for(target, **over):
     reading the global cache (when the target's head sizes differ; otherwise all read the sliding one)."""
     hd_l = target["head_dim"]
     hd_g = target.get("head_dim_full") or hd_l
-    spec = dict(ASSISTANT_DEFAULTS, n_backbone=target["n_embd"], n_vocab=target["n_vocab"], head_dim_swa=hd_l,
+    # the head's query heads share the target's KV heads: a multiple of their number
+    nkv = target["n_head_kv"]
+    heads = -(-ASSISTANT_DEFAULTS["n_head"] // nkv) * nkv
+    spec = dict(ASSISTANT_DEFAULTS, n_head=heads, n_backbone=target["n_embd"], n_vocab=target["n_vocab"], head_dim_swa=hd_l,
                 head_dim_full=hd_g, n_ff=1024, qk_norm=target.get("qk_norm", 0.0),
                 rope_base=target.get("rope_base", 1e6), rope_base_swa=target.get("rope_base_swa", 1e4))
     spec.update(over)

@@ -100,7 +100,7 @@ int32_t lgo_block_dot(const unsigned char *blk, const int8_t *q) {
 
 /* K segments of this build's matmul order: 8, or 32 for rows of more than 128 blocks (the
  * wide ffn_down rows), so that every lane's serial chain stays short. */
-int lgo_segments(int k) { return k / 32 > 128 ? 32 : 8; }
+int lgo_segments(int k) { return (k / 32 > 128 && (k / 32) % 32 == 0) ? 32 : 8; }
 
 /* ---- q4_0 x q8 matmul.  out[j*m+i] = sum_b (xd[j][b]*dw[i][b]) * dot(i,j,b)
  * (src/cuda/model-cuda-i8.cu:813-903); `order` picks how the f32 terms are summed. */

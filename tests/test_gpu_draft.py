@@ -250,3 +250,35 @@ def test_e4b_shape_head(lg, ob, gpu_required, model_path, model_dir):
         assert got2 == want2
     finally:
         gpu.mtp_close(t); gpu.close(); od.close(); o.close()
+
+
+def test_12b_width_head(lg, ob, gpu_required, model_path, model_dir):
+    """A head on a 3840-wide backbone (the 12B width on 6 layers): its pre-projection has 7680 inputs, 240 blocks,
+    which is above 128 and no multiple of 32, so it runs in 8 K segments; draft and chained draft against the oracle."""
+    path, spec = model_path("g12b", n_layer=6, n_ff=3072, n_vocab=8192)
+    head = write_head(lg, model_dir, "g12b_w", spec)
+    assert lg.hiplib.load_hip().lg_hip_segments(2 * spec["n_embd"]) == 8
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(1, spec["n_vocab"], 12).astype(np.int32)
+    o = ob.Oracle(path)
+    od = o.mtp_open(head)
+    gpu = lg.hiplib.HipBackend(path, 64, max_rows=5)
+    t = gpu.mtp_open(head)
+    try:
+        kv = o.kv_new(64, ob.I8)
+        o.prefill(kv, prompt[:-1], 0, ob.I8)
+        gpu.prefill(prompt[:-1], 0)
+        pos = len(prompt) - 1
+        best, _, hid = o.forward(kv, int(prompt[-1]), pos, ob.I8, want_logits=True, want_hidden=True)
+        assert gpu.forward_next(int(prompt[-1]), pos) == best
+        print("3840-wide head: draft + chained draft", flush=True)
+        want, wh, _ = od.draft(kv, best, pos + 1, hid, ob.I8)
+        got = gpu.mtp_draft(t, best, pos + 1)
+        assert np.array_equal(bits(gpu.mtp_hidden(t, od.info["n_inner"])), bits(wh))
+        assert got == want
+        want2, wh2, _ = od.draft(kv, want, pos + 2, od.post(wh, ob.I8), ob.I8)
+        got2 = gpu.mtp_draft(t, got, pos + 2, chain=True)
+        assert np.array_equal(bits(gpu.mtp_hidden(t, od.info["n_inner"])), bits(wh2))
+        assert got2 == want2
+    finally:
+        gpu.mtp_close(t); gpu.close(); od.close(); o.close()
