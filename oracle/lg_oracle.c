@@ -98,8 +98,9 @@ int32_t lgo_block_dot(const unsigned char *blk, const int8_t *q) {
     return acc;
 }
 
-/* K segments of this build's matmul order: 8, or 32 for rows of more than 128 blocks (the
- * wide ffn_down rows), so that every lane's serial chain stays short. */
+/* K segments of this build's matmul order: 8, or 32 for rows of more than 128 blocks whose
+ * block count 32 divides (the wide ffn_down rows), so that every lane's serial chain stays
+ * short; a row of 240 blocks (two 3840-wide halves) stays at 8 segments of 30. */
 int lgo_segments(int k) { return (k / 32 > 128 && (k / 32) % 32 == 0) ? 32 : 8; }
 
 /* ---- q4_0 x q8 matmul.  out[j*m+i] = sum_b (xd[j][b]*dw[i][b]) * dot(i,j,b)
