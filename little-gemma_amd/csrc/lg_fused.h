@@ -495,8 +495,13 @@ __global__ __launch_bounds__(320, 2) void lg_k_mm_kq(LG_MM_FIELDS(LG_XP, _) int 
 // ---------------------------------------------------------------------------------------------
 // Attention tiles of a verify block for layers with many tiles (long global contexts, wide sliding windows):
 // one workgroup per (tile, kv head) serves ALL rows of the block against one staged K/V tile, where lg_k_attn
-// runs a workgroup per row and stages every tile once per row.  The queries arrive normed and rotated
-// (lg_k_qkv_post has run and has written the block's K/V rows to the cache).  Same arithmetic and order as
+// runs a workgroup per row and stages every tile once per row.  FQ = false: the queries arrive normed and rotated
+// (lg_k_qkv_post has run and has written the block's K/V rows to the cache).  FQ = true: the kernel does that work
+// itself from the raw projections, one launch less per layer: every workgroup norms and rotates the M*G queries of
+// its kv head (a wavefront per query, written in the staged order), and the one workgroup whose tile holds rows of
+// the block builds those K/V rows straight into its LDS tile and stores them to the cache (K row r by wavefront
+// r % 4, V row r by wavefront 3 - r % 4; the ring has spare rows, so no row another workgroup reads is overwritten).
+// Same arithmetic and order as
 // lg_k_attn: score = (a0+a1)+(a2+a3) over four fma chains, tile max / exp / 32-lane tree sum, value accumulation
 // over the slots ascending; the partials go to the same slots and lg_k_attn_merge finishes them.
 //
@@ -526,11 +531,11 @@ template <int HD>
 struct AttnRowsGeo {
     static constexpr int KSD = HD / 2 + 4;                    // dwords per staged K row (16-byte reads of 8 slots cover all banks)
     static constexpr int VST = HD + 8;                        // halves per staged V row
-    static size_t bytes(int units) {
-        return (size_t)units * HD * 4 + (size_t)32 * KSD * 4 + (size_t)32 * VST * 2 + (size_t)units * 32 * 4;
+    static size_t bytes(int units, bool fq = false) {         // fq: a vector of staging per wavefront for the rotary
+        return (size_t)units * HD * 4 + (size_t)32 * KSD * 4 + (size_t)32 * VST * 2 + (size_t)units * 32 * 4 + (fq ? (size_t)(LG_WG / 64) * HD * 4 : 0);
     }
 };
-template <int M, int HD>
+template <int M, int HD, bool FQ = false>
 __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int tp, LG_ATTN_FIELDS(LG_XP, _) int p_end_) {
     AttnArgs a; LG_ATTN_FIELDS(LG_XI, a)
     using Geo = AttnRowsGeo<HD>;
@@ -540,9 +545,12 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int 
     uint32_t *kt = (uint32_t *)(qs + (size_t)units * HD);     // [32][KSD]: row sl = [hf][HD/4 dwords]
     uint16_t *vt = (uint16_t *)(kt + 32 * Geo::KSD);          // [32][VST]
     float *es = (float *)(vt + 32 * Geo::VST);                // [unit][32]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float *hv = es + (size_t)units * 32;                      // FQ: [wavefront][HD] staging of the rotary
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int kvh = blockIdx.y;
     const int pos0 = ctl->pos + a.pos_off, plast = pos0 + M - 1;
+    // FQ: positions tnew..plast are rows of the block itself (none when the layer reads another layer's cache)
+    const int tnew = (FQ && a.kcw) ? ctl->pos : 0x7FFFFFFF;
     const int start0 = lg_win_start(pos0, a.window), first = start0 >> 5, last = plast >> 5;
     const int b0 = blockIdx.x * tp;                           // tiles first + b0 .. first + b0 + tp - 1
     if (first + b0 > last) return;                            // no row of the block has keys here
@@ -568,6 +576,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int 
         for (int u = 0; u < KL; ++u) {
             const int idx = (int)threadIdx.x + u * LG_WG, row = idx / U4R, u4 = idx - row * U4R;
             if (32 * U4R < LG_WG && idx >= 32 * U4R) continue;
+            if (FQ && t0 + row >= tnew && row <= shi) continue;               // a row of the block: built below, not in the cache yet
             const uint32_t mk = (row >= slo && row <= shi) ? 0xFFFFFFFFu : 0u;
             uint32_t *d = kt + row * Geo::KSD + 2 * u4;
             *(uint2 *)d = make_uint2(kq[u].x & mk, kq[u].z & mk);             // chains 0,1 of two groups of four dims
@@ -575,8 +584,87 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int 
             *(uint4 *)(vt + row * Geo::VST + u4 * 8) = make_uint4(vq[u].x & mk, vq[u].y & mk, vq[u].z & mk, vq[u].w & mk);
         }
     };
+    constexpr int JOBS = 2 * ((M + 3) / 4);                   // FQ: K and V rows of the block one wavefront may have to build
+    constexpr int QBATCH = 4;                                 // FQ: queries one wavefront prepares at a time
+    HeadVec<1> hj[FQ ? JOBS : 1], hq[FQ ? QBATCH : 1], wk, wq;
+    RopeVals<1> rv;
+    if constexpr (FQ) {
+        // What the preparation reads is requested ahead of the tile (loads return in order): the block's projections
+        // come from the cache levels, the tile from memory, so the queries are prepared while the tile is on its way.
+        // Raw rows of the block that fall into this workgroup's tiles are requested here too and used when their tile
+        // is staged.
+        const int tlo = (first + b0) << 5, thi = ((first + b0 + tp) << 5) - 1;
+        rv = lg_rope_load<1>(a.rope_tab, a.rope_ff, HD);
+        wq = lg_head_load<1>(a.q_norm, HD);
+        #pragma unroll
+        for (int b = 0; b < QBATCH; ++b) {                    // unit u = (row j, head g), by wavefront u % 4
+            const int u = wave + b * (LG_WG / 64) < units ? wave + b * (LG_WG / 64) : min(wave, units - 1), j = u / G, g = u - j * G;
+            hq[b] = lg_head_load<1>(a.qkv + (size_t)j * a.ld + (size_t)(kvh * G + g) * HD, HD);
+        }
+        const bool any = tnew <= plast && plast >= tlo && tnew <= thi;
+        wk = lg_head_load<1>(any ? a.k_norm : a.q_norm, HD);  // (no K rows to build: k_norm may not exist)
+        #pragma unroll
+        for (int u = 0; u < JOBS; ++u) {                      // first half of the slots: K rows wave, wave+4; second half: V rows 3-wave, 7-wave
+            const bool isv = u >= JOBS / 2;
+            const int r = (isv ? 3 - wave : wave) + 4 * (u % (JOBS / 2)), t = tnew + r;
+            if (any && r < M && t >= tlo && t <= thi) hj[u] = lg_head_load<1>(a.qkv + (size_t)r * a.ld + (isv ? a.v_off : a.k_off) + (size_t)kvh * HD, HD);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     fetch(b0);
-    {   // the queries, once per workgroup (their loads follow the first tile's before any store)
+    if constexpr (FQ) {
+        __builtin_amdgcn_sched_barrier(0);
+        // a batch in stages, so that the sums and the rotary of its queries overlap: norms of all, each into its own
+        // slot of qs in natural order; all rotary pairs read back; then the slots rewritten in the staged order
+        // (a unit past the last repeats the batch's first one, a slot of this wavefront, and stores nothing)
+        auto unit_of = [&](int base, int b) { return base + b * (LG_WG / 64) < units ? base + b * (LG_WG / 64) : base; };
+        for (int base = wave; base < units; base += QBATCH * (LG_WG / 64)) {
+            if (base != wave) {
+                #pragma unroll
+                for (int b = 0; b < QBATCH; ++b) {
+                    const int u = unit_of(base, b), j = u / G, g = u - j * G;
+                    hq[b] = lg_head_load<1>(a.qkv + (size_t)j * a.ld + (size_t)(kvh * G + g) * HD, HD);
+                }
+            }
+            HeadVec<1> nq[QBATCH];
+            #pragma unroll
+            for (int b = 0; b < QBATCH; ++b) nq[b] = lg_head_norm<1>(hq[b], wq, true, HD, a.eps);
+            #pragma unroll
+            for (int b = 0; b < QBATCH; ++b)
+                if (4 * lane < HD) *(float4 *)(qs + (size_t)unit_of(base, b) * HD + 4 * lane) = nq[b].x[0];
+            lg_wave_lds_sync();
+            float lo[QBATCH][2], hi[QBATCH][2];
+            #pragma unroll
+            for (int b = 0; b < QBATCH; ++b) {
+                const int u = unit_of(base, b), j = u / G;
+                const float *vec = qs + (size_t)u * HD;
+                #pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int p = min(lane + 64 * i, HD / 2 - 1);
+                    const float ang = (float)(ctl->pos + j) * rv.tab[i] / rv.ff[i];
+                    float sn, cs;
+                    lg_sincosf(ang, &sn, &cs);
+                    const float x0 = vec[p], x1 = vec[p + HD / 2];
+                    lo[b][i] = x0 * cs - x1 * sn; hi[b][i] = x0 * sn + x1 * cs;
+                }
+            }
+            lg_wave_lds_sync();                               // (LDS serves a wavefront in order: every read above is ahead of the stores below)
+            #pragma unroll
+            for (int b = 0; b < QBATCH; ++b) {
+                const int u = base + b * (LG_WG / 64);
+                float *qd = qs + (size_t)unit_of(base, b) * HD;
+                #pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int p = lane + 64 * i, p1 = p + HD / 2;
+                    if (u >= units || p >= HD / 2) continue;
+                    // element i sits at hf = (i%4)/2, 2*(i/4) + i%2
+                    qd[((p & 3) >> 1) * (HD / 2) + 2 * (p >> 2) + (p & 1)] = lo[b][i];
+                    qd[((p1 & 3) >> 1) * (HD / 2) + 2 * (p1 >> 2) + (p1 & 1)] = hi[b][i];
+                }
+            }
+            lg_wave_lds_sync();
+        }
+    } else {   // the queries, once per workgroup (their loads follow the first tile's before any store)
         constexpr int QB = 4;                                 // float4 of query per thread and pass
         const int nq4 = units * (HD / 4);
         for (int base = 0; base < nq4; base += QB * LG_WG) {
@@ -604,6 +692,44 @@ __global__ __launch_bounds__(LG_WG) void lg_k_attn_rows(const StepCtl *ctl, int 
         const int bx = b0 + i, n = first + bx, t0 = n << 5;
         if (n > last) break;
         if (i > 0) __syncthreads();                           // the previous tile has been read by every wavefront
+        if constexpr (FQ) {                                   // rows of the block in this tile: built while the tile is on its way (stash leaves their slots alone)
+            if (tnew <= plast && tnew <= t0 + 31 && plast >= t0) {            // this tile holds rows of the block
+                float *vec = hv + (size_t)wave * HD;
+                HeadVec<1> nr[JOBS];
+                int slj[JOBS];
+                #pragma unroll
+                for (int u = 0; u < JOBS; ++u) {              // the norms of all of them first: their sums overlap
+                    const bool isv = u >= JOBS / 2;
+                    const int r = (isv ? 3 - wave : wave) + 4 * (u % (JOBS / 2)), sl = tnew + r - t0;
+                    slj[u] = (r < M && sl >= 0 && sl <= 31) ? sl : -1;
+                    if (slj[u] >= 0) nr[u] = lg_head_norm<1>(hj[u], wk, !isv, HD, a.eps);
+                }
+                #pragma unroll
+                for (int u = 0; u < JOBS; ++u) {
+                    const bool isv = u >= JOBS / 2;
+                    const int sl = slj[u], t = t0 + sl;
+                    if (sl < 0) continue;
+                    const size_t coff = (size_t)(t % a.seq) * a.kv_dim + (size_t)kvh * HD;
+                    if (isv) {                                // V: no rotary, straight from the registers
+                        if (4 * lane < HD) {
+                            const uint2 h4 = make_uint2((uint32_t)lg_f2h(nr[u].x[0].x) | ((uint32_t)lg_f2h(nr[u].x[0].y) << 16),
+                                                        (uint32_t)lg_f2h(nr[u].x[0].z) | ((uint32_t)lg_f2h(nr[u].x[0].w) << 16));
+                            *(uint2 *)(vt + sl * Geo::VST + 4 * lane) = h4;
+                            *(uint2 *)(a.vcw + coff + 4 * lane) = h4;
+                        }
+                    } else {
+                        uint16_t *row = (uint16_t *)(kt + sl * Geo::KSD), *crow = a.kcw + coff;
+                        lg_head_rope<1>(nr[u], HD, t, rv, vec, [&](int p, float lo, float hi) {
+                            const int p1 = p + HD / 2;        // dims 4g, 4g+1 in dword g of the first half, 4g+2, 4g+3 of the second
+                            const uint16_t hl = lg_f2h(lo), hh = lg_f2h(hi);
+                            row[2 * (((p & 3) >> 1) * (HD / 4) + (p >> 2)) + (p & 1)] = hl;
+                            row[2 * (((p1 & 3) >> 1) * (HD / 4) + (p1 >> 2)) + (p1 & 1)] = hh;
+                            crow[p] = hl; crow[p1] = hh;
+                        });
+                    }
+                }
+            }
+        }
         stash(bx);
         __syncthreads();
         if (i + 1 < tp && n + 1 <= last) fetch(bx + 1);

@@ -205,7 +205,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, head_mfma = 1, down_kq = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, attn_rows_fq = 1, head_mfma = 1, down_kq = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
     int down_m = 1;                          // option: ffn_down of 4..8-row blocks on the matrix cores (lg_k_down_m): 1 = the row group's four workgroups add
@@ -279,6 +279,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
     if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
+    if (const char *e = getenv("LG_HIP_ATTN_ROWS_FQ")) m->attn_rows_fq = atoi(e) != 0;   // 0: lg_k_qkv_post ahead of lg_k_attn_rows
     if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&m->stream2, hipStreamNonBlocking);
@@ -1331,7 +1332,8 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
             // ... unless the layer has so many (tile, kv head) pairs that one workgroup per pair can serve all rows of
             // the block against one staged tile (long global contexts, wide windows): the rows then arrive prepared
-            if (rows_shared(L)) fused_post = false;
+            // (that kernel prepares them itself unless the option says otherwise)
+            if (rows_shared(L) && !m->attn_rows_fq) fused_post = false;
             QkvPostArgs p{};
             p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
             p.H = H; p.nkv = y.nkv; p.hd = y.hd;
@@ -1361,9 +1363,17 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             } else
             if (shared) {
                 if constexpr (M > 1 && M <= LG_HIP_MAX_ROWS) {
-                    const size_t lds = y.hd == 256 ? AttnRowsGeo<256>::bytes(M * G) : y.hd == 128 ? AttnRowsGeo<128>::bytes(M * G) : AttnRowsGeo<64>::bytes(M * G);
+                    const size_t lds = y.hd == 256 ? AttnRowsGeo<256>::bytes(M * G, fused_post) : y.hd == 128 ? AttnRowsGeo<128>::bytes(M * G, fused_post) : AttnRowsGeo<64>::bytes(M * G, fused_post);
                     const int tp = attention_rows_tp(tiles, y.nkv);
                     const dim3 grid((tiles + tp - 1) / tp, y.nkv);
+                    if (fused_post) {
+                        a.qkv = m->qkv; a.ld = y.qkv_m; a.k_off = y.k_off; a.v_off = y.v_off;
+                        a.q_norm = y.q_norm; a.k_norm = y.k_norm; a.rope_tab = y.rope_tab; a.rope_ff = y.rope_ff;
+                        a.kcw = y.owns ? kv->k[L] : nullptr; a.vcw = y.owns ? kv->v[L] : nullptr; a.eps = m->eps;
+                        if (y.hd == 256)      LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 256, true>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+                        else if (y.hd == 128) LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 128, true>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+                        else                  LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 64, true>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
+                    } else
                     if (y.hd == 256)      LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 256>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
                     else if (y.hd == 128) LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 128>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
                     else                  LAUNCH(KC_ATTN, (lg_k_attn_rows<M, 64>), grid, dim3(LG_WG), lds, m->ctl, tp, LG_ATTN_FIELDS(LG_XA, a) 0);
@@ -1529,7 +1539,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1566,6 +1576,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "wide_prefill")) m->wide_prefill = value != 0;
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
+    else if (!strcmp(name, "attn_rows_fq")) m->attn_rows_fq = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
@@ -1701,7 +1712,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;

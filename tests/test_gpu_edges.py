@@ -168,7 +168,7 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
 
     base = run()
     assert np.isfinite(base[2]).all()                  # (a bitwise comparison would call two rows of NaN equal)
-    for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
+    for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("attn_rows_fq", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
                      ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
                      ("xcd_tail", 0), ("xcd_tail", 2),    # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
                      ("down_m", 0), ("down_m", 2),                      # (ffn_down of 4..8-row blocks on v_dot4 instead of the matrix cores; the last two cases have the long FFN rows)
@@ -180,3 +180,66 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
         assert np.array_equal(got[2].view(np.uint32), base[2].view(np.uint32)), opt
         for a, b in zip(got[3], base[3]):
             assert np.array_equal(a, b), opt
+
+
+@pytest.mark.parametrize("rows", [5, 8, 2])
+def test_shared_tile_attention_prepares_its_own_rows(lg, ob, gpu_required, model_path, rows):
+    """Layers with 256 and more (tile, kv head) pairs take the attention kernel that stages a tile once for all rows
+    of a block; it norms and rotates the block's queries and builds the block's K/V rows itself.  A 2048-key window
+    on 4 KV heads (66 tiles) and a global context of the same length, layers that own their cache and layers that
+    read another's, a block that starts 2 positions before a tile boundary (its rows fall into two tiles) and the
+    next one after it: against the oracle, and bit for bit against the same step with lg_k_qkv_post run ahead
+    (attn_rows_fq = 0) and with the per-row attention kernel (attn_rows = 0)."""
+    path, spec = model_path("tiny_full", n_head_kv=4, sliding_window=2048)
+    V, E = spec["n_vocab"], spec["n_embd"]
+    rng = np.random.default_rng(90 + rows)
+    n0 = 65 * 32 + 30
+    prompt = rng.integers(0, V, n0).astype(np.int32)
+    first, tail = int(rng.integers(0, V)), rng.integers(0, V, rows).astype(np.int32)
+    ctx = n0 + 64
+
+    def run(**opts):
+        gpu = lg.hiplib.HipBackend(path, ctx, max_rows=8)
+        try:
+            for k, v in opts.items():
+                gpu.set_option(k, v)
+            gpu.set_option("store_logits", 1)
+            gpu.prefill(prompt, 0)
+            chain = [first]                                # the model's own continuation: a block that is accepted whole
+            for i in range(rows):
+                chain.append(gpu.forward_next(chain[-1], n0 + i))
+            blocks = [np.array(chain[:rows], np.int32), np.concatenate(([chain[rows]], tail[1:])).astype(np.int32)]
+            res, pos = [], n0
+            for blk in blocks:
+                adv, out = gpu.forward_spec(blk, pos)
+                res.append((adv, out.copy(), np.stack([gpu.logits_row(j, V) for j in range(rows)]), gpu.last_hidden(E).copy(), blk))
+                pos += adv
+            cache = [gpu.kv_read(L, w).copy() for L in range(spec["n_layer"] - spec["shared_kv_layers"]) for w in (0, 1)]
+            return res, cache
+        finally:
+            gpu.close()
+
+    print(f"rows={rows}: default kernels", flush=True)
+    base, base_cache = run()
+    assert all(np.isfinite(r[2]).all() for r in base)
+    assert base[0][0] == rows                              # verify == plain decode
+    o = ob.Oracle(path)
+    try:
+        kv = o.kv_new(ctx, ob.I8)
+        o.prefill(kv, prompt, 0, ob.I8)
+        pos = n0
+        for adv, out, _, hid, blk in base:
+            oadv, oout, ohid = o.forward_spec(kv, blk, pos, ob.I8, want_hidden=True)
+            assert oadv == adv and oout[:adv].tolist() == out[:adv].tolist()
+            assert np.array_equal(hid.view(np.uint32), ohid.view(np.uint32))
+            pos += adv
+    finally:
+        o.close()
+    for opts in ({"attn_rows_fq": 0}, {"attn_rows": 0}):
+        print(f"rows={rows}: {opts}", flush=True)
+        got, cache = run(**opts)
+        for g, b in zip(got, base):
+            assert g[0] == b[0] and np.array_equal(g[1], b[1]), opts
+            assert np.array_equal(g[2].view(np.uint32), b[2].view(np.uint32)), opts
+        for a, b in zip(cache, base_cache):
+            assert np.array_equal(a, b), opts
