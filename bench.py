@@ -206,7 +206,8 @@ def xcd_handover():
 
 
 def tail_stamps(rows, model_dir):
-    """Phase boundaries of the one-XCD layer tail (lg_k_ple_tail) at the E4B shape: device wall-clock stamps of every
+    """Phase boundaries of the one-XCD layer tail (lg_k_ple_tail; lg_k_ple_tail_s from 5 rows on, where every stamp is its
+    workgroup's first wavefront's) at the E4B shape: device wall-clock stamps of every
     unit of the last layer's launch, over four verify steps from a 600-position cache."""
     path = os.path.join(model_dir, f"lg_bench_e4b_seed{lg.synth.E4B['seed']}.gguf")
     if not os.path.exists(path):
@@ -225,7 +226,8 @@ def tail_stamps(rows, model_dir):
         st = gpu.tail_stamps().astype(np.int64)
         s = st[st[:, 0] >= st[:, 0].max() - 1000]          # the units of the latest launch (older launches of other widths left theirs: > 10 us back)
         rel = (s - s[:, 0].min()) * 10                     # ns (100 MHz clock)
-        steps.append({n: {"first_unit_ns": int(rel[:, i][s[:, i] != 0].min()), "last_unit_ns": int(rel[:, i][s[:, i] != 0].max())}
+        seen = s >= s[:, :1]                               # (a unit that leaves after the projection keeps older stamps in its last slots)
+        steps.append({n: {"first_unit_ns": int(rel[:, i][seen[:, i]].min()), "last_unit_ns": int(rel[:, i][seen[:, i]].max())}
                       for i, n in enumerate(names)})
         units = int(s.shape[0])
     gpu.close()

@@ -205,7 +205,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, attn_rows_fq = 1, head_mfma = 1, down_kq = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, attn_rows_fq = 1, head_mfma = 1, down_kq = 1, tail_spread = 1;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
     int down_m = 1;                          // option: ffn_down of 4..8-row blocks on the matrix cores (lg_k_down_m): 1 = the row group's four workgroups add
@@ -222,6 +222,7 @@ struct lg_hip_model {
     // the per-layer-input block and the next row work as one launch on one XCD (lg_xtail.h)
     int xcd_tail = 1;                        // option: 0 off, 1 for blocks that do not fold the row work into q/k/v, 2 for every verify block
     XtailSync *tsync = nullptr;
+    float *tgf = nullptr;                    // [LG_HIP_MAX_ROWS][ple] gated values of lg_k_ple_tail_s
     unsigned long long *tstamps = nullptr;   // [LG_XTAIL_UNITS][8] phase stamps of the last such launch (option xcd_tail_stamps)
     int tail_stamps = 0;
     bool xffn_built = false;                 // streams and working memory exist
@@ -279,7 +280,8 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_GRAPH")) m->use_graph = 0;       // un-captured launches (kernel tracing tools)
     if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
-    if (const char *e = getenv("LG_HIP_ATTN_ROWS_FQ")) m->attn_rows_fq = atoi(e) != 0;   // 0: lg_k_qkv_post ahead of lg_k_attn_rows
+    if (const char *e = getenv("LG_HIP_ATTN_ROWS_FQ")) m->attn_rows_fq = atoi(e) != 0;
+    if (const char *e = getenv("LG_HIP_XCD_TAIL_SPREAD")) m->tail_spread = atoi(e) != 0;   // 0: the one-XCD tail of 5..8-row blocks as ple/32 x rows units   // 0: lg_k_qkv_post ahead of lg_k_attn_rows
     if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&m->stream2, hipStreamNonBlocking);
@@ -725,7 +727,8 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
         return -7;
     if (m->ple && dev_alloc(m, &m->eq, R * E * 5 / 4 + (size_t)12 * E)) return -7;
     if (!m->target) {                        // hand-over state of the one-XCD kernels (lg_xtail.h)
-        if (dev_alloc(m, &m->tsync, (size_t)1) || dev_alloc(m, &m->tstamps, (size_t)2 * LG_XTAIL_UNITS * 8)) return -7;
+        if (dev_alloc(m, &m->tsync, (size_t)1) || dev_alloc(m, &m->tstamps, (size_t)2 * LG_XTAIL_UNITS * 8) ||
+            dev_alloc(m, &m->tgf, (size_t)LG_HIP_MAX_ROWS * (m->ple > 0 ? m->ple : 1))) return -7;
         HIP_TRY(hipMemset(m->tstamps, 0, (size_t)2 * LG_XTAIL_UNITS * 8 * 8));
         HIP_TRY(hipMemset(m->tsync, 0, sizeof(XtailSync)));
         HIP_TRY(hipMemset(m->aq, 0, R * max_qd * 5 / 4));       // (row slots past the block are read as operand rows of the matrix cores)
@@ -1164,6 +1167,34 @@ static void launch_attn_tail(Launcher &lx, const XattnTailArgs &a) {
 
 template <int M>
 static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
+    if constexpr (M >= 5 && M <= LG_HIP_MAX_ROWS) {
+        // 5..8 rows: the form whose units fit one per CU (row j by 32 / M workgroups of 8 wavefronts)
+        lg_hip_model *m = lx.m;
+        const int E = a.r.g.k, W = M * (32 / M), G = (E / 8 + 8 * W - 1) / (8 * W);
+        if (m->tail_spread && a.gf && a.r.g.ple == 256 && G >= 1 && G <= 3) {
+            const size_t lds = (size_t)E * 5 / 4 + (size_t)M * a.r.g.ple * 5 / 4;
+            const dim3 grid(LG_XCDS * W);
+            static int fits[4] = { 0, 0, 0, 0 };              // per G: 0 unknown, 1 yes, -1 no (asked once, outside any capture)
+            if (!fits[G]) {
+                int per_cu = 0;
+                hipError_t e = hipErrorInvalidValue;
+                switch (G) {
+                    case 1: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail_s<M, 1>, 512, lds); break;
+                    case 2: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail_s<M, 2>, 512, lds); break;
+                    case 3: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lg_k_ple_tail_s<M, 3>, 512, lds); break;
+                }
+                fits[G] = (e == hipSuccess && per_cu * LG_XCD_WGS >= W) ? 1 : -1;
+            }
+            if (fits[G] > 0) {
+                switch (G) {
+                    case 1: LAUNCH(KC_TAIL, (lg_k_ple_tail_s<M, 1>), grid, dim3(512), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+                    case 2: LAUNCH(KC_TAIL, (lg_k_ple_tail_s<M, 2>), grid, dim3(512), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+                    case 3: LAUNCH(KC_TAIL, (lg_k_ple_tail_s<M, 3>), grid, dim3(512), lds, m->ctl, LG_XTAIL_FIELDS(LG_XA, a) 0); break;
+                }
+                return;
+            }
+        }
+    }
     if constexpr (M <= LG_HIP_MAX_ROWS) {
         lg_hip_model *m = lx.m;
         const int E = a.r.g.k, U = (a.r.g.ple / 32) * M;
@@ -1475,6 +1506,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 f.x_out = m->x[cur ^ 1]; f.h_out = last ? m->hidden_rows : nullptr;
                 f.q = m->hq; f.q_units = last && head_m ? 2 : 0;
                 f.sync = m->tsync; f.spin_limit = 1 << 16; f.stamps = m->tail_stamps ? m->tstamps : nullptr;
+                f.gf = m->tgf;
                 launch_ple_tail<M>(lx, f);
                 cur ^= 1;
                 pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
@@ -1539,7 +1571,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_spread ? "" : "n") + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1577,6 +1609,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else if (!strcmp(name, "attn_rows_fq")) m->attn_rows_fq = value != 0;
+    else if (!strcmp(name, "xcd_tail_spread")) m->tail_spread = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
@@ -1712,7 +1745,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->tail_spread ? "" : "n") + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;
