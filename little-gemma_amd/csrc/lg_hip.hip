@@ -1363,8 +1363,13 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             fused_post = M <= LG_HIP_MAX_ROWS && (pos_off == 0 || !y.owns);    // (a draft head's layers own no cache: queries only)
             // ... unless the layer has so many (tile, kv head) pairs that one workgroup per pair can serve all rows of
             // the block against one staged tile (long global contexts, wide windows): the rows then arrive prepared
-            // (that kernel prepares them itself unless the option says otherwise)
-            if (rows_shared(L) && !m->attn_rows_fq) fused_post = false;
+            // (that kernel prepares them itself while it has few workgroups: each of them repeats the preparation of its kv
+            // head's queries, which a layer of many hundred workgroups pays for with more than the launch it saves: 12B
+            // shape, 8192 keys, 688 workgroups: 36 -> 43 us; a 1024-key window, 272 workgroups: 11 -> 13.5 us against 4.2)
+            if (rows_shared(L)) {
+                const int tiles = layer_tiles(L), tp = attention_rows_tp(tiles, y.nkv);
+                if (!m->attn_rows_fq || ((tiles + tp - 1) / tp) * y.nkv > 2 * cu_count()) fused_post = false;
+            }
             QkvPostArgs p{};
             p.qkv = m->qkv; p.ld = y.qkv_m; p.k_off = y.k_off; p.v_off = y.v_off;
             p.H = H; p.nkv = y.nkv; p.hd = y.hd;
