@@ -341,7 +341,7 @@ def main():
     value = timed_tokens / (ms * 1e-3)
 
     # per-kernel-class device time of one step (un-captured, start/stop events filled in by each launch)
-    prof = gpu.profile_step(blocks[0], ctx, repeats=3)
+    prof = gpu.profile_step(blocks[0], ctx, repeats=10)
     step_bytes = sum(c["bytes"] for c in prof)
     # the roofline kernel: the class that moves the most bytes per step (gate/up + GeGLU: 47% of them at the E4B
     # shape).  By device time several classes of a layer are within 10% of it (kernel_classes lists them all).
