@@ -22,6 +22,7 @@
 #include "lg_xcd.h"
 #include "lg_xffn.h"
 #include "lg_xtail.h"
+#include "lg_xrg.h"
 
 static_assert(LG_HIP_MAX_ROWS == LG_HIP_MAX_ROWS_DEV, "row limits must agree");
 #define LG_FUSE_ROWS_MAX 2         // widest block whose q/k/v matmul does the preceding row work itself
@@ -205,7 +206,7 @@ struct lg_hip_model {
     int sched_cap = 0, sched_steps = 0, sched_rows = 0, sched_pos0 = 0, sched_loaded = 0;
     int32_t *pin = nullptr;            // pinned host staging
     int last_rows = 0, last_adv = 0;
-    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, attn_rows_fq = 1, head_mfma = 1, down_kq = 1, tail_spread = 1;
+    int store_logits = 0, use_graph = 1, wide_prefill = 1, fuse_rows = 1, attn_rows = 1, attn_rows_fq = 1, head_mfma = 1, down_kq = 1, tail_spread = 1, rows_geglu = 0;
     // the feed-forward half of a layer as one XCD-partitioned launch (lg_xffn.h): built when the shape and the chip fit
     int xcd_ffn = 0;                         // option: use it (verify blocks of 4..8 rows)
     int down_m = 1;                          // option: ffn_down of 4..8-row blocks on the matrix cores (lg_k_down_m): 1 = the row group's four workgroups add
@@ -223,6 +224,7 @@ struct lg_hip_model {
     int xcd_tail = 1;                        // option: 0 off, 1 for blocks that do not fold the row work into q/k/v, 2 for every verify block
     XtailSync *tsync = nullptr;
     float *tgf = nullptr;                    // [LG_HIP_MAX_ROWS][ple] gated values of lg_k_ple_tail_s
+    RgSync *rgsync = nullptr;                // flags and epoch base of lg_k_rows_geglu
     unsigned long long *tstamps = nullptr;   // [LG_XTAIL_UNITS][8] phase stamps of the last such launch (option xcd_tail_stamps)
     int tail_stamps = 0;
     bool xffn_built = false;                 // streams and working memory exist
@@ -281,6 +283,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_FUSE")) m->fuse_rows = 0;        // row work in kernels of its own (comparison runs)
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
     if (const char *e = getenv("LG_HIP_ATTN_ROWS_FQ")) m->attn_rows_fq = atoi(e) != 0;
+    if (const char *e = getenv("LG_HIP_ROWS_GEGLU")) m->rows_geglu = atoi(e) != 0;     // the row work ahead of gate/up inside the gate/up launch
     if (const char *e = getenv("LG_HIP_XCD_TAIL_SPREAD")) m->tail_spread = atoi(e) != 0;   // 0: the one-XCD tail of 5..8-row blocks as ple/32 x rows units   // 0: lg_k_qkv_post ahead of lg_k_attn_rows
     if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
@@ -731,6 +734,8 @@ extern "C" int lg_hip_model_commit(lg_hip_model *m, int max_rows) {
             dev_alloc(m, &m->tgf, (size_t)LG_HIP_MAX_ROWS * (m->ple > 0 ? m->ple : 1))) return -7;
         HIP_TRY(hipMemset(m->tstamps, 0, (size_t)2 * LG_XTAIL_UNITS * 8 * 8));
         HIP_TRY(hipMemset(m->tsync, 0, sizeof(XtailSync)));
+        if (dev_alloc(m, &m->rgsync, (size_t)1)) return -7;
+        HIP_TRY(hipMemset(m->rgsync, 0, sizeof(RgSync)));
         HIP_TRY(hipMemset(m->aq, 0, R * max_qd * 5 / 4));       // (row slots past the block are read as operand rows of the matrix cores)
         if (getenv("LG_HIP_XCD_TAIL")) m->xcd_tail = atoi(getenv("LG_HIP_XCD_TAIL"));
     }
@@ -1258,8 +1263,10 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
         RowArgs s{};
         s.q_units = M <= LG_HIP_MAX_ROWS ? units : 0;
         s.E = E; s.eps = m->eps; s.toks = m->sched; s.q = q_out ? q_out : m->hq;
-        if (!have_x) { s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E); }
-        else s.x = m->x[cur];
+        if (!have_x) {
+            s.emb = m->emb; s.emb_seg = lg_segments(E); s.emb_nit = E / 32 / s.emb_seg; s.emb_scale = sqrtf((float)E);
+            if (m->rgsync) s.bump = &m->rgsync->base;          // the step's first kernel: a new range of epochs for lg_k_rows_geglu
+        } else s.x = m->x[cur];
         s.dout = pend_dout; s.w_post = pend_w; s.os = pend_os; s.dparts = pend_parts;
         s.w_pre = w_pre; s.h_out = h_out;
         if (pend_dout || !have_x) s.x_out = m->x[cur ^ 1];
@@ -1467,6 +1474,27 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
             } else {
             const bool dn_m = mfma && m->down_m && y.wdn_m;       // ffn_down on the matrix cores: the activations as 80-dword blocks
             GegluArgs a{ y.wgu, E, y.nff, m->hq, m->gq, dn_m ? 2 : 0 };
+            bool rows_in_geglu = false;
+            if constexpr (mfma) {
+                // the row work as the first workgroups of the gate/up launch, whose other workgroups request their weights
+                // while it runs (lg_xrg.h); shapes whose K segment of E/256 tiles has a build
+                const int slices = (E + 1023) / 1024;
+                if (m->rows_geglu && m->rgsync && !ffn_rows_done && have_x && pend_dout && !pend_os && (pend_parts == 1 || pend_parts == 4) && (E == 2560 || E == 3840 || E == 512) &&
+                    M * slices <= LG_RG_MAXP && L < LG_RG_STEP - 1) {
+                    RowsGegluArgs f{ m->x[cur], pend_dout, pend_w, y.ffn_norm, m->x[cur ^ 1], m->hq, E, pend_parts, slices, m->eps,
+                                     y.wgu, y.nff, m->gq, dn_m ? 2 : 0, m->rgsync, L, 1 << 16, m->tail_stamps ? m->tstamps + LG_XTAIL_UNITS * 8 : nullptr };
+                    const dim3 grid(M * slices + y.nff / 32);
+                    const size_t lds = (size_t)(E / 32) * LG_MU_DWORDS * 4;
+                    if (E == 512)  LAUNCH(KC_GATEUP, (lg_k_rows_geglu<M, 2>), grid, dim3(512), lds, m->ctl, LG_RG_FIELDS(LG_XA, f) 0);
+                    else if (E == 2560) LAUNCH(KC_GATEUP, (lg_k_rows_geglu<M, 10>), grid, dim3(512), lds, m->ctl, LG_RG_FIELDS(LG_XA, f) 0);
+                    else           LAUNCH(KC_GATEUP, (lg_k_rows_geglu<M, 15>), grid, dim3(512), lds, m->ctl, LG_RG_FIELDS(LG_XA, f) 0);
+                    cur ^= 1;
+                    pend_dout = pend_w = pend_os = nullptr; pend_parts = 1;
+                    rows_in_geglu = true;
+                }
+            }
+            if (rows_in_geglu) {
+            } else {
             if (!ffn_rows_done) rows(y.ffn_norm, nullptr, mfma ? 2 : 1);
             if constexpr (M > LG_HIP_MAX_ROWS)
                 LAUNCH(KC_GATEUP, (lg_k_mm_geglu_wide<M>), dim3(y.nff / 32, (M + LG_WIDE - 1) / LG_WIDE), dim3(LG_WIDE_WG), MfmaGeo::lds_bytes, a, M);
@@ -1474,6 +1502,7 @@ static int enqueue_step(lg_hip_model *m, lg_hip_kv *kv, bool with_head, bool dry
                 LAUNCH(KC_GATEUP, (lg_k_geglu_m<M>), dim3(y.nff / 32), dim3(512), (size_t)(E / 32) * LG_MU_DWORDS * 4, LG_GEGLU_FIELDS(LG_XA, a) 0);
             else
                 LAUNCH(KC_GATEUP, (lg_k_geglu_t<M>), dim3(y.nff / 32), dim3(512), 0, LG_GEGLU_FIELDS(LG_XA, a) 0);
+            }
             MmArgs d{ y.wdown, y.nff, E, m->dout, m->gq, nullptr };
             if (dn_m) {
                 DownMArgs dm{ y.wdn_m, (const uint32_t *)m->gq, m->dout, E, y.nff, m->down_m == 1 ? m->dmsync : nullptr, m->ctl, 1 << 16 };
@@ -1576,7 +1605,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_spread ? "" : "n") + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_spread ? "" : "n") + (m->rows_geglu ? "g" : "") + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1615,6 +1644,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else if (!strcmp(name, "attn_rows_fq")) m->attn_rows_fq = value != 0;
     else if (!strcmp(name, "xcd_tail_spread")) m->tail_spread = value != 0;
+    else if (!strcmp(name, "rows_geglu")) m->rows_geglu = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
     else if (!strcmp(name, "fork_ple")) m->fork_ple = value != 0;
@@ -1750,7 +1780,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->tail_spread ? "" : "n") + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->tail_spread ? "" : "n") + (t->rows_geglu ? "g" : "") + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;

@@ -53,8 +53,10 @@ struct RowArgs {
     int            E;
     float          eps;
     int            slices;   // workgroups per row (gridDim.y): as an argument it arrives with the others, the launch dimensions need a load of their own
+    uint32_t      *bump;     // nullptr, or a counter that the launch advances by LG_RG_STEP (the step's first kernel: epochs of lg_k_rows_geglu)
 };
-#define LG_ROW_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(int, E, E, v) X(int, dparts, dparts, v) X(int, slices, slices, v) X(const float *, os, os, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(float, eps, eps, v) X(const uint8_t *, emb, emb, v) X(const int32_t *, toks, toks, v) X(int, emb_nit, emb_nit, v) X(int, emb_seg, emb_seg, v) X(float, emb_scale, emb_scale, v)
+#define LG_RG_STEP 256       // more than the launches of a step
+#define LG_ROW_FIELDS(X, v) X(const float *, x, x, v) X(const float *, dout, dout, v) X(const float *, w_post, w_post, v) X(const float *, w_pre, w_pre, v) X(int, E, E, v) X(int, dparts, dparts, v) X(int, slices, slices, v) X(const float *, os, os, v) X(float *, x_out, x_out, v) X(float *, h_out, h_out, v) X(int8_t *, q, q, v) X(int, q_units, q_units, v) X(float, eps, eps, v) X(const uint8_t *, emb, emb, v) X(const int32_t *, toks, toks, v) X(int, emb_nit, emb_nit, v) X(int, emb_seg, emb_seg, v) X(float, emb_scale, emb_scale, v) X(uint32_t *, bump, bump, v)
 
 // Sum over the 256 lanes of a workgroup in adjacent-pair tree order; every thread gets the result.
 // `scratch4` must not be in use by an earlier call that other wavefronts may still be reading: each call
@@ -101,6 +103,7 @@ __global__ __launch_bounds__(LG_WG) void lg_k_rows(const StepCtl *ctl, LG_ROW_FI
     // float4 t + 256*y of each lane (the tail of the kernel is the longest part of it and splits freely)
     const int vs = s.slices > 1 ? (int)blockIdx.y : -1;
     const int E = s.E, nq = E >> 2;                          // float4 quads in a row; thread t owns quads t + 256*v
+    if (s.bump && blockIdx.x == 0 && blockIdx.y == 0 && t == 0) *s.bump += LG_RG_STEP;
     float4 xv[LG_ROWV], dv[LG_ROWV], wpost[LG_ROWV], wpre[LG_ROWV];
     // issue every load up front: one memory round trip for the whole row
     if (!s.x) {                                              // (rows that are token lookups have no residual yet)

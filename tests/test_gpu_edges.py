@@ -170,7 +170,7 @@ def test_every_kernel_choice_gives_the_same_bits(lg, gpu_required, model_path, m
     assert np.isfinite(base[2]).all()                  # (a bitwise comparison would call two rows of NaN equal)
     for opt, val in (("fuse_rows", 0), ("attn_rows", 0), ("attn_rows_fq", 0), ("head_mfma", 0), ("wide_prefill", 0), ("use_graph", 0), ("down_kq", 0),
                      ("fork_ple", 1),        # (the per-layer inputs as a second branch of the graph: off by default)
-                     ("xcd_tail", 0), ("xcd_tail", 2), ("xcd_tail_spread", 0),   # (the per-layer-input block as separate kernels / as one launch also for narrow blocks)
+                     ("xcd_tail", 0), ("xcd_tail", 2), ("xcd_tail_spread", 0), ("rows_geglu", 1),   # (the row work ahead of gate/up inside the gate/up launch: off by default; the per-layer-input block as separate kernels / as one launch also for narrow blocks)
                      ("down_m", 0), ("down_m", 2),                      # (ffn_down of 4..8-row blocks on v_dot4 instead of the matrix cores; the last two cases have the long FFN rows)
                      ("xcd_attn_tail", 0), ("xcd_attn_tail", 2),   # (attention merge + output projection + row work: separate kernels / one launch on one XCD for every width)
                      ("merge_o", 0), ("merge_o", 2), ("merge_o_slices", 8)):   # (attention merge + output projection: separate / one launch for every width / another cut of the rows)

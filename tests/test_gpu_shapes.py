@@ -22,15 +22,18 @@ def seed_both(gpu, o, ob, okv, ctx, seed):
         gpu.kv_write(L, 0, k.view(np.uint16)); gpu.kv_write(L, 1, v.view(np.uint16))
 
 
-@pytest.mark.parametrize("name,ctx,steps,rows", [("e4b", 2048, 3, 5), ("g12b", 8192, 2, 5),
-                                                 ("e4b", 2048, 2, 4), ("g12b", 8192, 2, 4)])    # 4 rows: the reference's "block-4" (include/model.h:179-186)
-def test_verify_steps_at_full_shape(lg, ob, gpu_required, model_path, name, ctx, steps, rows):
+@pytest.mark.parametrize("name,ctx,steps,rows,opts", [("e4b", 2048, 3, 5, {}), ("g12b", 8192, 2, 5, {}),
+                                                      ("e4b", 2048, 2, 4, {}), ("g12b", 8192, 2, 4, {}),    # 4 rows: the reference's "block-4" (include/model.h:179-186)
+                                                      ("e4b", 2048, 2, 5, {"rows_geglu": 1}), ("g12b", 8192, 2, 5, {"rows_geglu": 1})])   # (the row work inside the gate/up launch: an option, off by default)
+def test_verify_steps_at_full_shape(lg, ob, gpu_required, model_path, name, ctx, steps, rows, opts):
     path, spec = model_path(name)
     V = spec["n_vocab"]
     print(f"{name}: model written, loading", flush=True)
     o = ob.Oracle(path)
     gpu = lg.hiplib.HipBackend(path, ctx + 64, max_rows=rows)
     try:
+        for k, v in opts.items():
+            gpu.set_option(k, v)
         okv = o.kv_new(ctx + 64, ob.I8)
         seed_both(gpu, o, ob, okv, ctx, 11)
         lg.hiplib.hip_check(gpu.H.lg_hip_kv_save_prefix(gpu.dkv, ctx), "save")
