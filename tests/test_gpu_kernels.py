@@ -1,4 +1,4 @@
-"""GPU parity of the parts, through the C ABI: the isolated q4_0 x q8 matmul (BASELINE config 2),
+"""GPU parity of the parts, through the C ABI: the isolated q4_0 x q8 matmul (the benchmark list's isolated-matmul configuration),
 the decode attention over an f16 ring (config 3), the row kernel (add-norm, norm, q8), the fused
 rows + per-layer gate kernel and the per-layer inputs.  Bar: int32 block dots and every integer
 bit-exact; f32 outputs bit-identical to the oracle in this build's summation order and within

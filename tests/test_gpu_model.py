@@ -20,7 +20,7 @@ def greedy_oracle(ob, o, prompt, n_gen, max_seq):
 
 @pytest.mark.parametrize("name", ["tiny", "tiny_full", "tiny_full_f32"])
 def test_config1_greedy_run_matches_oracle(lg, ob, gpu_required, model_path, golden, name):
-    """BASELINE config 1: 128-token uniform-random prompt, then 64 greedy tokens, against the int8-class oracle.
+    """The smallest benchmark configuration: 128-token uniform-random prompt, then 64 greedy tokens, against the int8-class oracle.
     The prompt is the one of the committed reference fixture; the comparison with the reference's own f32 run
     is test_gpu_against_the_reference_fixture_teacher_forced below."""
     path, spec = model_path(name)

@@ -1,4 +1,4 @@
-"""GPU parity at the benchmark shapes (BASELINE configs 4 and 5): a seeded 2048 / 8192-position cache,
+"""GPU parity at the benchmark shapes (the E4B and 12B configurations of the benchmark list): a seeded 2048 / 8192-position cache,
 K=4 draft blocks, the GPU against the int8-class oracle on the same GGUF and cache contents, plus the
 size-independent properties (verify == decode, accept counts as planted, fully accepting run)."""
 import numpy as np
