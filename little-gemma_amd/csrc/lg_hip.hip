@@ -1108,9 +1108,12 @@ static void launch_xffn(Launcher &lx, const XffnArgs &a, int cls) {
 static bool use_ple_tail(const lg_hip_model *m, int rows) {
     if (!m->ple || !m->tsync || m->xcd_tail <= 0 || m->target || rows < 1 || rows > LG_HIP_MAX_ROWS) return false;
     if (m->ple != 256 || (m->ple / 32) * rows > LG_XTAIL_UNITS || m->E % 256 || m->E > 4096 || (m->E + 1023) / 1024 > m->ple / 32) return false;
-    if (m->xcd_tail == 1 && rows <= LG_FUSE_ROWS_MAX && m->fuse_rows) return false;
     const int U = (m->ple / 32) * rows;
-    if ((m->E / 8 + 4 * U - 1) / (4 * U) > 4) return false;       // (few rows of a wide model: too few wavefronts for the projection)
+    const bool spread = m->tail_spread && (rows >= 5 || rows <= 2);   // (lg_k_ple_tail_s: 8 wavefronts per unit, enough of them at every width)
+    // blocks of one and two rows: with lg_k_ple_tail_s the tail beats folding the next layer's row work into its q/k/v
+    // matmul (E4B shape: 1.994 -> 1.958 ms at one row, 2.127 -> 2.032 at two); with lg_k_ple_tail alone it does not
+    if (m->xcd_tail == 1 && rows <= LG_FUSE_ROWS_MAX && m->fuse_rows && !spread) return false;
+    if (!spread && (m->E / 8 + 4 * U - 1) / (4 * U) > 4) return false;       // (few rows of a wide model: too few wavefronts for the projection)
     return cu_count() == LG_XCDS * LG_XCD_WGS;
 }
 // Slices of the E output rows per (head, row) of lg_k_merge_o: a divisor of the E/64 chunks that leaves at most two
@@ -1172,8 +1175,9 @@ static void launch_attn_tail(Launcher &lx, const XattnTailArgs &a) {
 
 template <int M>
 static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
-    if constexpr (M >= 5 && M <= LG_HIP_MAX_ROWS) {
-        // 5..8 rows: the form whose units fit one per CU (row j by 32 / M workgroups of 8 wavefronts)
+    if constexpr ((M >= 5 || M <= 2) && M <= LG_HIP_MAX_ROWS) {
+        // 5..8 rows: the form whose units fit one per CU (row j by 32 / M workgroups of 8 wavefronts); 1 and 2 rows: the
+        // form that has enough wavefronts for the projection
         lg_hip_model *m = lx.m;
         const int E = a.r.g.k, W = M * (32 / M), G = (E / 8 + 8 * W - 1) / (8 * W);
         if (m->tail_spread && a.gf && a.r.g.ple == 256 && G >= 1 && G <= 3) {
