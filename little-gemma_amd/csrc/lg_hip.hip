@@ -284,7 +284,7 @@ extern "C" int lg_hip_model_create(const struct lg_hip_config *c, int device, lg
     if (getenv("LG_HIP_NO_ATTN_ROWS")) m->attn_rows = 0;   // attention tiles per row everywhere (comparison runs)
     if (const char *e = getenv("LG_HIP_ATTN_ROWS_FQ")) m->attn_rows_fq = atoi(e) != 0;
     if (const char *e = getenv("LG_HIP_ROWS_GEGLU")) m->rows_geglu = atoi(e) != 0;     // the row work ahead of gate/up inside the gate/up launch
-    if (const char *e = getenv("LG_HIP_XCD_TAIL_SPREAD")) m->tail_spread = atoi(e) != 0;   // 0: the one-XCD tail of 5..8-row blocks as ple/32 x rows units   // 0: lg_k_qkv_post ahead of lg_k_attn_rows
+    if (const char *e = getenv("LG_HIP_XCD_TAIL_SPREAD")) m->tail_spread = atoi(e);   // 0: the one-XCD tail as ple/32 x rows units of 4 wavefronts only; 2: as 8-wavefront units at 3 and 4 rows too
     if (getenv("LG_HIP_NO_DOWN_KQ")) m->down_kq = 0;       // ffn_down of verify blocks by whole rows everywhere (comparison runs)
     hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&m->stream2, hipStreamNonBlocking);
@@ -1175,12 +1175,12 @@ static void launch_attn_tail(Launcher &lx, const XattnTailArgs &a) {
 
 template <int M>
 static void launch_ple_tail(Launcher &lx, const XtailArgs &a) {
-    if constexpr ((M >= 5 || M <= 2) && M <= LG_HIP_MAX_ROWS) {
+    if constexpr (M <= LG_HIP_MAX_ROWS) {
         // 5..8 rows: the form whose units fit one per CU (row j by 32 / M workgroups of 8 wavefronts); 1 and 2 rows: the
         // form that has enough wavefronts for the projection
         lg_hip_model *m = lx.m;
         const int E = a.r.g.k, W = M * (32 / M), G = (E / 8 + 8 * W - 1) / (8 * W);
-        if (m->tail_spread && a.gf && a.r.g.ple == 256 && G >= 1 && G <= 3) {
+        if ((m->tail_spread == 2 || (m->tail_spread && (M >= 5 || M <= 2))) && a.gf && a.r.g.ple == 256 && G >= 1 && G <= 3) {
             const size_t lds = (size_t)E * 5 / 4 + (size_t)M * a.r.g.ple * 5 / 4;
             const dim3 grid(LG_XCDS * W);
             static int fits[4] = { 0, 0, 0, 0 };              // per G: 0 unknown, 1 yes, -1 no (asked once, outside any capture)
@@ -1609,7 +1609,7 @@ static int enqueue_step_rows(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with
 // launch one step, through a captured graph when enabled
 static int launch_step(lg_hip_model *m, lg_hip_kv *kv, int rows, bool with_head) {
     if (!m->use_graph || m->prof.on) return enqueue_step_rows(m, kv, rows, with_head);
-    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_spread ? "" : "n") + (m->rows_geglu ? "g" : "") + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
+    const std::string key = "kv" + std::to_string(kv->id) + ":" + std::to_string(rows) + (with_head ? "h" : "p") + (m->store_logits ? "l" : "") + (m->draft_chain ? "c" : "") + (m->fuse_rows ? "" : "u") + (m->attn_rows ? "" : "r") + (m->attn_rows_fq ? "" : "q") + (m->head_mfma ? "" : "s") + (m->down_kq ? "" : "d") + (m->xcd_ffn ? "x" + std::to_string(m->xffn_delay) : "") + (m->fork_ple ? "" : "f") + "t" + std::to_string(m->xcd_tail) + (m->tail_spread == 1 ? "" : m->tail_spread ? "N" : "n") + (m->rows_geglu ? "g" : "") + (m->tail_stamps ? "s" : "") + (m->down_m ? "D" + std::to_string(m->down_m) : "") + "a" + std::to_string(m->xcd_attn_tail) + "o" + std::to_string(m->merge_o) + "." + std::to_string(m->merge_o_slices);
     auto it = m->graphs.find(key);
     if (it == m->graphs.end()) {
         hipGraph_t graph = nullptr;
@@ -1647,7 +1647,7 @@ extern "C" int lg_hip_set_option(lg_hip_model *m, const char *name, int value) {
     else if (!strcmp(name, "fuse_rows")) m->fuse_rows = value != 0;
     else if (!strcmp(name, "attn_rows")) m->attn_rows = value != 0;
     else if (!strcmp(name, "attn_rows_fq")) m->attn_rows_fq = value != 0;
-    else if (!strcmp(name, "xcd_tail_spread")) m->tail_spread = value != 0;
+    else if (!strcmp(name, "xcd_tail_spread")) m->tail_spread = value;
     else if (!strcmp(name, "rows_geglu")) m->rows_geglu = value != 0;
     else if (!strcmp(name, "down_kq")) m->down_kq = value != 0;
     else if (!strcmp(name, "xcd_ffn")) m->xcd_ffn = value != 0 && m->xffn_built;
@@ -1784,7 +1784,7 @@ extern "C" int lg_hip_mtp_rounds(lg_hip_model *d, lg_hip_kv *kv, int token, int 
     if (!t->use_graph || t->prof.on || d->prof.on) {
         for (int r = 0; r < n_rounds; ++r) if ((rc = enqueue_round(d, kv, rows, false))) return rc;
     } else {
-        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->tail_spread ? "" : "n") + (t->rows_geglu ? "g" : "") + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
+        const std::string key = "kv" + std::to_string(kv->id) + ":round" + std::to_string(rows) + (t->store_logits ? "l" : "") + (d->store_logits ? "L" : "") + (t->fuse_rows ? "" : "u") + (d->fuse_rows ? "" : "v") + (t->attn_rows ? "" : "r") + (t->attn_rows_fq ? "" : "q") + (t->head_mfma ? "" : "s") + (t->down_kq ? "" : "d") + (t->xcd_ffn ? "x" : "") + (t->fork_ple ? "" : "f") + "t" + std::to_string(t->xcd_tail) + (t->tail_spread == 1 ? "" : t->tail_spread ? "N" : "n") + (t->rows_geglu ? "g" : "") + (t->down_m ? "D" + std::to_string(t->down_m) : "") + "a" + std::to_string(t->xcd_attn_tail) + "o" + std::to_string(t->merge_o) + "." + std::to_string(t->merge_o_slices);
         auto it = d->graphs.find(key);            // kept by the head: the graph dies with it or with the cache
         if (it == d->graphs.end()) {
             hipGraph_t graph = nullptr;

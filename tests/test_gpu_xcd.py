@@ -107,11 +107,11 @@ def test_verify_steps_with_the_xcd_ffn_kernel_match_the_oracle(lg, ob, gpu_requi
 
 
 @pytest.mark.parametrize("name", ["tiny_full"])
-@pytest.mark.parametrize("rows,spread", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (7, 1), (8, 1), (5, 0), (6, 0), (8, 0)])
+@pytest.mark.parametrize("rows,spread", [(1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (7, 1), (8, 1), (5, 0), (6, 0), (8, 0), (3, 2), (4, 2)])
 def test_verify_steps_with_the_one_xcd_tail_match_the_oracle(lg, ob, gpu_required, model_path, name, rows, spread):
     """Whole verify steps with the per-layer-input block and the following row work as one launch on one XCD
     (lg_k_ple_tail, option xcd_tail = 2: for every block width, also the ones that otherwise fold the row work into
-    the q/k/v matmul; from 5 rows on lg_k_ple_tail_s, whose units fit one per CU, unless xcd_tail_spread = 0): accept counts, successors, every row's logits and the kept hidden state are the oracle's, bit
+    the q/k/v matmul; at 1, 2 and 5..8 rows lg_k_ple_tail_s, units of 8 wavefronts that fit one per CU, unless xcd_tail_spread = 0; at 3 and 4 rows too with xcd_tail_spread = 2): accept counts, successors, every row's logits and the kept hidden state are the oracle's, bit
     for bit, over several steps (each step is one launch per layer: the hand-over flags of a launch start from what the
     launch before left), and the same as with the separate kernels."""
     path, spec = model_path(name)
