@@ -269,6 +269,13 @@ size_t lg_hip_attention_noalloc_limit(void);
  * or here as the consumer kernel adds them (join = 0).  The model path is ffn_down of
  * src/cuda/model-cuda-i8.cu's q4_0 x q8 matmul; this entry exists for parity tests and timing. */
 int    lg_hip_down_m(const float *act, const void *down_q4_0, int rows, int E, int FF, int join, float *out, int repeats, float *kernel_ms);
+/* Gate/up + GeGLU of a verify block in isolation: x = rows x E floats (quantized to q8 on the device by the step's row
+ * kernel), gate / up = FF plain q4_0 rows of E each; aq / ad / asum receive the q8 of gelu(gate) * up in natural order
+ * (rows x FF values, rows x FF/32 scales and sums).  1..3 rows run lg_k_geglu_t, 4..8 rows lg_k_geglu_m.  The model path
+ * is the FFN of src/cuda/model-cuda.cuh:663-698 on src/cuda/model-cuda-i8.cu's q4_0 x q8 matmul; this entry exists for
+ * parity tests and timing. */
+int    lg_hip_gate_up_geglu(const float *x, const void *gate_q4_0, const void *up_q4_0, int rows, int E, int FF,
+                            int8_t *aq, float *ad, int32_t *asum, int repeats, float *kernel_ms);
 /* Host-side weight layout transform used by lg_hip_model_tensor, exposed for tests: q4_0 rows
  * -> the kernels' tile order.  dst needs lg_hip_repacked_bytes(k, m) bytes. */
 int    lg_hip_segments(int k);      /* K segments of a row of k weights: 8, or 32 when k/32 > 128 and a multiple of 32 */

@@ -12,6 +12,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <thread>
 #include <vector>
 
@@ -2597,6 +2598,76 @@ extern "C" int lg_hip_down_m(const float *act, const void *down, int rows, int E
     { const int erc = step_err("down_m", c.err); if (erc) return erc; }
     for (size_t i = 0; i < n; ++i) out[i] = join ? slabs[i] : (slabs[i] + slabs[n + i]) + (slabs[2 * n + i] + slabs[3 * n + i]);    // (what the consumer kernel does)
     return 0;
+}
+
+// Gate/up + GeGLU of a verify block in isolation (tests): `rows` float rows of E are quantized as the step's row
+// kernel does it (the q8 order of the kernel that follows: lg_k_geglu_t for 1..3 rows, lg_k_geglu_m for 4..8), then
+// the kernel runs on gate / up (FF plain q4_0 rows of E each) and the q8 of gelu(gate) * up comes back in natural order.
+extern "C" int lg_hip_gate_up_geglu(const float *x, const void *gate, const void *up, int rows, int E, int FF,
+                                    int8_t *aq, float *ad, int32_t *asum, int repeats, float *kernel_ms) {
+    if (!x || !gate || !up) return fail(-1, "gate_up_geglu: null argument");
+    if (rows < 1 || rows > LG_HIP_MAX_ROWS || E < 256 || E % 256 || E > 4096 || FF < 32 || FF % 32 || lg_segments(E) != 8)
+        return fail(-2, "gate_up_geglu: rows %d (1..%d), E %d (a multiple of 256 up to 4096), FF %d (a multiple of 32)", rows, LG_HIP_MAX_ROWS, E, FF);
+    if (lg_hip_device_count() < 1) return fail(-3, "gate_up_geglu: no HIP device");
+    const size_t rb = (size_t)(E / 32) * 18;
+    std::vector<const uint8_t *> wrows;
+    for (int t = 0; t < FF / 32; ++t) {
+        for (int r = 0; r < 32; ++r) wrows.push_back((const uint8_t *)gate + ((size_t)t * 32 + r) * rb);
+        for (int r = 0; r < 32; ++r) wrows.push_back((const uint8_t *)up + ((size_t)t * 32 + r) * rb);
+    }
+    std::vector<uint8_t> stage(lg_hip_repacked_bytes(E, 2 * FF));
+    if (stage.empty()) return fail(-2, "gate_up_geglu: cannot tile a %d x %d matrix", 2 * FF, E);
+    repack_rowblocks(wrows.data(), E, 2 * FF, stage.data());
+    Scratch sc;
+    uint8_t *dw; float *dx; int8_t *dq, *dgq; StepCtl *ctl;
+    const size_t qbytes = (size_t)(E / 32) * LG_MU_DWORDS * 4 + (size_t)rows * E * 2;     // (room for either block order)
+    if (sc.get(&dw, stage.size()) || sc.get(&dx, (size_t)rows * E) || sc.get(&dq, qbytes) || sc.get(&dgq, (size_t)rows * FF * 5 / 4) || sc.get(&ctl, (size_t)1)) return -7;
+    HIP_TRY(hipMemcpy(dw, stage.data(), stage.size(), hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(dx, x, (size_t)rows * E * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(dq, 0, qbytes));                        // (row slots past the block are read as operand rows of the matrix cores)
+    HIP_TRY(hipMemset(ctl, 0, sizeof(StepCtl)));
+    hipStream_t st;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    RowArgs s{};
+    s.x = dx; s.dparts = 1; s.q = dq; s.E = E; s.eps = 1e-6f; s.q_units = rows >= 4 ? 2 : 1;
+    GegluArgs a{ dw, E, FF, dq, dgq, 0 };
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    auto body = [&]() -> int {
+        HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+        int rc = 0;
+        auto run = [&](auto tag) {
+            constexpr int M = decltype(tag)::value;
+            rows_isolated<M>(st, s, ctl);
+            for (int r = 0; r < repeats + 1; ++r) {
+                if (r == 1) (void)hipEventRecord(e0, st);
+                if constexpr (M >= 4) {
+                    const size_t lds = (size_t)(E / 32) * LG_MU_DWORDS * 4;
+                    rc = set_lds(lg_k_geglu_m<M>, lds);
+                    if (rc) return;
+                    hipLaunchKernelGGL((lg_k_geglu_m<M>), dim3(FF / 32), dim3(512), lds, st, LG_GEGLU_FIELDS(LG_XA, a) 0);
+                } else hipLaunchKernelGGL((lg_k_geglu_t<M>), dim3(FF / 32), dim3(512), 0, st, LG_GEGLU_FIELDS(LG_XA, a) 0);
+            }
+        };
+        switch (rows) {
+#define CASE(M) case M: run(std::integral_constant<int, M>{}); break;
+            CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+#undef CASE
+        }
+        if (rc) return rc;
+        HIP_TRY(hipEventRecord(e1, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        HIP_TRY(hipGetLastError());
+        float t = 0;
+        if (repeats > 0) HIP_TRY(hipEventElapsedTime(&t, e0, e1));
+        if (kernel_ms) *kernel_ms = repeats > 0 ? t / repeats : 0.0f;
+        return 0;
+    };
+    int rc = body();
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipStreamDestroy(st);
+    if (rc) return rc;
+    return read_back_q8(dgq, rows, FF, aq, ad, asum);
 }
 
 extern "C" int lg_hip_ffn_xcd(const float *x, const float *dout, const float *w_post, const float *w_pre,

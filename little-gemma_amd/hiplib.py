@@ -395,6 +395,20 @@ def down_m(act, down_q4_0, E, repeats=0, join=1):
     return out, ms.value
 
 
+def gate_up_geglu(x, gate_q4_0, up_q4_0, FF, repeats=0):
+    """lg_k_geglu_t / lg_k_geglu_m in isolation: x [rows][E] f32, gate / up raw q4_0 rows [FF][E]; returns dict(aq, ad, asum, ms):
+    the q8 of gelu(gate) * up in natural order."""
+    H = load_hip()
+    x = np.ascontiguousarray(x, np.float32)
+    rows, E = x.shape
+    H.lg_hip_gate_up_geglu.argtypes = [f32p, u8p, u8p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.POINTER(C.c_float)]
+    aq = np.zeros((rows, FF), np.int8); ad = np.zeros((rows, FF // 32), np.float32); asum = np.zeros((rows, FF // 32), np.int32)
+    ms = C.c_float(0)
+    hip_check(H.lg_hip_gate_up_geglu(x, np.ascontiguousarray(gate_q4_0, np.uint8), np.ascontiguousarray(up_q4_0, np.uint8), rows, E, FF,
+                                     aq.ctypes.data, ad.ctypes.data, asum.ctypes.data, repeats, C.byref(ms)), "gate_up_geglu")
+    return dict(aq=aq, ad=ad, asum=asum, ms=ms.value)
+
+
 def ffn_xcd(x, dout, w_post, w_pre, gate_q4_0, up_q4_0, down_q4_0, FF, eps=1e-6, repeats=0, flush_mb=0, want_stamps=False, delay_w=0):
     """The XCD-partitioned feed-forward half of a layer through the C ABI.  x, dout: [rows, E] (rows 4..8); gate / up:
     FF q4_0 rows of E, down: E q4_0 rows of FF.  Returns dict(x_out, act [rows, FF], out [rows, E], kernel_ms)."""

@@ -275,3 +275,31 @@ def test_bad_arguments_are_refused(lg, gpu_required):
     with pytest.raises(lg.hiplib.HipError):
         lg.hiplib.attention(np.zeros((2, 8 * 256), np.float32), np.zeros((64, 512), np.uint16), np.zeros((64, 512), np.uint16),
                             8, 2, 256, 0, 100)                                                        # cache too short
+
+
+@pytest.mark.parametrize("rows,E,FF", [(1, 2560, 10240), (3, 2560, 10240), (4, 2560, 10240), (5, 2560, 10240), (8, 2560, 10240),
+                                       (2, 512, 2048), (6, 512, 2048), (5, 3840, 15360), (1, 3840, 15360)])
+def test_gate_up_geglu_matches_oracle(lg, ob, gpu_required, rows, E, FF):
+    """The gate/up kernels in isolation (lg_k_geglu_t for 1..3 rows, lg_k_geglu_m on the matrix cores for 4..8): the
+    q8 of gelu(gate . x) * (up . x) against the oracle's matmuls, GELU and quantization, at the E4B and 12B widths
+    and a small one; a row that starts with zeros and rows of different scale."""
+    rng = np.random.default_rng(rows * 13 + E + FF)
+    x = (rng.normal(0, 1, (rows, E)) * rng.uniform(0.3, 2.0, (rows, 1))).astype(np.float32)
+    x[0, :64] = 0.0
+    wg, wu = random_q4_0(rng, FF, E), random_q4_0(rng, FF, E)
+    print(f"gate/up rows={rows} E={E} FF={FF}", flush=True)
+    r = lg.hiplib.gate_up_geglu(x, wg, wu, FF, repeats=3)
+    L = ob.lib()
+    _, _, _, gate, _ = oracle_matmul(ob, wg, E, FF, x)
+    _, _, _, up, _ = oracle_matmul(ob, wu, E, FF, x)
+    act = np.zeros((rows, FF), np.float32)
+    for j in range(rows):
+        act[j] = np.array([L.lgo_gelu(float(v), 1) for v in gate[j]], np.float32) * up[j]
+    aq = np.zeros((rows, FF), np.int8); ad = np.zeros((rows, FF // 32), np.float32); asum = np.zeros((rows, FF // 32), np.int32)
+    for j in range(rows):
+        L.lgo_quant_q8(act[j], FF, aq[j], ad[j], asum[j])
+    assert np.array_equal(r["ad"].view(np.uint32), ad.view(np.uint32)), "scales"
+    assert np.array_equal(r["aq"], aq), "values"
+    assert np.array_equal(r["asum"], asum), "sums"
+    print(f"  kernel {1e3 * r['ms']:.2f} us", flush=True)
+
